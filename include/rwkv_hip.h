@@ -1,0 +1,220 @@
+/*
+ * rwkv_hip.h -- C ABI of librwkv_hip.so: the MI355X (gfx950) backend for the
+ * FASTQUANT (fp32i8) RWKV-4 forward path.
+ *
+ * Conventions for every entry point
+ *   - returns 0 (RWKV_OK) or a negative rwkv_status; never throws, never
+ *     synchronises the device, never retains caller pointers past the call
+ *     (the model handle retains the pointers in its descriptor by design);
+ *   - all data pointers are DEVICE pointers unless a comment says "host";
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*; NULL is the
+ *     null stream) and is ordered with other work on that stream;
+ *   - arguments are validated on the host (null pointers, sizes, alignment)
+ *     before anything is launched; rwkv_last_error() describes the last
+ *     failure on the calling thread.
+ *
+ * File:line citations name the reference interface each entry point replaces,
+ * relative to the reference repository's src/rwkvstic/.
+ */
+#ifndef RWKV_HIP_H
+#define RWKV_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *rwkv_stream_t; /* hipStream_t */
+
+typedef enum rwkv_status {
+    RWKV_OK = 0,
+    RWKV_ERR_ARG = -1,       /* null pointer / non-positive size / bad enum   */
+    RWKV_ERR_ALIGN = -2,     /* pointer or stride not aligned as documented   */
+    RWKV_ERR_SIZE = -3,      /* shape outside what the kernels support        */
+    RWKV_ERR_WORKSPACE = -4, /* workspace too small                           */
+    RWKV_ERR_HIP = -5,       /* a HIP runtime call failed                     */
+    RWKV_ERR_DEVICE = -6     /* no gfx950 device                              */
+} rwkv_status;
+
+int rwkv_version(void);
+const char *rwkv_last_error(void);
+
+/* ------------------------------------------------------------------------
+ * 1. The three operators of the reference's native library "rwkv"
+ *    (agnostic/backends/cuda/wrapper.cpp:131-141), same argument meaning,
+ *    same in-place semantics, reference memory layouts.
+ * ---------------------------------------------------------------------- */
+
+/* Bytes of scratch rwkv_mm8_one / rwkv_mm8_three need for a given shape
+ * (n_mat = 1 or 3).  The scratch holds per-row-split partial sums that are
+ * then added in a fixed order, which makes the result deterministic (the
+ * reference races 16 atomicAdds per output, operators32.cu:38). */
+size_t rwkv_mm8_workspace_bytes(int64_t n_in, int64_t n_out, int n_mat);
+
+/* mm8_one (wrapper.cpp:52-79, operators32.cu:18-40,105-115):
+ *   y[k] += sum_j x[j] * (w[j*w_stride + k] * r[j]),  j < n_in, k < n_out.
+ * x[n_in], r[n_in], y[n_out] float32 (y is accumulated into, as in the
+ * reference where the caller zero-fills it, matmul.py:44); w uint8 rows of
+ * n_out bytes, row stride w_stride >= n_out bytes.  The zero-point term is
+ * NOT added here (the reference adds it in Python, matmul.py:59-62). */
+int rwkv_mm8_one(rwkv_stream_t stream, int64_t n_in, int64_t n_out,
+                 const float *x, const uint8_t *w, int64_t w_stride,
+                 float *y, const float *r,
+                 void *workspace, size_t workspace_bytes);
+
+/* mm8_three (wrapper.cpp:82-127, operators32.cu:44-104): three independent
+ * (x, w, r, y) problems sharing n_in and n_out in one launch. */
+int rwkv_mm8_three(rwkv_stream_t stream, int64_t n_in, int64_t n_out,
+                   const float *x0, const float *x1, const float *x2,
+                   const uint8_t *w0, int64_t w0_stride,
+                   const uint8_t *w1, int64_t w1_stride,
+                   const uint8_t *w2, int64_t w2_stride,
+                   float *y0, float *y1, float *y2,
+                   const float *r0, const float *r1, const float *r2,
+                   void *workspace, size_t workspace_bytes);
+
+/* wkv_forward (wrapper.cpp:45-50, operators.cu:6-44), float64, reference
+ * state convention: k, v, y are [B, T, C]; w (= -exp(time_decay)), u are [C];
+ * aa, bb, pp are [B, C] and are updated in place; on return aa, bb hold the
+ * reference's e^w-premultiplied sums and pp is left untouched.  Internally
+ * the recurrence runs in the max-shifted form, so it does not overflow where
+ * the reference's naive form would not either. */
+int rwkv_wkv_forward_f64(rwkv_stream_t stream, int64_t B, int64_t T, int64_t C,
+                         const double *w, const double *u,
+                         const double *k, const double *v, double *y,
+                         double *aa, double *bb, double *pp);
+
+/* ------------------------------------------------------------------------
+ * 2. Quantiser and weight layouts (agnostic/backends/modules/matmul.py:18-40)
+ * ---------------------------------------------------------------------- */
+
+/* MM8.QuantizeMatrix: weight[n_out, n_in] float32 row-major (the checkpoint
+ * orientation) -> codes[n_in, n_out] uint8 row-major (the reference/.rwkv
+ * layout), range[n_in] float32, offset[n_in] float64; one scale and one
+ * minimum per INPUT channel, float64 arithmetic, truncating codes, mean
+ * truncated fraction folded into the offset.  A constant input channel
+ * (max == min) gets range 0, codes 0, offset = the constant (the reference
+ * divides by zero there). */
+int rwkv_quantize_u8(rwkv_stream_t stream, const float *weight,
+                     int64_t n_out, int64_t n_in,
+                     uint8_t *codes, float *range, double *offset);
+
+/* Device layout the matvec/GEMM kernels stream: 1 KiB blocks of 8 output
+ * columns x 128 input rows, blocks ordered [ceil(n_out/8)][ceil(n_in/128)],
+ * zero padded.  Within a block, byte 16*(8*s + c) + 4*m + e holds
+ * codes[128*kb + 32*m + 4*s + e][8*ct + c]  (c, s < 8; m, e < 4), so that a
+ * 64-lane wavefront reads the block with one 16-byte load per lane and lane
+ * (s, c) multiplies against four 16-byte LDS reads that are conflict free. */
+size_t rwkv_packed_bytes(int64_t n_in, int64_t n_out);
+int rwkv_pack_u8(rwkv_stream_t stream, const uint8_t *codes, int64_t codes_stride,
+                 int64_t n_in, int64_t n_out, uint8_t *packed);
+/* Inverse of rwkv_pack_u8 (used by .rwkv export and by the parity tests). */
+int rwkv_unpack_u8(rwkv_stream_t stream, const uint8_t *packed,
+                   int64_t n_in, int64_t n_out, uint8_t *codes, int64_t codes_stride);
+
+/* Canonical dequantisation fp32(fp64(code)*fp64(range[j]) + offset[j]) of a
+ * packed matrix into dq[n_in, n_out] float32 row-major (parity/debug). */
+int rwkv_dequant_packed(rwkv_stream_t stream, const uint8_t *packed,
+                        const float *range, const double *offset,
+                        int64_t n_in, int64_t n_out, float *dq);
+
+/* ------------------------------------------------------------------------
+ * 3. Stand-alone kernels on the packed layout
+ * ---------------------------------------------------------------------- */
+
+/* Quantised matrix-vector product with the general four-vector dequantisation
+ *   dq[j,k] = code[j,k]*r_row[j]*r_col[k] + m_row[j] + m_col[k]
+ *   y[b,k]  = r_col[k]*sum_j fp32(x[b,j]*r_row[j])*code[j,k]
+ *             + sum_j x[b,j]*m_row[j] + m_col[k]*sum_j x[b,j]
+ * for b < B <= 8.  x[B, n_in] float32, y[B, n_out] float64 (float32
+ * accumulation of the matrix term, float64 zero-point terms, as in
+ * MM8.forward matmul.py:51-62).  r_col / m_col may be NULL (= 1 / 0): that
+ * is the reference layout.  Replaces MM8.forward for T == 1. */
+int rwkv_mm8_packed(rwkv_stream_t stream, int64_t B, int64_t n_in, int64_t n_out,
+                    const float *x, const uint8_t *packed,
+                    const float *r_row, const double *m_row,
+                    const float *r_col, const float *m_col,
+                    double *y);
+
+/* Max-shifted float32 WKV recurrence, one thread per (b, c), state in
+ * registers.  k, v, y [B, T, C]; w, u [C]; state (aa, bb, pp) [B, C] updated
+ * in place and related to the reference's naive state by
+ * aa_ref = aa*exp(pp), bb_ref = bb*exp(pp) (operators.cu:21-36; closed form
+ * of the shifted recurrence: agnostic/agnosticRwkv.py:68-103). */
+int rwkv_wkv_f32(rwkv_stream_t stream, int64_t B, int64_t T, int64_t C,
+                 const float *w, const float *u,
+                 const float *k, const float *v, float *y,
+                 float *aa, float *bb, float *pp);
+
+/* ------------------------------------------------------------------------
+ * 4. Whole-model forward (replaces myRWKV.forward, agnostic/backends/opt.py:61-76,
+ *    and everything it calls: modules/block.py:56-102, modules/layernorm.py:11-20,
+ *    modules/emb.py:9, modules/matmul.py:51-102, modules/wkv.py:8-19)
+ * ---------------------------------------------------------------------- */
+
+typedef struct rwkv_qmat {
+    const uint8_t *packed; /* rwkv_pack_u8 layout, 16-byte aligned            */
+    const float *range;    /* [n_in]                                          */
+    const double *offset;  /* [n_in]                                          */
+    int64_t n_in, n_out;
+} rwkv_qmat;
+
+typedef struct rwkv_layer_desc {
+    const double *ln1_w, *ln1_b, *ln2_w, *ln2_b; /* [C]                       */
+    const double *att_mix;    /* [3, C]  rows k, v, r   (block.py:35-37)     */
+    const double *ffn_mix;    /* [2, C]  rows k, r      (block.py:46-47)     */
+    const double *time_decay; /* [C]  = -exp(raw)       (block.py:41)        */
+    const double *time_first; /* [C]                    (block.py:39)        */
+    rwkv_qmat att_k, att_v, att_r, att_o, ffn_k, ffn_r, ffn_v;
+} rwkv_layer_desc;
+
+typedef struct rwkv_model_desc {
+    int64_t n_layer, n_embd, n_ffn, n_vocab;
+    const float *emb;            /* [V, C] float32, device                    */
+    const double *ln0_w, *ln0_b; /* blocks.0.ln0 (opt.py:40-43)               */
+    const double *ln_out_w, *ln_out_b;
+    rwkv_qmat head;
+    const rwkv_layer_desc *layers; /* HOST array of n_layer descriptors       */
+} rwkv_model_desc;
+
+typedef struct rwkv_model rwkv_model;
+
+/* Copies the descriptor (host side); the device buffers it names must outlive
+ * the handle. */
+int rwkv_model_create(const rwkv_model_desc *desc, rwkv_model **out);
+void rwkv_model_destroy(rwkv_model *m);
+
+/* Scratch needed by rwkv_model_forward for chunks of up to max_tokens tokens. */
+size_t rwkv_model_workspace_bytes(const rwkv_model *m, int64_t max_tokens);
+
+/* logits[V], state = forward(tokens[T], state):  emb -> ln0 -> L x Block ->
+ * ln_out -> head(last token).  tokens: int64 [T] on the device; state:
+ * float64 [L, 5, C] on the device, rows (att shift, ffn shift, aa, bb, pp),
+ * updated in place.  WKV rows hold the max-shifted triple (see rwkv_wkv_f32);
+ * the reference's empty state (0, 0, 0, 0, -1e30) is valid as is.
+ * logits: float64 [V].  T == 1 takes the matvec path, T > 1 the GEMM path. */
+int rwkv_model_forward(rwkv_model *m, rwkv_stream_t stream,
+                       const int64_t *tokens, int64_t T,
+                       double *state, double *logits,
+                       void *workspace, size_t workspace_bytes);
+
+/* Greedy decode entirely on the device: for i < n:
+ *   logits, state = forward(tokens[i], state); tokens[i+1] = argmax(logits).
+ * tokens: int64 [n + 1] on the device, tokens[0] is the input token.  This is
+ * RWKVMaster.forward(number=n) (rwkvMaster.py:28-56) with the sampler
+ * replaced by argmax and no host round trip per token. */
+int rwkv_model_decode_greedy(rwkv_model *m, rwkv_stream_t stream,
+                             int64_t *tokens, int64_t n,
+                             double *state, double *logits,
+                             void *workspace, size_t workspace_bytes);
+
+/* out_token[0] = index of the first maximum of logits[V]. */
+int rwkv_argmax_f64(rwkv_stream_t stream, const double *logits, int64_t V,
+                    int64_t *out_token);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RWKV_HIP_H */

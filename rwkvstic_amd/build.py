@@ -1,0 +1,47 @@
+"""Build librwkv_hip.so (gfx950) in-tree with hipcc.
+
+``python -m rwkvstic_amd.build`` or ``build()``; hipcc cross-compiles without a
+GPU.  The library is written next to this file so it travels with the tree.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "librwkv_hip.so")
+SOURCES = ["rwkv_quant.hip", "rwkv_ops.hip", "rwkv_model.hip"]
+
+FLAGS = [
+    "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950",
+    # scalar/float2 code must not be turned into packed-fp32 instructions
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-result",
+]
+
+
+def hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found")
+    return exe
+
+
+def build(verbose: bool = True, extra_flags=()) -> str:
+    srcs = [os.path.join(CSRC, s) for s in SOURCES]
+    tmp = LIB + ".tmp"
+    cmd = [hipcc(), *FLAGS, *extra_flags, "-o", tmp, *srcs]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    os.replace(tmp, LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    build()
+    print(LIB)

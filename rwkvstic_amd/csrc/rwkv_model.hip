@@ -1,0 +1,519 @@
+// Whole-model forward for the FASTQUANT RWKV-4 path (reference
+// agnostic/backends/opt.py:61-76, modules/block.py:56-102).
+//
+// One token step is a chain of dependent "phases"; each phase is one launch
+// whose workgroups own 8-column tiles of the phase's matrices:
+//
+//   embed    x = ln0(emb[token])
+//   per layer
+//     att_kvr  prologue: xy = ln1(x); mix_{k,v,r} = lerp(shift, xy); xs = fp32(mix*range)
+//              product : k, v, r columns of the tile
+//              epilogue: r = sigmoid(r); one WKV step on the tile's channels;
+//                        att_in = wkv * r
+//     att_out  prologue: xs = fp32(att_in*range)
+//              epilogue: x += W_o(att_in)              ; commit att shift state
+//     ffn_rk   prologue: ddd = ln2(x); mix_{k,r}
+//              epilogue: rf = sigmoid(.) | h = relu(.)^2
+//     ffn_v    prologue: xs = fp32(h*range)
+//              epilogue: x = W_v(h)*rf + x             ; commit ffn shift state
+//   head     prologue: ln_out(x)                       ; logits
+//
+// Numeric types follow the reference: residual stream, LayerNorm, token shift,
+// lerp, zero-point dot products and state are float64 (block.py:37-47,
+// layernorm.py:7-10); the matrix term is fp32(x*range) times uint8 codes with
+// float32 accumulation (matmul.py:58,131); WKV runs in float32 in the
+// max-shifted form.
+#include "rwkv_common.h"
+
+#include <new>
+#include <string>
+#include <vector>
+
+namespace rwkv {
+
+constexpr int kMaxCPT = 24;   // channels per thread in the LayerNorm prologue: C <= 6144
+constexpr int kXsBudgetBlocks = 96;   // 96 blocks * 128 rows * 4 B = 48 KiB of staged activations
+
+struct QMatDev {
+    const uint8_t *packed;
+    const float *range;
+    const double *offset;
+    int n_in, n_out, n_kb;
+};
+
+static QMatDev to_dev(const rwkv_qmat &q) {
+    QMatDev d;
+    d.packed = q.packed; d.range = q.range; d.offset = q.offset;
+    d.n_in = (int)q.n_in; d.n_out = (int)q.n_out; d.n_kb = (int)ceil_div(q.n_in, kBlockRows);
+    return d;
+}
+
+// ---------------------------------------------------------------------------
+// LayerNorm over C channels held in registers: thread t owns channels
+// t, t+256, ...  (layernorm.py:15-20: biased variance, eps inside the sqrt,
+// division by the standard deviation).  val[] is replaced by the normalised
+// values.  red: LDS scratch of kWaves doubles.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void layernorm_regs(int C, double (&val)[kMaxCPT],
+                                               const double *__restrict__ w,
+                                               const double *__restrict__ b, double *red) {
+    double s[1] = {0.0};
+#pragma unroll
+    for (int i = 0; i < kMaxCPT; ++i) {
+        const int c = threadIdx.x + i * kThreads;
+        if (c < C) s[0] += val[i];
+    }
+    block_sum<1>(s, red);
+    const double mean = s[0] / (double)C;
+    double q[1] = {0.0};
+#pragma unroll
+    for (int i = 0; i < kMaxCPT; ++i) {
+        const int c = threadIdx.x + i * kThreads;
+        if (c < C) { val[i] -= mean; q[0] += val[i] * val[i]; }
+    }
+    block_sum<1>(q, red);
+    const double sd = sqrt(q[0] / (double)C + 1e-5);
+#pragma unroll
+    for (int i = 0; i < kMaxCPT; ++i) {
+        const int c = threadIdx.x + i * kThreads;
+        if (c < C) val[i] = w[c] * (val[i] / sd) + b[c];
+    }
+}
+
+// ---------------------------------------------------------------------------
+// embed: x = ln0(emb[token])      (emb.py:9, opt.py:63-64)
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(kThreads)
+embed_ln0_kernel(const int64_t *__restrict__ token, int V, int C, const float *__restrict__ emb,
+                 const double *__restrict__ w, const double *__restrict__ b, double *__restrict__ x) {
+    __shared__ double red[kWaves];
+    int64_t tok = token[0];
+    if (tok < 0) tok = 0;
+    if (tok >= V) tok = V - 1;
+    double val[kMaxCPT];
+#pragma unroll
+    for (int i = 0; i < kMaxCPT; ++i) {
+        const int c = threadIdx.x + i * kThreads;
+        val[i] = c < C ? (double)emb[(size_t)tok * C + c] : 0.0;
+    }
+    layernorm_regs(C, val, w, b, red);
+#pragma unroll
+    for (int i = 0; i < kMaxCPT; ++i) {
+        const int c = threadIdx.x + i * kThreads;
+        if (c < C) x[c] = val[i];
+    }
+}
+
+// ---------------------------------------------------------------------------
+// att_kvr
+// ---------------------------------------------------------------------------
+struct AttKvrArgs {
+    int C;
+    const double *x;
+    const double *ln_w, *ln_b;
+    const double *mix;          // [3, C] k, v, r
+    double *state;              // this layer's [5, C]
+    QMatDev k, v, r;
+    const double *time_decay, *time_first;
+    double *att_in;             // out: wkv * sigmoid(r)
+    double *xy_tmp;             // out: ln1(x), committed to state[0] by att_out
+};
+
+__global__ void __launch_bounds__(kThreads)
+att_kvr_kernel(const AttKvrArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int C = a.C;
+    const int n_kb = a.k.n_kb;
+    const int in_pad = n_kb * kBlockRows;
+    float *xs = reinterpret_cast<float *>(smem);                         // [3][in_pad]
+    double *dred = reinterpret_cast<double *>(xs + 3 * (size_t)in_pad);  // [3*kWaves]
+    float *fred = reinterpret_cast<float *>(dred + 3 * kWaves);          // [3*kWaves*8]
+    const int ct = blockIdx.x;
+
+    double val[kMaxCPT];
+#pragma unroll
+    for (int i = 0; i < kMaxCPT; ++i) {
+        const int c = threadIdx.x + i * kThreads;
+        val[i] = c < C ? a.x[c] : 0.0;
+    }
+    layernorm_regs(C, val, a.ln_w, a.ln_b, dred);
+
+    double zp[3] = {0.0, 0.0, 0.0};
+    const QMatDev *mats[3] = {&a.k, &a.v, &a.r};
+#pragma unroll
+    for (int i = 0; i < kMaxCPT; ++i) {
+        const int c = threadIdx.x + i * kThreads;
+        if (c < in_pad) {
+            if (c < C) {
+                const double xy = val[i];
+                const double sh = a.state[c];                 // state[0]: previous token's ln1 output
+#pragma unroll
+                for (int m = 0; m < 3; ++m) {
+                    const double mu = a.mix[(size_t)m * C + c];
+                    const double mixed = xy * mu + sh * (1.0 - mu);          // block.py:67
+                    xs[(size_t)m * in_pad + c] = (float)(mixed * (double)mats[m]->range[c]);  // matmul.py:131
+                    zp[m] += mixed * mats[m]->offset[c];
+                }
+                if (c / kTileCols == ct) a.xy_tmp[c] = xy;
+            } else {
+#pragma unroll
+                for (int m = 0; m < 3; ++m) xs[(size_t)m * in_pad + c] = 0.f;
+            }
+        }
+    }
+    block_sum<3>(zp, dred);   // also orders the xs writes before the reads below
+
+    const uint8_t *const wtile[3] = {a.k.packed + (size_t)ct * n_kb * kBlockBytes,
+                                     a.v.packed + (size_t)ct * n_kb * kBlockBytes,
+                                     a.r.packed + (size_t)ct * n_kb * kBlockBytes};
+    const float *const xsp[3] = {xs, xs + in_pad, xs + 2 * (size_t)in_pad};
+    float acc[3][1] = {{0.f}, {0.f}, {0.f}};
+    tile_accumulate<3, 1>(wtile, xsp, in_pad, 0, n_kb, acc);
+    float out[3][1];
+    tile_reduce<3, 1>(acc, fred, out);
+
+    if (threadIdx.x < kTileCols) {
+        const int c = ct * kTileCols + threadIdx.x;
+        if (c < C) {
+            const double kd = (double)out[0][0] + zp[0];      // matmul.py:59-62
+            const double vd = (double)out[1][0] + zp[1];
+            const double rd = (double)out[2][0] + zp[2];
+            const float r = sigmoid_f32((float)rd);           // block.py:72
+            float aa = (float)a.state[2 * (size_t)C + c];
+            float bb = (float)a.state[3 * (size_t)C + c];
+            double pp = a.state[4 * (size_t)C + c];
+            const float y = wkv_step_f32(a.time_decay[c], a.time_first[c], (float)kd, (float)vd, aa, bb, pp);
+            a.state[2 * (size_t)C + c] = (double)aa;
+            a.state[3 * (size_t)C + c] = (double)bb;
+            a.state[4 * (size_t)C + c] = pp;
+            a.att_in[c] = (double)(y * r);                    // block.py:78
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// att_out / ffn_v: input vector already formed by the previous phase.
+// ---------------------------------------------------------------------------
+struct VecMatArgs {
+    QMatDev w;
+    const double *vin;        // [n_in]
+    double *x;                // residual stream [n_out], updated in place
+    const double *gate;       // ffn_v: rf [n_out]; att_out: null
+    const double *shift_src;  // ln output of this token for the tile's channels
+    double *shift_dst;        // state row to commit it to
+    int kc_blocks;
+};
+
+__global__ void __launch_bounds__(kThreads)
+vec_matvec_kernel(const VecMatArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int n_kb = a.w.n_kb, n_in = a.w.n_in;
+    const int kc_rows = a.kc_blocks * kBlockRows;
+    float *xs = reinterpret_cast<float *>(smem);                  // [kc_rows]
+    double *dred = reinterpret_cast<double *>(xs + kc_rows);      // [kWaves]
+    float *fred = reinterpret_cast<float *>(dred + kWaves);       // [kWaves*8]
+    const int ct = blockIdx.x;
+    const uint8_t *const wtile[1] = {a.w.packed + (size_t)ct * n_kb * kBlockBytes};
+    const float *const xsp[1] = {xs};
+    float acc[1][1] = {{0.f}};
+    double zp[1] = {0.0};
+    for (int kb0 = 0; kb0 < n_kb; kb0 += a.kc_blocks) {
+        const int kb1 = min(kb0 + a.kc_blocks, n_kb);
+        const int j0 = kb0 * kBlockRows;
+        for (int i = threadIdx.x; i < (kb1 - kb0) * kBlockRows; i += kThreads) {
+            const int j = j0 + i;
+            float v = 0.f;
+            if (j < n_in) {
+                const double h = a.vin[j];
+                v = (float)(h * (double)a.w.range[j]);
+                zp[0] += h * a.w.offset[j];
+            }
+            xs[i] = v;
+        }
+        __syncthreads();
+        tile_accumulate<1, 1>(wtile, xsp, kc_rows, kb0, kb1, acc);
+        __syncthreads();
+    }
+    block_sum<1>(zp, dred);
+    float out[1][1];
+    tile_reduce<1, 1>(acc, fred, out);
+    if (threadIdx.x < kTileCols) {
+        const int c = ct * kTileCols + threadIdx.x;
+        if (c < a.w.n_out) {
+            const double y = (double)out[0][0] + zp[0];
+            if (a.gate) a.x[c] = y * a.gate[c] + a.x[c];     // block.py:100
+            else        a.x[c] = a.x[c] + y;                 // block.py:80
+            a.shift_dst[c] = a.shift_src[c];                 // block.py:63-64 / 87-88
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// ffn_rk / head: LayerNorm prologue, one matrix per tile.
+// ---------------------------------------------------------------------------
+enum { EPI_LOGITS = 0, EPI_FFN = 1 };
+
+struct LnMatArgs {
+    int C, mode;
+    const double *x;
+    const double *ln_w, *ln_b;
+    // EPI_FFN: tiles [0, C/8) belong to `r` (mix row 1), the rest to `k` (mix row 0)
+    const double *mix;          // [2, C] k, r   (null for the head)
+    const double *shift;        // state[1]
+    QMatDev k, r;               // head: only k is used
+    double *out_k;              // EPI_FFN: h = relu(.)^2 [F]; EPI_LOGITS: logits [V]
+    double *out_r;              // EPI_FFN: rf = sigmoid(.) [C]
+    double *ln_tmp;             // EPI_FFN: ln2(x) for the tile's channels
+};
+
+__global__ void __launch_bounds__(kThreads)
+ln_matvec_kernel(const LnMatArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int C = a.C;
+    const int n_kb = a.k.n_kb;
+    const int in_pad = n_kb * kBlockRows;
+    float *xs = reinterpret_cast<float *>(smem);                 // [in_pad]
+    double *dred = reinterpret_cast<double *>(xs + in_pad);      // [kWaves]
+    float *fred = reinterpret_cast<float *>(dred + kWaves);      // [kWaves*8]
+
+    int ct = blockIdx.x;
+    bool is_r = false;
+    if (a.mode == EPI_FFN) {
+        const int r_tiles = (a.r.n_out + kTileCols - 1) / kTileCols;
+        if (ct < r_tiles) is_r = true; else ct -= r_tiles;
+    }
+    const QMatDev &W = is_r ? a.r : a.k;
+
+    double val[kMaxCPT];
+#pragma unroll
+    for (int i = 0; i < kMaxCPT; ++i) {
+        const int c = threadIdx.x + i * kThreads;
+        val[i] = c < C ? a.x[c] : 0.0;
+    }
+    layernorm_regs(C, val, a.ln_w, a.ln_b, dred);
+
+    double zp[1] = {0.0};
+#pragma unroll
+    for (int i = 0; i < kMaxCPT; ++i) {
+        const int c = threadIdx.x + i * kThreads;
+        if (c < in_pad) {
+            float v = 0.f;
+            if (c < C) {
+                double mixed = val[i];
+                if (a.mix) {
+                    const double mu = a.mix[(size_t)(is_r ? 1 : 0) * C + c];
+                    mixed = val[i] * mu + a.shift[c] * (1.0 - mu);      // block.py:91
+                    if (is_r && c / kTileCols == ct) a.ln_tmp[c] = val[i];
+                }
+                v = (float)(mixed * (double)W.range[c]);
+                zp[0] += mixed * W.offset[c];
+            }
+            xs[c] = v;
+        }
+    }
+    block_sum<1>(zp, dred);
+
+    const uint8_t *const wtile[1] = {W.packed + (size_t)ct * n_kb * kBlockBytes};
+    const float *const xsp[1] = {xs};
+    float acc[1][1] = {{0.f}};
+    tile_accumulate<1, 1>(wtile, xsp, in_pad, 0, n_kb, acc);
+    float out[1][1];
+    tile_reduce<1, 1>(acc, fred, out);
+    if (threadIdx.x < kTileCols) {
+        const int k = ct * kTileCols + threadIdx.x;
+        if (k < W.n_out) {
+            const double y = (double)out[0][0] + zp[0];
+            if (a.mode == EPI_LOGITS) a.out_k[k] = y;
+            else if (is_r) a.out_r[k] = (double)sigmoid_f32((float)y);   // block.py:95
+            else { const double h = y > 0.0 ? y : 0.0; a.out_k[k] = h * h; }  // block.py:97-98
+        }
+    }
+}
+
+}  // namespace rwkv
+
+using namespace rwkv;
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+struct rwkv_model {
+    rwkv_model_desc d;
+    std::vector<rwkv_layer_desc> layers;
+};
+
+namespace {
+
+struct Workspace {
+    double *x, *xy_tmp, *ddd_tmp, *att_in, *rf, *h;
+};
+
+size_t ws_doubles(int64_t C, int64_t F) { return (size_t)(5 * C + F); }
+
+Workspace carve(void *ws, int64_t C, int64_t F) {
+    Workspace w;
+    double *p = static_cast<double *>(ws);
+    w.x = p; p += C;
+    w.xy_tmp = p; p += C;
+    w.ddd_tmp = p; p += C;
+    w.att_in = p; p += C;
+    w.rf = p; p += C;
+    w.h = p; p += F;
+    return w;
+}
+
+int check_qmat(const rwkv_qmat &q, int64_t n_in, int64_t n_out, const char *name) {
+    if (!q.packed || !q.range || !q.offset)
+        return set_error(RWKV_ERR_ARG, "rwkv_model_create: %s has a null pointer", name);
+    if (q.n_in != n_in || q.n_out != n_out)
+        return set_error(RWKV_ERR_SIZE, "rwkv_model_create: %s is %lldx%lld, expected %lldx%lld", name,
+                         (long long)q.n_in, (long long)q.n_out, (long long)n_in, (long long)n_out);
+    if (reinterpret_cast<uintptr_t>(q.packed) % 16)
+        return set_error(RWKV_ERR_ALIGN, "rwkv_model_create: %s.packed must be 16-byte aligned", name);
+    if (reinterpret_cast<uintptr_t>(q.range) % 4 || reinterpret_cast<uintptr_t>(q.offset) % 8)
+        return set_error(RWKV_ERR_ALIGN, "rwkv_model_create: %s.range/offset misaligned", name);
+    return RWKV_OK;
+}
+
+// One token through every layer; logits only when `with_head`.
+int step_token(rwkv_model *m, hipStream_t st, const int64_t *token, double *state, double *logits,
+               const Workspace &w, bool with_head) {
+    const rwkv_model_desc &d = m->d;
+    const int C = (int)d.n_embd, F = (int)d.n_ffn, V = (int)d.n_vocab;
+    const int c_tiles = (int)ceil_div(C, kTileCols), f_tiles = (int)ceil_div(F, kTileCols);
+    const int c_kb = (int)ceil_div(C, kBlockRows), f_kb = (int)ceil_div(F, kBlockRows);
+    const size_t red_bytes = 3 * kWaves * 8 + 3 * kWaves * 8 * 4;
+
+    hipLaunchKernelGGL(embed_ln0_kernel, dim3(1), dim3(kThreads), 0, st, token, V, C, d.emb, d.ln0_w, d.ln0_b, w.x);
+    for (int64_t l = 0; l < d.n_layer; ++l) {
+        const rwkv_layer_desc &L = m->layers[l];
+        double *sl = state + (size_t)l * 5 * C;
+        AttKvrArgs a;
+        a.C = C; a.x = w.x; a.ln_w = L.ln1_w; a.ln_b = L.ln1_b; a.mix = L.att_mix; a.state = sl;
+        a.k = to_dev(L.att_k); a.v = to_dev(L.att_v); a.r = to_dev(L.att_r);
+        a.time_decay = L.time_decay; a.time_first = L.time_first; a.att_in = w.att_in; a.xy_tmp = w.xy_tmp;
+        hipLaunchKernelGGL(att_kvr_kernel, dim3(c_tiles), dim3(kThreads),
+                           3 * (size_t)c_kb * kBlockRows * 4 + red_bytes, st, a);
+
+        VecMatArgs o;
+        o.w = to_dev(L.att_o); o.vin = w.att_in; o.x = w.x; o.gate = nullptr;
+        o.shift_src = w.xy_tmp; o.shift_dst = sl; o.kc_blocks = c_kb < kXsBudgetBlocks ? c_kb : kXsBudgetBlocks;
+        hipLaunchKernelGGL(vec_matvec_kernel, dim3(c_tiles), dim3(kThreads),
+                           (size_t)o.kc_blocks * kBlockRows * 4 + red_bytes, st, o);
+
+        LnMatArgs f;
+        f.C = C; f.mode = EPI_FFN; f.x = w.x; f.ln_w = L.ln2_w; f.ln_b = L.ln2_b; f.mix = L.ffn_mix;
+        f.shift = sl + C; f.k = to_dev(L.ffn_k); f.r = to_dev(L.ffn_r);
+        f.out_k = w.h; f.out_r = w.rf; f.ln_tmp = w.ddd_tmp;
+        hipLaunchKernelGGL(ln_matvec_kernel, dim3(c_tiles + f_tiles), dim3(kThreads),
+                           (size_t)c_kb * kBlockRows * 4 + red_bytes, st, f);
+
+        VecMatArgs v;
+        v.w = to_dev(L.ffn_v); v.vin = w.h; v.x = w.x; v.gate = w.rf;
+        v.shift_src = w.ddd_tmp; v.shift_dst = sl + C; v.kc_blocks = f_kb < kXsBudgetBlocks ? f_kb : kXsBudgetBlocks;
+        hipLaunchKernelGGL(vec_matvec_kernel, dim3(c_tiles), dim3(kThreads),
+                           (size_t)v.kc_blocks * kBlockRows * 4 + red_bytes, st, v);
+    }
+    if (with_head) {
+        LnMatArgs h;
+        h.C = C; h.mode = EPI_LOGITS; h.x = w.x; h.ln_w = d.ln_out_w; h.ln_b = d.ln_out_b; h.mix = nullptr;
+        h.shift = nullptr; h.k = to_dev(d.head); h.r = h.k; h.out_k = logits; h.out_r = nullptr; h.ln_tmp = nullptr;
+        hipLaunchKernelGGL(ln_matvec_kernel, dim3((unsigned)ceil_div(V, kTileCols)), dim3(kThreads),
+                           (size_t)c_kb * kBlockRows * 4 + red_bytes, st, h);
+    }
+    RWKV_CHECK_LAUNCH("token step");
+    return RWKV_OK;
+}
+
+int check_forward_args(const rwkv_model *m, const void *tokens, const double *state, const double *logits,
+                       const void *ws, size_t ws_bytes, int64_t T, const char *fn) {
+    if (!m || !tokens || !state || !logits || !ws) return set_error(RWKV_ERR_ARG, "%s: null pointer", fn);
+    if (T <= 0) return set_error(RWKV_ERR_ARG, "%s: token count must be positive", fn);
+    if (reinterpret_cast<uintptr_t>(tokens) % 8 || reinterpret_cast<uintptr_t>(state) % 8 ||
+        reinterpret_cast<uintptr_t>(logits) % 8 || reinterpret_cast<uintptr_t>(ws) % 16)
+        return set_error(RWKV_ERR_ALIGN, "%s: tokens/state/logits need 8-byte, workspace 16-byte alignment", fn);
+    const size_t need = rwkv_model_workspace_bytes(m, T);
+    if (ws_bytes < need)
+        return set_error(RWKV_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", fn, need, ws_bytes);
+    return RWKV_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rwkv_model_create(const rwkv_model_desc *desc, rwkv_model **out) {
+    RWKV_CHECK_ARG(desc && out, "rwkv_model_create: null pointer");
+    RWKV_CHECK_ARG(desc->layers, "rwkv_model_create: null layer table");
+    const int64_t L = desc->n_layer, C = desc->n_embd, F = desc->n_ffn, V = desc->n_vocab;
+    RWKV_CHECK_ARG(L > 0 && C > 0 && F > 0 && V > 0, "rwkv_model_create: sizes must be positive");
+    if (C > (int64_t)kMaxCPT * kThreads)
+        return set_error(RWKV_ERR_SIZE, "rwkv_model_create: n_embd %lld exceeds the supported %d", (long long)C,
+                         kMaxCPT * kThreads);
+    if (F >= (1 << 24) || V >= (1 << 28))
+        return set_error(RWKV_ERR_SIZE, "rwkv_model_create: n_ffn/n_vocab too large");
+    RWKV_CHECK_ARG(desc->emb && desc->ln0_w && desc->ln0_b && desc->ln_out_w && desc->ln_out_b,
+                   "rwkv_model_create: null model-level pointer");
+    int rc = check_qmat(desc->head, C, V, "head");
+    if (rc) return rc;
+    for (int64_t l = 0; l < L; ++l) {
+        const rwkv_layer_desc &ld = desc->layers[l];
+        RWKV_CHECK_ARG(ld.ln1_w && ld.ln1_b && ld.ln2_w && ld.ln2_b && ld.att_mix && ld.ffn_mix &&
+                       ld.time_decay && ld.time_first, "rwkv_model_create: layer %lld has a null pointer", (long long)l);
+        if ((rc = check_qmat(ld.att_k, C, C, "att_k")) || (rc = check_qmat(ld.att_v, C, C, "att_v")) ||
+            (rc = check_qmat(ld.att_r, C, C, "att_r")) || (rc = check_qmat(ld.att_o, C, C, "att_o")) ||
+            (rc = check_qmat(ld.ffn_k, C, F, "ffn_k")) || (rc = check_qmat(ld.ffn_r, C, C, "ffn_r")) ||
+            (rc = check_qmat(ld.ffn_v, F, C, "ffn_v")))
+            return rc;
+    }
+    int dev = 0;
+    RWKV_CHECK_HIP(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    RWKV_CHECK_HIP(hipGetDeviceProperties(&prop, dev));
+    if (std::string(prop.gcnArchName).rfind("gfx950", 0) != 0)
+        return set_error(RWKV_ERR_DEVICE, "rwkv_model_create: device is %s, this library is built for gfx950",
+                         prop.gcnArchName);
+    rwkv_model *m = new (std::nothrow) rwkv_model();
+    if (!m) return set_error(RWKV_ERR_ARG, "rwkv_model_create: out of host memory");
+    m->d = *desc;
+    m->layers.assign(desc->layers, desc->layers + L);
+    m->d.layers = m->layers.data();
+    *out = m;
+    return RWKV_OK;
+}
+
+void rwkv_model_destroy(rwkv_model *m) { delete m; }
+
+size_t rwkv_model_workspace_bytes(const rwkv_model *m, int64_t max_tokens) {
+    if (!m || max_tokens <= 0) return 0;
+    return round_up(ws_doubles(m->d.n_embd, m->d.n_ffn) * sizeof(double), 256);
+}
+
+int rwkv_model_forward(rwkv_model *m, rwkv_stream_t stream, const int64_t *tokens, int64_t T, double *state,
+                       double *logits, void *workspace, size_t workspace_bytes) {
+    int rc = check_forward_args(m, tokens, state, logits, workspace, workspace_bytes, T, "rwkv_model_forward");
+    if (rc) return rc;
+    const Workspace w = carve(workspace, m->d.n_embd, m->d.n_ffn);
+    for (int64_t t = 0; t < T; ++t) {
+        rc = step_token(m, (hipStream_t)stream, tokens + t, state, logits, w, t == T - 1);
+        if (rc) return rc;
+    }
+    return RWKV_OK;
+}
+
+int rwkv_model_decode_greedy(rwkv_model *m, rwkv_stream_t stream, int64_t *tokens, int64_t n, double *state,
+                             double *logits, void *workspace, size_t workspace_bytes) {
+    int rc = check_forward_args(m, tokens, state, logits, workspace, workspace_bytes, 1, "rwkv_model_decode_greedy");
+    if (rc) return rc;
+    RWKV_CHECK_ARG(n > 0, "rwkv_model_decode_greedy: n must be positive");
+    const Workspace w = carve(workspace, m->d.n_embd, m->d.n_ffn);
+    for (int64_t i = 0; i < n; ++i) {
+        rc = step_token(m, (hipStream_t)stream, tokens + i, state, logits, w, true);
+        if (rc) return rc;
+        rc = rwkv_argmax_f64(stream, logits, m->d.n_vocab, tokens + i + 1);
+        if (rc) return rc;
+    }
+    return RWKV_OK;
+}
+
+}  // extern "C"

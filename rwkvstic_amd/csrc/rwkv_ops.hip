@@ -1,0 +1,371 @@
+// Stand-alone operators: the packed uint8 matvec, the WKV recurrences, argmax,
+// and the reference-layout mm8_one / mm8_three drop-ins.
+#include "rwkv_common.h"
+
+namespace rwkv {
+
+// ---------------------------------------------------------------------------
+// y[b,k] = r_col[k] * sum_j fp32(x[b,j] r_row[j]) code[j,k]
+//          + sum_j x[b,j] m_row[j] + m_col[k] sum_j x[b,j]
+// One workgroup per 8-column tile.  The scaled activations are staged in LDS
+// in chunks of kc_rows rows (NB * kc_rows * 4 bytes <= 64 KiB); the matrix is
+// read exactly once, with one 16-byte load per lane per 1 KiB block.
+// ---------------------------------------------------------------------------
+template <int NB>
+__global__ void __launch_bounds__(kThreads)
+mm8_packed_kernel(int n_in, int n_out, int n_kb, int kc_blocks,
+                  const float *__restrict__ x, const uint8_t *__restrict__ packed,
+                  const float *__restrict__ r_row, const double *__restrict__ m_row,
+                  const float *__restrict__ r_col, const float *__restrict__ m_col,
+                  double *__restrict__ y) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    float *xs = reinterpret_cast<float *>(smem);                    // [NB][kc_rows]
+    const int kc_rows = kc_blocks * kBlockRows;
+    double *dred = reinterpret_cast<double *>(xs + (size_t)NB * kc_rows);   // [2*NB*kWaves]
+    float *fred = reinterpret_cast<float *>(dred + 2 * NB * kWaves);        // [NB*kWaves*8]
+
+    const int ct = blockIdx.x;
+    const uint8_t *const wtile[1] = {packed + (size_t)ct * n_kb * kBlockBytes};
+    const float *const xsp[1] = {xs};
+
+    float acc[1][NB];
+    double zsum[2 * NB];   // [b]: sum x*m_row ; [NB+b]: sum x
+#pragma unroll
+    for (int b = 0; b < NB; ++b) { acc[0][b] = 0.f; zsum[b] = 0.0; zsum[NB + b] = 0.0; }
+
+    for (int kb0 = 0; kb0 < n_kb; kb0 += kc_blocks) {
+        const int kb1 = min(kb0 + kc_blocks, n_kb);
+        const int j0 = kb0 * kBlockRows;
+        for (int i = threadIdx.x; i < (kb1 - kb0) * kBlockRows; i += kThreads) {
+            const int j = j0 + i;
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                float v = 0.f;
+                if (j < n_in) {
+                    const double xv = (double)x[(size_t)b * n_in + j];
+                    v = (float)(xv * (double)r_row[j]);
+                    zsum[b] += xv * m_row[j];
+                    zsum[NB + b] += xv;
+                }
+                xs[(size_t)b * kc_rows + i] = v;
+            }
+        }
+        __syncthreads();
+        tile_accumulate<1, NB>(wtile, xsp, kc_rows, kb0, kb1, acc);
+        __syncthreads();
+    }
+    block_sum<2 * NB>(zsum, dred);
+    float out[1][NB];
+    tile_reduce<1, NB>(acc, fred, out);
+    if (threadIdx.x < kTileCols) {
+        const int k = ct * kTileCols + threadIdx.x;
+        if (k < n_out) {
+            const double rc = r_col ? (double)r_col[k] : 1.0;
+            const double mc = m_col ? (double)m_col[k] : 0.0;
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+                y[(size_t)b * n_out + k] = rc * (double)out[0][b] + zsum[b] + mc * zsum[NB + b];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// WKV: one thread per (b, c); k/v loads are independent of the recurrence, so
+// the compiler can hoist them ahead of the dependent exp chain (unroll 4).
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(64)
+wkv_f32_kernel(int B, int T, int C, const float *__restrict__ w, const float *__restrict__ u,
+               const float *__restrict__ k, const float *__restrict__ v, float *__restrict__ y,
+               float *__restrict__ aa, float *__restrict__ bb, float *__restrict__ pp) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= B * C) return;
+    const int b = idx / C, c = idx % C;
+    const size_t base = (size_t)b * T * C + c;
+    const double wc = (double)w[c], uc = (double)u[c];
+    float a = aa[idx], bsum = bb[idx];
+    double p = (double)pp[idx];
+#pragma unroll 4
+    for (int t = 0; t < T; ++t) {
+        const size_t o = base + (size_t)t * C;
+        y[o] = wkv_step_f32(wc, uc, k[o], v[o], a, bsum, p);
+    }
+    aa[idx] = a; bb[idx] = bsum; pp[idx] = (float)p;
+}
+
+// Reference convention (cuda/operators.cu:6-37): naive pre-multiplied state in
+// and out, pp untouched; the max-shifted form runs in between.
+__global__ void __launch_bounds__(64)
+wkv_f64_ref_kernel(int B, int T, int C, const double *__restrict__ w, const double *__restrict__ u,
+                   const double *__restrict__ k, const double *__restrict__ v, double *__restrict__ y,
+                   double *__restrict__ aa, double *__restrict__ bb) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= B * C) return;
+    const int b = idx / C, c = idx % C;
+    const size_t base = (size_t)b * T * C + c;
+    const double wc = w[c], uc = u[c];
+    // naive (aa, bb) == shifted (aa, bb, pp = 0)
+    double a = aa[idx], bsum = bb[idx], p = 0.0;
+    if (!(bsum > 0.0)) p = -1e300;   // empty state: let the first token dominate exactly
+    for (int t = 0; t < T; ++t) {
+        const size_t o = base + (size_t)t * C;
+        y[o] = wkv_step<double>(wc, uc, k[o], v[o], a, bsum, p);
+    }
+    const double e = exp(p);
+    aa[idx] = a * e;
+    bb[idx] = bsum * e;
+}
+
+// First index of the maximum (torch.argmax tie rule is unspecified; greedy
+// decoding here takes the lowest index).
+__global__ void __launch_bounds__(1024)
+argmax_f64_kernel(const double *__restrict__ logits, int V, int64_t *__restrict__ out) {
+    __shared__ double sval[16];
+    __shared__ int sidx[16];
+    double best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = threadIdx.x; i < V; i += blockDim.x) {
+        const double x = logits[i];
+        if (x > best) { best = x; bi = i; }
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const double ob = __shfl_xor(best, off, 64);
+        const int oi = __shfl_xor(bi, off, 64);
+        if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) { sval[wave] = best; sidx[wave] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int wv = 1; wv < (int)(blockDim.x >> 6); ++wv)
+            if (sval[wv] > best || (sval[wv] == best && sidx[wv] < bi)) { best = sval[wv]; bi = sidx[wv]; }
+        out[0] = (bi == 0x7fffffff) ? 0 : bi;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Reference layout w[n_in][n_out] (row stride w_stride), operators32.cu:18-83.
+// Workgroup (ct, sp): columns 256*ct .. +255, rows of split sp.  Lane cx of
+// wave ky handles VEC consecutive columns of rows ky, ky+4, ...; x[j]*r[j] is
+// wave-uniform.  Partials go to scratch[sp][m][k]; mm8_ref_reduce_kernel adds
+// them in split order and accumulates into y (deterministic).
+// ---------------------------------------------------------------------------
+constexpr int kRefSplitRows = 128;
+
+template <int NM, int VEC>
+__global__ void __launch_bounds__(kThreads)
+mm8_ref_partial_kernel(int n_in, int n_out,
+                       const float *x0, const float *x1, const float *x2,
+                       const uint8_t *w0, const uint8_t *w1, const uint8_t *w2,
+                       int64_t s0, int64_t s1, int64_t s2,
+                       const float *r0, const float *r1, const float *r2,
+                       float *__restrict__ scratch) {
+    __shared__ float xs[NM][kRefSplitRows];
+    __shared__ float red[kWaves][NM][64 * VEC];
+    const float *xp[3] = {x0, x1, x2};
+    const float *rp[3] = {r0, r1, r2};
+    const uint8_t *wp[3] = {w0, w1, w2};
+    const int64_t sp_[3] = {s0, s1, s2};
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int j0 = blockIdx.y * kRefSplitRows;
+    const int rows = min(kRefSplitRows, n_in - j0);
+    for (int i = threadIdx.x; i < NM * kRefSplitRows; i += kThreads) {
+        const int m = i / kRefSplitRows, jj = i % kRefSplitRows;
+        // operators32.cu:33-36 multiplies x[j] * (w * r[j]); here x[j]*r[j] is
+        // formed once per row (same rounding as the reference CPU path,
+        // matmul.py:131).
+        xs[m][jj] = jj < rows ? xp[m][j0 + jj] * rp[m][j0 + jj] : 0.f;
+    }
+    __syncthreads();
+    const int k0 = (blockIdx.x * 64 + lane) * VEC;
+    float acc[NM][VEC];
+#pragma unroll
+    for (int m = 0; m < NM; ++m)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[m][e] = 0.f;
+    if (k0 < n_out) {
+        for (int jj = wave; jj < rows; jj += kWaves) {
+#pragma unroll
+            for (int m = 0; m < NM; ++m) {
+                const uint8_t *row = wp[m] + (size_t)(j0 + jj) * sp_[m] + k0;
+                const float xv = xs[m][jj];
+                if (VEC == 4) {
+                    uint32_t d;
+                    if (k0 + 4 <= n_out) {
+                        d = *reinterpret_cast<const uint32_t *>(row);
+                    } else {   // ragged last group: never read past the row
+                        d = 0;
+                        for (int e = 0; k0 + e < n_out; ++e) d |= (uint32_t)row[e] << (8 * e);
+                    }
+                    acc[m][0] = fmaf(ubyte0(d), xv, acc[m][0]);
+                    acc[m][1] = fmaf(ubyte1(d), xv, acc[m][1]);
+                    acc[m][2] = fmaf(ubyte2(d), xv, acc[m][2]);
+                    acc[m][3] = fmaf(ubyte3(d), xv, acc[m][3]);
+                } else {
+                    acc[m][0] = fmaf((float)row[0], xv, acc[m][0]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < NM; ++m)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) red[wave][m][lane * VEC + e] = acc[m][e];
+    __syncthreads();
+    for (int i = threadIdx.x; i < NM * 64 * VEC; i += kThreads) {
+        const int m = i / (64 * VEC), kk = i % (64 * VEC);
+        const int k = blockIdx.x * 64 * VEC + kk;
+        if (k < n_out)
+            scratch[((size_t)blockIdx.y * NM + m) * n_out + k] =
+                (red[0][m][kk] + red[1][m][kk]) + (red[2][m][kk] + red[3][m][kk]);
+    }
+}
+
+template <int NM>
+__global__ void __launch_bounds__(256)
+mm8_ref_reduce_kernel(int n_out, int n_split, const float *__restrict__ scratch,
+                      float *y0, float *y1, float *y2) {
+    float *yp[3] = {y0, y1, y2};
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= n_out) return;
+#pragma unroll
+    for (int m = 0; m < NM; ++m) {
+        float s = 0.f;
+        for (int sp = 0; sp < n_split; ++sp) s += scratch[((size_t)sp * NM + m) * n_out + k];
+        yp[m][k] += s;   // the reference accumulates into y (operators32.cu:38)
+    }
+}
+
+static int mm8_ref_launch(hipStream_t st, int nm, int64_t n_in, int64_t n_out,
+                          const float *const x[3], const uint8_t *const w[3], const int64_t stride[3],
+                          float *const y[3], const float *const r[3], void *ws, size_t ws_bytes) {
+    RWKV_CHECK_ARG(n_in > 0 && n_out > 0 && n_in < (1 << 30) && n_out < (1 << 30), "mm8: bad sizes");
+    bool vec4 = true;
+    for (int m = 0; m < nm; ++m) {
+        RWKV_CHECK_ARG(x[m] && w[m] && y[m] && r[m], "mm8: null pointer");
+        RWKV_CHECK_ARG(stride[m] >= n_out, "mm8: w_stride < n_out");
+        RWKV_CHECK_ALIGN(x[m], 4); RWKV_CHECK_ALIGN(y[m], 4); RWKV_CHECK_ALIGN(r[m], 4);
+        if (reinterpret_cast<uintptr_t>(w[m]) % 4 || stride[m] % 4) vec4 = false;
+    }
+    const size_t need = rwkv_mm8_workspace_bytes(n_in, n_out, nm);
+    if (!ws || ws_bytes < need)
+        return set_error(RWKV_ERR_WORKSPACE, "mm8: workspace of %zu bytes needed, %zu given", need, ws_bytes);
+    RWKV_CHECK_ALIGN(ws, 4);
+    const int n_split = (int)ceil_div(n_in, kRefSplitRows);
+    float *scratch = static_cast<float *>(ws);
+    const int vec = vec4 ? 4 : 1;
+    dim3 grid((unsigned)ceil_div(n_out, 64 * vec), (unsigned)n_split);
+#define LAUNCH_P(NM, VEC) \
+    hipLaunchKernelGGL((mm8_ref_partial_kernel<NM, VEC>), grid, dim3(kThreads), 0, st, (int)n_in, (int)n_out, \
+                       x[0], x[1], x[2], w[0], w[1], w[2], stride[0], stride[1], stride[2], r[0], r[1], r[2], scratch)
+    if (nm == 1) { if (vec4) LAUNCH_P(1, 4); else LAUNCH_P(1, 1); }
+    else         { if (vec4) LAUNCH_P(3, 4); else LAUNCH_P(3, 1); }
+#undef LAUNCH_P
+    RWKV_CHECK_LAUNCH("mm8_ref_partial_kernel");
+    dim3 rgrid((unsigned)ceil_div(n_out, 256));
+    if (nm == 1)
+        hipLaunchKernelGGL(mm8_ref_reduce_kernel<1>, rgrid, dim3(256), 0, st, (int)n_out, n_split, scratch, y[0], y[1], y[2]);
+    else
+        hipLaunchKernelGGL(mm8_ref_reduce_kernel<3>, rgrid, dim3(256), 0, st, (int)n_out, n_split, scratch, y[0], y[1], y[2]);
+    RWKV_CHECK_LAUNCH("mm8_ref_reduce_kernel");
+    return RWKV_OK;
+}
+
+}  // namespace rwkv
+
+using namespace rwkv;
+
+extern "C" {
+
+size_t rwkv_mm8_workspace_bytes(int64_t n_in, int64_t n_out, int n_mat) {
+    if (n_in <= 0 || n_out <= 0 || n_mat <= 0) return 0;
+    return (size_t)(ceil_div(n_in, kRefSplitRows) * n_mat * n_out) * sizeof(float);
+}
+
+int rwkv_mm8_one(rwkv_stream_t stream, int64_t n_in, int64_t n_out, const float *x, const uint8_t *w,
+                 int64_t w_stride, float *y, const float *r, void *workspace, size_t workspace_bytes) {
+    const float *xs[3] = {x, x, x};
+    const uint8_t *ws_[3] = {w, w, w};
+    const int64_t st[3] = {w_stride, w_stride, w_stride};
+    float *ys[3] = {y, y, y};
+    const float *rs[3] = {r, r, r};
+    return mm8_ref_launch((hipStream_t)stream, 1, n_in, n_out, xs, ws_, st, ys, rs, workspace, workspace_bytes);
+}
+
+int rwkv_mm8_three(rwkv_stream_t stream, int64_t n_in, int64_t n_out,
+                   const float *x0, const float *x1, const float *x2,
+                   const uint8_t *w0, int64_t w0_stride, const uint8_t *w1, int64_t w1_stride,
+                   const uint8_t *w2, int64_t w2_stride, float *y0, float *y1, float *y2,
+                   const float *r0, const float *r1, const float *r2,
+                   void *workspace, size_t workspace_bytes) {
+    const float *xs[3] = {x0, x1, x2};
+    const uint8_t *ws_[3] = {w0, w1, w2};
+    const int64_t st[3] = {w0_stride, w1_stride, w2_stride};
+    float *ys[3] = {y0, y1, y2};
+    const float *rs[3] = {r0, r1, r2};
+    return mm8_ref_launch((hipStream_t)stream, 3, n_in, n_out, xs, ws_, st, ys, rs, workspace, workspace_bytes);
+}
+
+int rwkv_wkv_forward_f64(rwkv_stream_t stream, int64_t B, int64_t T, int64_t C,
+                         const double *w, const double *u, const double *k, const double *v,
+                         double *y, double *aa, double *bb, double *pp) {
+    RWKV_CHECK_ARG(w && u && k && v && y && aa && bb && pp, "rwkv_wkv_forward_f64: null pointer");
+    RWKV_CHECK_ARG(B > 0 && T > 0 && C > 0 && B * C < (1ll << 31) && T < (1ll << 31), "rwkv_wkv_forward_f64: bad sizes");
+    RWKV_CHECK_ALIGN(k, 8); RWKV_CHECK_ALIGN(v, 8); RWKV_CHECK_ALIGN(y, 8);
+    hipLaunchKernelGGL(wkv_f64_ref_kernel, dim3((unsigned)ceil_div(B * C, 64)), dim3(64), 0, (hipStream_t)stream,
+                       (int)B, (int)T, (int)C, w, u, k, v, y, aa, bb);
+    RWKV_CHECK_LAUNCH("wkv_f64_ref_kernel");
+    (void)pp;  // passed through untouched, as in the reference kernel
+    return RWKV_OK;
+}
+
+int rwkv_wkv_f32(rwkv_stream_t stream, int64_t B, int64_t T, int64_t C, const float *w, const float *u,
+                 const float *k, const float *v, float *y, float *aa, float *bb, float *pp) {
+    RWKV_CHECK_ARG(w && u && k && v && y && aa && bb && pp, "rwkv_wkv_f32: null pointer");
+    RWKV_CHECK_ARG(B > 0 && T > 0 && C > 0 && B * C < (1ll << 31) && T < (1ll << 31), "rwkv_wkv_f32: bad sizes");
+    RWKV_CHECK_ALIGN(k, 4); RWKV_CHECK_ALIGN(v, 4); RWKV_CHECK_ALIGN(y, 4);
+    hipLaunchKernelGGL(wkv_f32_kernel, dim3((unsigned)ceil_div(B * C, 64)), dim3(64), 0, (hipStream_t)stream,
+                       (int)B, (int)T, (int)C, w, u, k, v, y, aa, bb, pp);
+    RWKV_CHECK_LAUNCH("wkv_f32_kernel");
+    return RWKV_OK;
+}
+
+int rwkv_argmax_f64(rwkv_stream_t stream, const double *logits, int64_t V, int64_t *out_token) {
+    RWKV_CHECK_ARG(logits && out_token, "rwkv_argmax_f64: null pointer");
+    RWKV_CHECK_ARG(V > 0 && V < (1ll << 31), "rwkv_argmax_f64: bad size");
+    hipLaunchKernelGGL(argmax_f64_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, logits, (int)V, out_token);
+    RWKV_CHECK_LAUNCH("argmax_f64_kernel");
+    return RWKV_OK;
+}
+
+int rwkv_mm8_packed(rwkv_stream_t stream, int64_t B, int64_t n_in, int64_t n_out, const float *x,
+                    const uint8_t *packed, const float *r_row, const double *m_row,
+                    const float *r_col, const float *m_col, double *y) {
+    RWKV_CHECK_ARG(x && packed && r_row && m_row && y, "rwkv_mm8_packed: null pointer");
+    RWKV_CHECK_ARG(n_in > 0 && n_out > 0 && n_in < (1 << 30) && n_out < (1 << 30), "rwkv_mm8_packed: bad sizes");
+    if (!(B == 1 || B == 2 || B == 4 || B == 8))
+        return set_error(RWKV_ERR_SIZE, "rwkv_mm8_packed: B must be 1, 2, 4 or 8 (got %lld)", (long long)B);
+    RWKV_CHECK_ALIGN(packed, 16);
+    RWKV_CHECK_ALIGN(x, 4); RWKV_CHECK_ALIGN(r_row, 4); RWKV_CHECK_ALIGN(m_row, 8); RWKV_CHECK_ALIGN(y, 8);
+    const int n_kb = (int)ceil_div(n_in, kBlockRows);
+    // LDS budget for the staged activations: 48 KiB per chunk
+    int kc_blocks = (int)(49152 / (B * kBlockRows * 4));
+    if (kc_blocks > n_kb) kc_blocks = n_kb;
+    const size_t lds = (size_t)B * kc_blocks * kBlockRows * 4 + 2 * B * kWaves * 8 + B * kWaves * 8 * 4;
+    dim3 grid((unsigned)ceil_div(n_out, kTileCols));
+    hipStream_t st = (hipStream_t)stream;
+#define LAUNCH_B(NB) \
+    hipLaunchKernelGGL(mm8_packed_kernel<NB>, grid, dim3(kThreads), lds, st, (int)n_in, (int)n_out, n_kb, kc_blocks, \
+                       x, packed, r_row, m_row, r_col, m_col, y)
+    switch (B) {
+        case 1: LAUNCH_B(1); break;
+        case 2: LAUNCH_B(2); break;
+        case 4: LAUNCH_B(4); break;
+        default: LAUNCH_B(8); break;
+    }
+#undef LAUNCH_B
+    RWKV_CHECK_LAUNCH("mm8_packed_kernel");
+    return RWKV_OK;
+}
+
+}  // extern "C"

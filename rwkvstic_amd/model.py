@@ -1,0 +1,214 @@
+"""FASTQUANT RWKV-4 model on the HIP backend.
+
+``HipRWKV`` plays the role of the reference's ``myRWKV`` module
+(reference src/rwkvstic/agnostic/backends/opt.py:27-84): same constructor
+inputs (a BlinkDL ``.pth`` state dict), same ``forward(tokens, state) ->
+(logits[V], state[L,5,C])`` contract, same ``emptyState``.  Loading quantises
+every matrix on the GPU with the reference scheme (matmul.py:18-40) and repacks
+it into the streaming block layout; the forward pass is one C-ABI call.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Dict, Iterable, List, Optional, Tuple, Union
+
+import torch
+
+from . import _native as N
+from . import ops
+
+
+class QuantMatrix:
+    """Device-resident quantised matrix: packed codes + per-input-channel range/offset."""
+
+    def __init__(self, packed: torch.Tensor, rng: torch.Tensor, off: torch.Tensor, n_in: int, n_out: int):
+        self.packed, self.range, self.offset, self.n_in, self.n_out = packed, rng, off, n_in, n_out
+
+    @classmethod
+    def from_weight(cls, weight: torch.Tensor, device) -> "QuantMatrix":
+        """``weight[out, in]`` in any float dtype, on any device."""
+        w = weight.to(device=device, dtype=torch.float32).contiguous()
+        codes, rng, off = ops.quantize(w)
+        n_in, n_out = codes.shape
+        packed = ops.pack(codes)
+        return cls(packed, rng, off, n_in, n_out)
+
+    @classmethod
+    def from_codes(cls, codes: torch.Tensor, rng: torch.Tensor, off: torch.Tensor, device) -> "QuantMatrix":
+        """From the reference/.rwkv layout: ``codes[in, out]`` uint8, ``range[in]``, ``offset[in]``."""
+        codes = codes.to(device)
+        n_in, n_out = codes.shape
+        return cls(ops.pack(codes), rng.to(device=device, dtype=torch.float32).contiguous(),
+                   off.to(device=device, dtype=torch.float64).contiguous(), n_in, n_out)
+
+    def codes(self) -> torch.Tensor:
+        return ops.unpack(self.packed, self.n_in, self.n_out)
+
+    def desc(self) -> N.QMat:
+        return N.QMat(self.packed.data_ptr(), self.range.data_ptr(), self.offset.data_ptr(), self.n_in, self.n_out)
+
+    def nbytes(self) -> int:
+        return self.n_in * self.n_out
+
+
+class HipRWKV:
+    def __init__(self, weights: Union[Dict[str, torch.Tensor], Iterable[Tuple[str, torch.Tensor]]],
+                 device: str = "cuda"):
+        if not torch.cuda.is_available():
+            raise RuntimeError("HipRWKV needs a ROCm GPU (gfx950); there is no CPU path in this backend")
+        N.lib()
+        self.device = torch.device(device)
+        f64 = dict(device=self.device, dtype=torch.float64)
+        items = weights.items() if isinstance(weights, dict) else weights
+        vec: Dict[str, torch.Tensor] = {}
+        mats: Dict[str, QuantMatrix] = {}
+        self.emb: Optional[torch.Tensor] = None
+        for key, t in items:
+            if key == "emb.weight":
+                self.emb = t.to(device=self.device, dtype=torch.float32).contiguous()
+            elif key.endswith(".weight") and t.dim() == 2:
+                mats[key] = QuantMatrix.from_weight(t, self.device)
+            else:
+                vec[key] = t
+        if self.emb is None:
+            raise KeyError("emb.weight")
+        # opt.py:96-98
+        self.dims = mats["blocks.0.att.key.weight"].n_out
+        self.layers = len([k for k in vec if "blocks" in k and "ln1.bias" in k])
+        self.ffn = mats["blocks.0.ffn.key.weight"].n_out
+        self.vocab = self.emb.shape[0]
+        Cn = self.dims
+
+        def v64(key):
+            return vec[key].reshape(-1).to(**f64).contiguous()
+
+        self._keep: List[torch.Tensor] = []
+        self.ln0 = (v64("blocks.0.ln0.weight"), v64("blocks.0.ln0.bias"))
+        self.ln_out = (v64("ln_out.weight"), v64("ln_out.bias"))
+        self.head = mats["head.weight"]
+        self.blocks: List[dict] = []
+        for i in range(self.layers):
+            p = f"blocks.{i}."
+            blk = dict(
+                ln1_w=v64(p + "ln1.weight"), ln1_b=v64(p + "ln1.bias"),
+                ln2_w=v64(p + "ln2.weight"), ln2_b=v64(p + "ln2.bias"),
+                # block.py:35-47
+                att_mix=torch.stack([v64(p + "att.time_mix_k"), v64(p + "att.time_mix_v"),
+                                     v64(p + "att.time_mix_r")]).contiguous(),
+                ffn_mix=torch.stack([v64(p + "ffn.time_mix_k"), v64(p + "ffn.time_mix_r")]).contiguous(),
+                time_first=v64(p + "att.time_first"),
+                time_decay=v64(p + "att.time_decay").exp().neg().contiguous(),
+                att_k=mats[p + "att.key.weight"], att_v=mats[p + "att.value.weight"],
+                att_r=mats[p + "att.receptance.weight"], att_o=mats[p + "att.output.weight"],
+                ffn_k=mats[p + "ffn.key.weight"], ffn_r=mats[p + "ffn.receptance.weight"],
+                ffn_v=mats[p + "ffn.value.weight"],
+            )
+            self.blocks.append(blk)
+        # opt.py:31-32,80
+        es = torch.zeros((self.layers, 5, Cn), **f64)
+        es[:, 4] = -1e30
+        self.emptyState = es
+        self._build_handle()
+
+    # ------------------------------------------------------------------
+    def _build_handle(self) -> None:
+        L = N.lib()
+        self._layer_arr = (N.LayerDesc * self.layers)()
+        for i, b in enumerate(self.blocks):
+            d = self._layer_arr[i]
+            for name in ("ln1_w", "ln1_b", "ln2_w", "ln2_b", "att_mix", "ffn_mix", "time_decay", "time_first"):
+                setattr(d, name, b[name].data_ptr())
+            for name in ("att_k", "att_v", "att_r", "att_o", "ffn_k", "ffn_r", "ffn_v"):
+                setattr(d, name, b[name].desc())
+        desc = N.ModelDesc(self.layers, self.dims, self.ffn, self.vocab, self.emb.data_ptr(),
+                           self.ln0[0].data_ptr(), self.ln0[1].data_ptr(),
+                           self.ln_out[0].data_ptr(), self.ln_out[1].data_ptr(),
+                           self.head.desc(), self._layer_arr)
+        handle = C.c_void_p()
+        with torch.cuda.device(self.device):
+            N.check(L.rwkv_model_create(C.byref(desc), C.byref(handle)))
+        self._handle = handle
+        self._ws: Optional[torch.Tensor] = None
+        self._ws_tokens = 0
+
+    def __del__(self):
+        h = getattr(self, "_handle", None)
+        if h:
+            try:
+                N.lib().rwkv_model_destroy(h)
+            except Exception:
+                pass
+            self._handle = None
+
+    def _workspace(self, T: int) -> torch.Tensor:
+        if self._ws is None or T > self._ws_tokens:
+            nbytes = N.lib().rwkv_model_workspace_bytes(self._handle, T)
+            self._ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+            self._ws_tokens = T
+        return self._ws
+
+    def weight_bytes(self) -> int:
+        """uint8 weight bytes streamed per decoded token: L*13*C^2 + V*C."""
+        n = self.head.nbytes()
+        for b in self.blocks:
+            n += sum(b[k].nbytes() for k in ("att_k", "att_v", "att_r", "att_o", "ffn_k", "ffn_r", "ffn_v"))
+        return n
+
+    # ------------------------------------------------------------------
+    def _check_state(self, state: torch.Tensor) -> None:
+        if (not isinstance(state, torch.Tensor) or state.device.type != "cuda" or state.dtype != torch.float64
+                or tuple(state.shape) != (self.layers, 5, self.dims) or not state.is_contiguous()):
+            raise ValueError(f"state must be a contiguous CUDA float64 tensor of shape "
+                             f"({self.layers}, 5, {self.dims})")
+
+    def forward(self, tokens, state: torch.Tensor):
+        """``(logits[V] float64, state)``; ``state`` is updated in place and returned (opt.py:61-76)."""
+        tok = torch.as_tensor(tokens, dtype=torch.int64).reshape(-1).to(self.device)
+        if tok.numel() == 0:
+            raise ValueError("forward needs at least one token")
+        self._check_state(state)
+        T = tok.numel()
+        ws = self._workspace(T)
+        logits = torch.empty(self.vocab, dtype=torch.float64, device=self.device)
+        with torch.cuda.device(self.device):
+            N.check(N.lib().rwkv_model_forward(self._handle, torch.cuda.current_stream().cuda_stream,
+                                               tok.data_ptr(), T, state.data_ptr(), logits.data_ptr(),
+                                               ws.data_ptr(), ws.numel()))
+        return logits, state
+
+    __call__ = forward
+
+    def decode_greedy(self, token: int, n: int, state: torch.Tensor):
+        """Feed ``token`` then greedily generate: returns ``(tokens[n] int64 on device, last logits, state)``
+        where ``tokens[i] = argmax(forward(previous token))``.  No host round trip per token."""
+        self._check_state(state)
+        toks = torch.empty(n + 1, dtype=torch.int64, device=self.device)
+        toks[0] = int(token)
+        ws = self._workspace(1)
+        logits = torch.empty(self.vocab, dtype=torch.float64, device=self.device)
+        with torch.cuda.device(self.device):
+            N.check(N.lib().rwkv_model_decode_greedy(self._handle, torch.cuda.current_stream().cuda_stream,
+                                                     toks.data_ptr(), n, state.data_ptr(), logits.data_ptr(),
+                                                     ws.data_ptr(), ws.numel()))
+        return toks[1:], logits, state
+
+
+def wkv_state_to_reference(state: torch.Tensor) -> torch.Tensor:
+    """Rows 2-4 hold the max-shifted triple ``(aa', bb', pp')``; the reference's naive kernel keeps
+    ``aa = aa' e^{pp'}``, ``bb = bb' e^{pp'}`` and never touches ``pp`` (cuda/operators.cu:21-36).
+    Returns a copy in the reference convention (pp reset to -1e30)."""
+    out = state.clone()
+    e = torch.exp(state[:, 4])
+    out[:, 2] = state[:, 2] * e
+    out[:, 3] = state[:, 3] * e
+    out[:, 4] = -1e30
+    return out
+
+
+def wkv_state_from_reference(state: torch.Tensor) -> torch.Tensor:
+    """Inverse of :func:`wkv_state_to_reference`: a naive ``(aa, bb)`` is the shifted triple with ``pp' = 0``
+    (or the empty state where ``bb == 0``)."""
+    out = state.clone()
+    empty = ~(state[:, 3] > 0)
+    out[:, 4] = torch.where(empty, torch.full_like(state[:, 4], -1e30), torch.zeros_like(state[:, 4]))
+    return out

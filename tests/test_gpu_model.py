@@ -1,0 +1,127 @@
+"""GPU parity of the whole-model forward against the CPU oracle (the reference's CPU path restated)."""
+import pytest
+import torch
+
+from oracle import rwkv_oracle as O
+from rwkvstic_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+LOGIT_TOL = 1e-3       # max-abs on logits
+STATE_TOL = 1e-4       # relative, WKV state in the reference convention
+
+
+def _say(msg):
+    print(msg, flush=True)
+
+
+def _state_close(st_gpu, st_ref, tol=STATE_TOL):
+    from rwkvstic_amd.model import wkv_state_to_reference
+    s = wkv_state_to_reference(st_gpu).cpu()
+    # shift rows: LayerNorm outputs, O(1)
+    assert (s[:, 0] - st_ref[:, 0]).abs().max() < 1e-4
+    assert (s[:, 1] - st_ref[:, 1]).abs().max() < 1e-4
+    bb_ref = st_ref[:, 3]
+    assert ((s[:, 3] - bb_ref).abs() <= tol * bb_ref.abs() + 1e-30).all(), "bb"
+    assert ((s[:, 2] - st_ref[:, 2]).abs() <= tol * torch.maximum(st_ref[:, 2].abs(), bb_ref) + 1e-30).all(), "aa"
+
+
+@pytest.fixture(scope="module")
+def tiny():
+    from rwkvstic_amd.model import HipRWKV
+    sd = synth.make_state_dict(layers=3, C=64, V=512, seed=5)
+    return O.OracleModel(sd), HipRWKV(sd)
+
+
+def test_tiny_single_tokens(tiny):
+    ref, hip = tiny
+    assert hip.layers == 3 and hip.dims == 64 and hip.vocab == 512
+    assert torch.equal(hip.emptyState.cpu(), ref.emptyState)
+    toks = synth.random_tokens(12, V=512, seed=3).tolist()
+    sr, sg = ref.emptyState.clone(), hip.emptyState.clone()
+    for i, t in enumerate(toks):
+        _say(f"tiny token {i}")
+        lr, sr = ref.forward([t], sr)
+        lg, sg = hip.forward([t], sg)
+        assert (lg.cpu() - lr).abs().max() < LOGIT_TOL
+        assert int(lg.argmax()) == int(lr.argmax())
+    _state_close(sg, sr)
+
+
+def test_tiny_chunked_prefill_matches_oracle_and_single_steps(tiny):
+    ref, hip = tiny
+    toks = synth.random_tokens(19, V=512, seed=4).tolist()
+    lr, sr = ref.forward(toks, ref.emptyState.clone())
+    lg, sg = hip.forward(toks, hip.emptyState.clone())
+    assert (lg.cpu() - lr).abs().max() < LOGIT_TOL
+    _state_close(sg, sr)
+    # chunk-size invariance on the GPU path itself
+    s2 = hip.emptyState.clone()
+    l2, s2 = hip.forward(toks[:7], s2)
+    l2, s2 = hip.forward(toks[7:], s2)
+    assert (l2 - lg).abs().max() < 1e-5
+    assert (s2[:, :2] - sg[:, :2]).abs().max() < 1e-6
+
+
+def test_ragged_shape_model():
+    """C not a multiple of 128, V not a multiple of 8, F != 4C."""
+    from rwkvstic_amd.model import HipRWKV
+    sd = synth.make_state_dict(layers=2, C=72, F=200, V=301, seed=8)
+    ref, hip = O.OracleModel(sd), HipRWKV(sd)
+    toks = synth.random_tokens(6, V=301, seed=1).tolist()
+    sr, sg = ref.emptyState.clone(), hip.emptyState.clone()
+    for t in toks:
+        lr, sr = ref.forward([t], sr)
+        lg, sg = hip.forward([t], sg)
+        assert (lg.cpu() - lr).abs().max() < LOGIT_TOL
+    _state_close(sg, sr)
+
+
+def test_decode_greedy_device_loop_matches_host_loop(tiny):
+    ref, hip = tiny
+    s1 = hip.emptyState.clone()
+    toks, logits, s1 = hip.decode_greedy(17, 10, s1)
+    s2 = hip.emptyState.clone()
+    t, out = 17, []
+    for _ in range(10):
+        l2, s2 = hip.forward([t], s2)
+        t = int(l2.argmax()); out.append(t)
+    assert toks.tolist() == out
+    assert torch.equal(logits, l2) and torch.equal(s1, s2)
+
+
+def test_forward_rejects_bad_state(tiny):
+    _, hip = tiny
+    with pytest.raises(ValueError):
+        hip.forward([1], hip.emptyState.clone().float())
+    with pytest.raises(ValueError):
+        hip.forward([1], hip.emptyState.clone()[:2])
+    with pytest.raises(ValueError):
+        hip.forward([], hip.emptyState.clone())
+
+
+def test_169m_shape_greedy_128_tokens():
+    """The plumbing configuration: 12 layers, C=768, F=3072, V=50277; 32-token prompt, 128 greedy tokens."""
+    from rwkvstic_amd.model import HipRWKV
+    L, C, F, V = synth.SHAPES["169M"]
+    sd = synth.make_state_dict(L, C, F, V, seed=0)
+    ref, hip = O.OracleModel(sd), HipRWKV(sd)
+    assert hip.weight_bytes() == 130_625_280
+    prompt = synth.random_tokens(32, V=V, seed=0).tolist()
+    _say("169M oracle greedy (CPU) ...")
+    toks_r, logits_r, st_r = ref.greedy(prompt, 128)
+    _say("169M GPU prefill + greedy ...")
+    st = hip.emptyState.clone()
+    lg, st = hip.forward(prompt, st)
+    worst = 0.0
+    toks_g = []
+    for i in range(128):
+        worst = max(worst, float((lg.cpu() - logits_r[i]).abs().max()))
+        t = int(lg.argmax())
+        toks_g.append(t)
+        lg, st = hip.forward([t], st)
+    worst = max(worst, float((lg.cpu() - logits_r[128]).abs().max()))
+    _say(f"169M worst logit max-abs {worst:.3e}")
+    assert toks_g == toks_r, "greedy tokens differ from the CPU oracle"
+    assert worst <= LOGIT_TOL
+    _state_close(st, st_r)

@@ -1,0 +1,238 @@
+"""GPU parity of the stand-alone operators against the CPU oracle.
+Every case goes through the C ABI (rwkvstic_amd.ops -> ctypes -> librwkv_hip.so)."""
+import pytest
+import torch
+
+from oracle import rwkv_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from rwkvstic_amd import ops as _ops
+    return _ops
+
+
+def _say(msg):
+    print(msg, flush=True)
+
+
+# ------------------------------------------------------------------ quantiser + layouts
+@pytest.mark.parametrize("shape", [(8, 8), (5, 3), (300, 130), (3072, 768), (2560, 2560), (1000, 257)])
+def test_quantiser_bit_exact_codes_and_1ulp_dequant(ops, shape):
+    _say(f"quantise {shape}")
+    g = torch.Generator().manual_seed(shape[0] * 7 + shape[1])
+    W = torch.randn(*shape, generator=g) * 0.02
+    c_ref, r_ref, o_ref = O.quantize_matrix(W)
+    codes, rng, off = ops.quantize(W.cuda())
+    torch.cuda.synchronize()
+    assert torch.equal(codes.cpu(), c_ref), "codes differ"
+    assert torch.equal(rng.cpu(), r_ref), "range differs"
+    # offset differs only by the summation order of the mean fraction
+    assert torch.allclose(off.cpu(), o_ref, rtol=1e-13, atol=1e-300)
+    packed = ops.pack(codes)
+    assert torch.equal(ops.unpack(packed, *codes.shape).cpu(), c_ref), "pack/unpack round trip"
+    dq = ops.dequant_packed(packed, rng, off, *codes.shape).cpu()
+    want = O.dequant_canonical(c_ref, r_ref, o_ref)
+    ulp = torch.abs(torch.nextafter(want, torch.full_like(want, float("inf"))) - want)
+    assert ((dq - want).abs() <= ulp).all(), "dequantised weights differ by more than 1 ulp"
+
+
+def test_quantiser_constant_channel(ops):
+    W = torch.randn(40, 16) * 0.02
+    W[:, 3] = 0.125
+    codes, rng, off = ops.quantize(W.cuda())
+    assert int(codes[3].max()) == 0 and float(rng[3]) == 0.0 and float(off[3]) == 0.125
+
+
+def test_pack_strided_and_ragged(ops):
+    big = torch.randint(0, 256, (200, 400), dtype=torch.uint8, device="cuda")
+    view = big[:130, :77]                      # stride 400, ragged in both dims
+    packed = ops.pack(view)
+    assert torch.equal(ops.unpack(packed, 130, 77), view)
+
+
+# ------------------------------------------------------------------ packed matvec (isolated workload)
+SHAPES = [(2560, 2560), (2560, 10240), (10240, 2560)]
+
+
+@pytest.mark.parametrize("n_in,n_out", SHAPES + [(96, 40), (130, 77), (768, 50277)])
+@pytest.mark.parametrize("B", [1, 8])
+def test_mm8_packed_general_form(ops, n_in, n_out, B):
+    _say(f"mm8_packed in={n_in} out={n_out} B={B}")
+    g = torch.Generator().manual_seed(n_in + 3 * n_out + B)
+    codes = torch.randint(0, 256, (n_in, n_out), generator=g, dtype=torch.uint8)
+    m_row = torch.randn(n_in, generator=g) * 0.01
+    m_col = torch.randn(n_out, generator=g) * 0.01
+    r_row = torch.rand(n_in, generator=g) * 9e-4 + 1e-4
+    r_col = torch.rand(n_out, generator=g) * 9e-4 + 1e-4
+    x = torch.randn(B, n_in, generator=g)
+    want = O.mm8_general_f64(x, codes, r_row, m_row, r_col, m_col)
+    packed = ops.pack(codes.cuda())
+    got = ops.mm8_packed(x.cuda(), packed, n_in, n_out, r_row.cuda(), m_row.double().cuda(),
+                         r_col.cuda(), m_col.cuda()).cpu()
+    # float32 accumulation of n_in terms: bound n * 2^-23 * max |partial sum scale|
+    scale = (x.abs().double() * r_row.double()) @ codes.double() * r_col.double()
+    tol = 2.0 ** -23 * 8 * scale.max()
+    err = (got - want).abs().max()
+    _say(f"  max err {err:.3e} tol {tol:.3e} |y| {want.abs().max():.3e}")
+    assert err <= tol
+
+
+@pytest.mark.parametrize("B", [1, 2, 4])
+def test_mm8_packed_reference_form_matches_cpu_path(ops, B):
+    """r_col = m_col = None is MM8.forward; compare with the oracle's mm8_naive."""
+    W = torch.randn(1000, 384) * 0.02
+    c, r, o = O.quantize_matrix(W)
+    x = torch.randn(B, 384)
+    want = O.mm8_naive(x.double(), c, r, o)
+    got = ops.mm8_packed(x.cuda(), ops.pack(c.cuda()), 384, 1000, r.cuda(), o.cuda()).cpu()
+    assert (got - want).abs().max() < 2e-5
+
+
+def test_mm8_packed_rejects_bad_arguments(ops):
+    from rwkvstic_amd._native import RwkvHipError
+    c = torch.zeros((128, 8), dtype=torch.uint8, device="cuda")
+    p = ops.pack(c)
+    x = torch.zeros((3, 128), device="cuda")
+    r = torch.ones(128, device="cuda"); m = torch.zeros(128, dtype=torch.float64, device="cuda")
+    with pytest.raises(RwkvHipError):
+        ops.mm8_packed(x, p, 128, 8, r, m)          # B = 3 unsupported
+    with pytest.raises(ValueError):
+        ops.mm8_packed(x[:1], p[:512], 128, 8, r, m)  # packed too small
+    with pytest.raises(TypeError):
+        ops.mm8_packed(x[:1].double(), p, 128, 8, r, m)
+
+
+# ------------------------------------------------------------------ reference-layout operators
+@pytest.mark.parametrize("n_in,n_out", [(768, 768), (2560, 2560), (96, 50277), (130, 77)])
+def test_mm8_one_reference_semantics(ops, n_in, n_out):
+    _say(f"mm8_one in={n_in} out={n_out}")
+    g = torch.Generator().manual_seed(n_in * 5 + n_out)
+    w = torch.randint(0, 256, (n_in, n_out), generator=g, dtype=torch.uint8)
+    r = torch.rand(n_in, generator=g) * 1e-3
+    x = torch.randn(n_in, generator=g)
+    y0 = torch.randn(n_out, generator=g)
+    want = y0.double() + (x.double() * r.double()) @ w.double()
+    y = y0.clone().cuda()
+    ops.mm8_one(n_in, n_out, x.cuda(), w.cuda(), y, r.cuda())      # accumulates into y
+    scale = ((x.abs().double() * r.double()) @ w.double()).max()
+    assert (y.cpu().double() - want).abs().max() <= 2.0 ** -23 * 8 * scale + 1e-6 * y0.abs().max()
+
+
+def test_mm8_three_matches_three_mm8_one(ops):
+    n_in, n_out = 512, 520
+    g = torch.Generator().manual_seed(11)
+    ws = [torch.randint(0, 256, (n_in, n_out), generator=g, dtype=torch.uint8).cuda() for _ in range(3)]
+    rs = [(torch.rand(n_in, generator=g) * 1e-3).cuda() for _ in range(3)]
+    xs = [torch.randn(n_in, generator=g).cuda() for _ in range(3)]
+    y3 = [torch.zeros(n_out, device="cuda") for _ in range(3)]
+    y1 = [torch.zeros(n_out, device="cuda") for _ in range(3)]
+    ops.mm8_three(n_in, n_out, *xs, *ws, *y3, *rs)
+    for i in range(3):
+        ops.mm8_one(n_in, n_out, xs[i], ws[i], y1[i], rs[i])
+        assert torch.equal(y3[i], y1[i])       # same kernel arithmetic, deterministic
+
+
+def test_mm8_one_strided_rows(ops):
+    big = torch.randint(0, 256, (64, 1003), dtype=torch.uint8, device="cuda")   # odd stride: byte path
+    w = big[:, :1000]
+    x = torch.randn(64, device="cuda"); r = torch.rand(64, device="cuda")
+    y = torch.zeros(1000, device="cuda")
+    ops.mm8_one(64, 1000, x, w, y, r)
+    want = (x.double() * r.double()) @ w.double()
+    assert (y.double() - want).abs().max() < 1e-2 * 1e-3 * want.abs().max() + 1e-3
+
+
+def test_torch_ops_registered_with_reference_schema(ops):
+    ops.register_torch_ops()
+    n_in, n_out = 128, 64
+    w = torch.randint(0, 256, (n_in, n_out), dtype=torch.uint8, device="cuda")
+    x = torch.randn(n_in, device="cuda"); r = torch.rand(n_in, device="cuda")
+    y = torch.zeros(n_out, device="cuda")
+    torch.ops.rwkv.mm8_one(n_in, n_out, x, w, y, r)
+    assert (y.double() - (x.double() * r.double()) @ w.double()).abs().max() < 1e-2
+
+
+# ------------------------------------------------------------------ WKV
+def _wkv_case(B, T, C, seed, lo=-8.0):
+    g = torch.Generator().manual_seed(seed)
+    k = torch.randn(B, T, C, generator=g)
+    v = torch.randn(B, T, C, generator=g)
+    w = -torch.exp(torch.rand(C, generator=g) * (1.0 - lo) + lo)
+    u = torch.rand(C, generator=g) * 2 - 1
+    return w, u, k, v
+
+
+def _check_wkv_f32(ops, B, T, C, seed):
+    w, u, k, v = _wkv_case(B, T, C, seed)
+    aa = torch.zeros(B, C); bb = torch.zeros(B, C); pp = torch.full((B, C), -1e38)
+    d = lambda t: t.cuda()
+    aa_d, bb_d, pp_d = d(aa), d(bb), d(pp)
+    y = ops.wkv_f32(d(w), d(u), d(k), d(v), aa_d, bb_d, pp_d).cpu()
+    for b in range(B):
+        yr, ar, br, _ = O.wkv_naive(w.double(), u.double(), k[b].double(), v[b].double(),
+                                    aa[b].double(), bb[b].double(), pp[b].double())
+        assert (y[b].double() - yr).abs().max() < 1e-4 * max(1.0, float(yr.abs().max()))
+        an, bn = O.state_naive_from_stable(aa_d[b].cpu(), bb_d[b].cpu(), pp_d[b].cpu())
+        # bb is a positive sum; aa is a signed sum of the same weights times v ~ N(0,1)
+        assert ((bn - br).abs() <= 1e-4 * br).all()
+        assert ((an - ar).abs() <= 1e-4 * torch.maximum(ar.abs(), br)).all()
+
+
+def test_wkv_f32_small(ops):
+    _say("wkv_f32 B=2 T=37 C=130")
+    _check_wkv_f32(ops, 2, 37, 130, seed=3)
+
+
+def test_wkv_f32_isolated_workload(ops):
+    _say("wkv_f32 B=8 T=1024 C=2560")
+    _check_wkv_f32(ops, 8, 1024, 2560, seed=2)
+
+
+def test_wkv_f32_split_invariance_and_large_k(ops):
+    """Carrying the state across two calls equals one call; k up to +-60 must not overflow float32."""
+    w, u, k, v = _wkv_case(1, 64, 64, seed=9)
+    k = k * 20
+    d = lambda t: t.cuda()
+    s1 = [torch.zeros(1, 64).cuda(), torch.zeros(1, 64).cuda(), torch.full((1, 64), -1e38).cuda()]
+    y_all = ops.wkv_f32(d(w), d(u), d(k), d(v), *s1)
+    s2 = [torch.zeros(1, 64).cuda(), torch.zeros(1, 64).cuda(), torch.full((1, 64), -1e38).cuda()]
+    ya = ops.wkv_f32(d(w), d(u), d(k[:, :20].contiguous()), d(v[:, :20].contiguous()), *s2)
+    yb = ops.wkv_f32(d(w), d(u), d(k[:, 20:].contiguous()), d(v[:, 20:].contiguous()), *s2)
+    # the exponent is float64 inside a call and rounded to float32 at the call boundary
+    assert torch.allclose(torch.cat([ya, yb], 1), y_all, rtol=2e-5, atol=2e-5)
+    assert torch.isfinite(y_all).all()
+    yr = O.wkv_stable(w.double(), u.double(), k[0].double(), v[0].double(),
+                      torch.zeros(64).double(), torch.zeros(64).double(), torch.full((64,), -1e38).double())[0]
+    assert (y_all[0].cpu().double() - yr).abs().max() < 1e-4 * max(1.0, float(yr.abs().max()))
+
+
+def test_wkv_forward_f64_reference_convention(ops):
+    """Drop-in for torch.ops.rwkv.wkv_forward: naive state in/out, pp untouched."""
+    B, T, C = 1, 50, 96
+    w, u, k, v = _wkv_case(B, T, C, seed=4)
+    w, u, k, v = (t.double() for t in (w, u, k, v))
+    aa = torch.rand(C).double(); bb = torch.rand(C).double() + 0.5; pp = torch.full((C,), -1e30).double()
+    yr, ar, br, pr = O.wkv_naive(w, u, k[0], v[0], aa, bb, pp)
+    d = lambda t: t.cuda()
+    aa_d, bb_d, pp_d = d(aa.clone()), d(bb.clone()), d(pp.clone())
+    y = torch.empty(T, C, dtype=torch.float64, device="cuda")
+    ops.wkv_forward(1, T, C, d(w), d(u), d(k[0].contiguous()), d(v[0].contiguous()), y, aa_d, bb_d, pp_d)
+    assert torch.allclose(y.cpu(), yr, rtol=1e-11, atol=1e-12)
+    assert torch.allclose(aa_d.cpu(), ar, rtol=1e-10) and torch.allclose(bb_d.cpu(), br, rtol=1e-10)
+    assert torch.equal(pp_d.cpu(), pp)
+    # from the empty state too
+    z = torch.zeros(C).double()
+    yr, ar, br, _ = O.wkv_naive(w, u, k[0], v[0], z, z.clone(), pp)
+    aa_d, bb_d = d(z.clone()), d(z.clone())
+    ops.wkv_forward(1, T, C, d(w), d(u), d(k[0].contiguous()), d(v[0].contiguous()), y, aa_d, bb_d, pp_d)
+    assert torch.allclose(y.cpu(), yr, rtol=1e-11, atol=1e-12)
+    assert torch.allclose(bb_d.cpu(), br, rtol=1e-10)
+
+
+def test_argmax_first_maximum(ops):
+    x = torch.randn(50277, dtype=torch.float64)
+    x[40000] = 9.0; x[123] = 9.0
+    assert int(ops.argmax(x.cuda())) == 123
