@@ -114,6 +114,18 @@ int rwkv_pack_u8(rwkv_stream_t stream, const uint8_t *codes, int64_t codes_strid
 int rwkv_unpack_u8(rwkv_stream_t stream, const uint8_t *packed,
                    int64_t n_in, int64_t n_out, uint8_t *codes, int64_t codes_stride);
 
+/* Second device layout, for the single-token matrix-core kernel: 1 KiB blocks
+ * of 16 output columns x 64 input rows, blocks ordered
+ * [ceil(n_out/16)][ceil(n_in/64)], zero padded; byte 16*(16*g + n) + i of a
+ * block holds codes[64*kb + 16*g + i][16*ct + n] - 128 as a signed byte
+ * (g < 4, n < 16, i < 16): one wavefront-wide 16-byte load is the B operand
+ * of v_mfma_i32_16x16x64_i8. */
+size_t rwkv_packed_m16_bytes(int64_t n_in, int64_t n_out);
+int rwkv_pack_m16(rwkv_stream_t stream, const uint8_t *codes, int64_t codes_stride,
+                  int64_t n_in, int64_t n_out, uint8_t *packed);
+int rwkv_unpack_m16(rwkv_stream_t stream, const uint8_t *packed,
+                    int64_t n_in, int64_t n_out, uint8_t *codes, int64_t codes_stride);
+
 /* Canonical dequantisation fp32(fp64(code)*fp64(range[j]) + offset[j]) of a
  * packed matrix into dq[n_in, n_out] float32 row-major (parity/debug). */
 int rwkv_dequant_packed(rwkv_stream_t stream, const uint8_t *packed,
@@ -155,9 +167,12 @@ int rwkv_wkv_f32(rwkv_stream_t stream, int64_t B, int64_t T, int64_t C,
  * ---------------------------------------------------------------------- */
 
 typedef struct rwkv_qmat {
-    const uint8_t *packed; /* rwkv_pack_u8 layout, 16-byte aligned            */
-    const float *range;    /* [n_in]                                          */
-    const double *offset;  /* [n_in]                                          */
+    const uint8_t *packed;   /* rwkv_pack_u8 layout, 16-byte aligned          */
+    const uint8_t *packed16; /* rwkv_pack_m16 layout, 16-byte aligned, or NULL:
+                                without it the single-token step runs as one
+                                launch per phase instead of one per token     */
+    const float *range;      /* [n_in]                                        */
+    const double *offset;    /* [n_in]                                        */
     int64_t n_in, n_out;
 } rwkv_qmat;
 
@@ -181,10 +196,22 @@ typedef struct rwkv_model_desc {
 
 typedef struct rwkv_model rwkv_model;
 
-/* Copies the descriptor (host side); the device buffers it names must outlive
- * the handle. */
+/* Copies the descriptor; the device buffers it names must outlive the handle.
+ * This is the one entry point that allocates device memory (a table of the
+ * layer pointers and three small exchange vectors for the single-token
+ * kernel); rwkv_model_destroy frees it.  One forward call may be in flight
+ * per handle at a time. */
 int rwkv_model_create(const rwkv_model_desc *desc, rwkv_model **out);
 void rwkv_model_destroy(rwkv_model *m);
+
+/* 1 if single-token steps of this handle run as one persistent launch (all
+ * matrices have packed16 and the shape is supported), else 0. */
+int rwkv_model_has_fused_step(const rwkv_model *m);
+
+/* Synchronises the device and returns RWKV_ERR_HIP if a single-token launch
+ * gave up waiting for another workgroup (it then left logits/state
+ * incomplete), else RWKV_OK.  For tests and diagnostics. */
+int rwkv_model_check(rwkv_model *m);
 
 /* Scratch needed by rwkv_model_forward for chunks of up to max_tokens tokens. */
 size_t rwkv_model_workspace_bytes(const rwkv_model *m, int64_t max_tokens);

@@ -75,15 +75,21 @@ def dequant_canonical(codes: Tensor, rng: Tensor, offset: Tensor) -> Tensor:
 # --------------------------------------------------------------------------
 # a12  mm8Naive / mm8_3Naive  (matmul.py:124-142)
 # --------------------------------------------------------------------------
-def mm8_naive(x: Tensor, codes: Tensor, rng: Tensor, offset: Tensor) -> Tensor:
+def mm8_naive(x: Tensor, codes: Tensor, rng: Tensor, offset: Tensor,
+              dtype: torch.dtype = torch.float32) -> Tensor:
     """``fp32(x*range) @ fp32(codes) + (x @ offset)[:, None]`` for ``x[T,in]`` float64.
 
     matmul.py:131: the product ``x*range`` is formed in float64 (float64 times
-    float32 promotes), rounded to float32, multiplied by the float32 cast of
-    the codes with float32 accumulation, and the float64 zero-point term is
-    added last (float32 + float64 -> float64).
+    float32 promotes), rounded to ``dtype``, multiplied by the ``dtype`` cast of
+    the codes with ``dtype`` accumulation, and the float64 zero-point term is
+    added last (float32 + float64 -> float64).  ``dtype`` is the reference's
+    ``naivedtype`` (matmul.py:183: float32 on the CPU by default; float64 is
+    the same network evaluated without accumulation error and is what the
+    float32 path is noisy around: for F = 10240 the float32 sum of the
+    all-positive relu^2 terms cancels against the zero-point term and loses
+    about 1e-4 absolute, by an amount that changes with the BLAS thread count).
     """
-    main = (x * rng).to(torch.float32) @ codes.to(torch.float32)
+    main = (x * rng).to(dtype) @ codes.to(dtype)
     return main + x.mv(offset).reshape(-1, 1)
 
 
@@ -173,18 +179,21 @@ def wkv_stable(w: Tensor, u: Tensor, k: Tensor, v: Tensor,
 class QMat:
     """One quantised matrix in the reference layout (matmul.py:12-16)."""
 
-    def __init__(self, weight: Tensor):
+    def __init__(self, weight: Tensor, dtype: torch.dtype = torch.float32):
         self.codes, self.range, self.offset = quantize_matrix(weight.float())
         self.n_in, self.n_out = self.codes.shape
+        self.dtype = dtype
 
     def __call__(self, x: Tensor) -> Tensor:
-        return mm8_naive(x, self.codes, self.range, self.offset)
+        return mm8_naive(x, self.codes, self.range, self.offset, self.dtype)
 
 
 class OracleModel:
     """CPU restatement of ``myRWKV`` (agnostic/backends/opt.py:27-84)."""
 
-    def __init__(self, w: Dict[str, Tensor]):
+    def __init__(self, w: Dict[str, Tensor], matmul_dtype: torch.dtype = torch.float32):
+        self.matmul_dtype = matmul_dtype
+        QMat = lambda t: globals()["QMat"](t, matmul_dtype)   # noqa: E731  (naivedtype, matmul.py:183)
         self.dims = len(w["blocks.0.att.key.weight"])                 # opt.py:96
         self.layers = len([k for k in w if "blocks" in k and "ln1.bias" in k])  # opt.py:97-98
         f64 = torch.float64

@@ -16,14 +16,16 @@ EXPORTS = (
     "rwkv_version", "rwkv_last_error",
     "rwkv_mm8_workspace_bytes", "rwkv_mm8_one", "rwkv_mm8_three", "rwkv_wkv_forward_f64",
     "rwkv_quantize_u8", "rwkv_packed_bytes", "rwkv_pack_u8", "rwkv_unpack_u8", "rwkv_dequant_packed",
+    "rwkv_packed_m16_bytes", "rwkv_pack_m16", "rwkv_unpack_m16",
     "rwkv_mm8_packed", "rwkv_wkv_f32",
     "rwkv_model_create", "rwkv_model_destroy", "rwkv_model_workspace_bytes",
+    "rwkv_model_has_fused_step", "rwkv_model_check",
     "rwkv_model_forward", "rwkv_model_decode_greedy", "rwkv_argmax_f64",
 )
 
 
 class QMat(C.Structure):
-    _fields_ = [("packed", C.c_void_p), ("range", C.c_void_p), ("offset", C.c_void_p),
+    _fields_ = [("packed", C.c_void_p), ("packed16", C.c_void_p), ("range", C.c_void_p), ("offset", C.c_void_p),
                 ("n_in", C.c_int64), ("n_out", C.c_int64)]
 
 
@@ -76,6 +78,12 @@ def lib() -> C.CDLL:
     L.rwkv_pack_u8.argtypes = [vp, vp, i64, i64, i64, vp]
     L.rwkv_unpack_u8.argtypes = [vp, vp, i64, i64, vp, i64]
     L.rwkv_dequant_packed.argtypes = [vp, vp, vp, vp, i64, i64, vp]
+    L.rwkv_packed_m16_bytes.restype = sz
+    L.rwkv_packed_m16_bytes.argtypes = [i64, i64]
+    L.rwkv_pack_m16.argtypes = [vp, vp, i64, i64, i64, vp]
+    L.rwkv_unpack_m16.argtypes = [vp, vp, i64, i64, vp, i64]
+    L.rwkv_model_has_fused_step.argtypes = [vp]
+    L.rwkv_model_check.argtypes = [vp]
     L.rwkv_mm8_packed.argtypes = [vp, i64, i64, i64, vp, vp, vp, vp, vp, vp, vp]
     L.rwkv_wkv_f32.argtypes = [vp, i64, i64, i64] + [vp] * 8
     L.rwkv_model_create.argtypes = [C.POINTER(ModelDesc), C.POINTER(vp)]

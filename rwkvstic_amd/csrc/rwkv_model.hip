@@ -24,6 +24,7 @@
 // float32 accumulation (matmul.py:58,131); WKV runs in float32 in the
 // max-shifted form.
 #include "rwkv_common.h"
+#include "rwkv_decode.h"
 
 #include <new>
 #include <string>
@@ -340,6 +341,13 @@ using namespace rwkv;
 struct rwkv_model {
     rwkv_model_desc d;
     std::vector<rwkv_layer_desc> layers;
+    // single-token persistent kernel (absent when the shape or layouts do not allow it)
+    bool fused = false;
+    int device = 0;
+    rwkv::DModel dm{};
+    rwkv::DecodeBuffers db{};
+    void *dev_block = nullptr;     // one allocation: layer table + exchange vectors + abort flag
+    unsigned epoch = 0;
 };
 
 namespace {
@@ -438,6 +446,55 @@ int check_forward_args(const rwkv_model *m, const void *tokens, const double *st
     return RWKV_OK;
 }
 
+rwkv::DQ to_dq(const rwkv_qmat &q) { return rwkv::DQ{q.packed16, q.range, q.offset}; }
+
+// Device-side copy of the layer table plus the exchange vectors of the
+// persistent single-token kernel.  Leaves m->fused false when the shape or the
+// supplied layouts do not allow that kernel.
+int setup_fused(rwkv_model *m) {
+    const rwkv_model_desc &d = m->d;
+    if (!decode_supported(d.n_layer, d.n_embd, d.n_ffn, d.n_vocab)) return RWKV_OK;
+    bool all16 = d.head.packed16 != nullptr;
+    for (const rwkv_layer_desc &ld : m->layers)
+        all16 = all16 && ld.att_k.packed16 && ld.att_v.packed16 && ld.att_r.packed16 && ld.att_o.packed16 &&
+                ld.ffn_k.packed16 && ld.ffn_r.packed16 && ld.ffn_v.packed16;
+    if (!all16) return RWKV_OK;
+    const size_t L = (size_t)d.n_layer, C = (size_t)d.n_embd, F = (size_t)d.n_ffn;
+    const size_t table_bytes = round_up(L * sizeof(DLayer), 256);
+    const size_t xchg_bytes = (2 * C + F) * sizeof(u64);
+    const size_t total = table_bytes + xchg_bytes + 256;
+    RWKV_CHECK_HIP(hipMalloc(&m->dev_block, total));
+    RWKV_CHECK_HIP(hipMemset(m->dev_block, 0, total));
+    std::vector<DLayer> tab(L);
+    for (size_t l = 0; l < L; ++l) {
+        const rwkv_layer_desc &ld = m->layers[l];
+        DLayer &t = tab[l];
+        t.att_k = to_dq(ld.att_k); t.att_v = to_dq(ld.att_v); t.att_r = to_dq(ld.att_r); t.att_o = to_dq(ld.att_o);
+        t.ffn_k = to_dq(ld.ffn_k); t.ffn_r = to_dq(ld.ffn_r); t.ffn_v = to_dq(ld.ffn_v);
+        t.ln1_w = ld.ln1_w; t.ln1_b = ld.ln1_b; t.ln2_w = ld.ln2_w; t.ln2_b = ld.ln2_b;
+        t.att_mix = ld.att_mix; t.ffn_mix = ld.ffn_mix; t.time_decay = ld.time_decay; t.time_first = ld.time_first;
+    }
+    RWKV_CHECK_HIP(hipMemcpy(m->dev_block, tab.data(), L * sizeof(DLayer), hipMemcpyHostToDevice));
+    unsigned char *base = static_cast<unsigned char *>(m->dev_block);
+    m->dm.L = (int)L; m->dm.C = (int)C; m->dm.F = (int)F; m->dm.V = (int)d.n_vocab;
+    m->dm.emb = d.emb; m->dm.ln0_w = d.ln0_w; m->dm.ln0_b = d.ln0_b;
+    m->dm.lnout_w = d.ln_out_w; m->dm.lnout_b = d.ln_out_b; m->dm.head = to_dq(d.head);
+    m->dm.layers = reinterpret_cast<const DLayer *>(base);
+    u64 *x = reinterpret_cast<u64 *>(base + table_bytes);
+    m->db.X = x; m->db.A = x + C; m->db.H = x + 2 * C;
+    m->db.abort_flag = reinterpret_cast<unsigned *>(base + table_bytes + xchg_bytes);
+    m->epoch = 0;
+    m->fused = true;
+    return RWKV_OK;
+}
+
+// One token through the persistent kernel (argument checks done by the caller).
+int fused_token(rwkv_model *m, hipStream_t st, const int64_t *token, double *state, double *logits) {
+    const int rc = decode_launch(st, m->dm, m->db, m->epoch, token, state, logits);
+    m->epoch += decode_epochs_per_token(m->d.n_layer);
+    return rc;
+}
+
 }  // namespace
 
 extern "C" {
@@ -478,11 +535,30 @@ int rwkv_model_create(const rwkv_model_desc *desc, rwkv_model **out) {
     m->d = *desc;
     m->layers.assign(desc->layers, desc->layers + L);
     m->d.layers = m->layers.data();
+    m->device = dev;
+    rc = setup_fused(m);
+    if (rc) { delete m; return rc; }
     *out = m;
     return RWKV_OK;
 }
 
-void rwkv_model_destroy(rwkv_model *m) { delete m; }
+void rwkv_model_destroy(rwkv_model *m) {
+    if (!m) return;
+    if (m->dev_block) (void)hipFree(m->dev_block);
+    delete m;
+}
+
+int rwkv_model_has_fused_step(const rwkv_model *m) { return (m && m->fused) ? 1 : 0; }
+
+int rwkv_model_check(rwkv_model *m) {
+    RWKV_CHECK_ARG(m, "rwkv_model_check: null handle");
+    RWKV_CHECK_HIP(hipDeviceSynchronize());
+    if (!m->fused) return RWKV_OK;
+    unsigned flag = 0;
+    RWKV_CHECK_HIP(hipMemcpy(&flag, m->db.abort_flag, sizeof(flag), hipMemcpyDeviceToHost));
+    if (flag) return set_error(RWKV_ERR_HIP, "a single-token launch gave up waiting for another workgroup");
+    return RWKV_OK;
+}
 
 size_t rwkv_model_workspace_bytes(const rwkv_model *m, int64_t max_tokens) {
     if (!m || max_tokens <= 0) return 0;
@@ -495,7 +571,8 @@ int rwkv_model_forward(rwkv_model *m, rwkv_stream_t stream, const int64_t *token
     if (rc) return rc;
     const Workspace w = carve(workspace, m->d.n_embd, m->d.n_ffn);
     for (int64_t t = 0; t < T; ++t) {
-        rc = step_token(m, (hipStream_t)stream, tokens + t, state, logits, w, t == T - 1);
+        if (m->fused) rc = fused_token(m, (hipStream_t)stream, tokens + t, state, logits);
+        else rc = step_token(m, (hipStream_t)stream, tokens + t, state, logits, w, t == T - 1);
         if (rc) return rc;
     }
     return RWKV_OK;
@@ -508,7 +585,8 @@ int rwkv_model_decode_greedy(rwkv_model *m, rwkv_stream_t stream, int64_t *token
     RWKV_CHECK_ARG(n > 0, "rwkv_model_decode_greedy: n must be positive");
     const Workspace w = carve(workspace, m->d.n_embd, m->d.n_ffn);
     for (int64_t i = 0; i < n; ++i) {
-        rc = step_token(m, (hipStream_t)stream, tokens + i, state, logits, w, true);
+        if (m->fused) rc = fused_token(m, (hipStream_t)stream, tokens + i, state, logits);
+        else rc = step_token(m, (hipStream_t)stream, tokens + i, state, logits, w, true);
         if (rc) return rc;
         rc = rwkv_argmax_f64(stream, logits, m->d.n_vocab, tokens + i + 1);
         if (rc) return rc;

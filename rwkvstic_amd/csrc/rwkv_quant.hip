@@ -138,6 +138,53 @@ dequant_packed_kernel(const uint8_t *__restrict__ packed, const float *__restric
     dq[g] = (float)((double)code * (double)range[j] + offset[j]);
 }
 
+// ---------------------------------------------------------------------------
+// "M16" layout for the int8 matrix-core decode kernel: 1 KiB blocks of 16
+// output columns x 64 input rows, ordered [ceil(n_out/16)][ceil(n_in/64)].
+// Lane l = 16*g + n of a wavefront owns bytes 16*l .. 16*l+15 of the block:
+// rows 64*kb + 16*g + (0..15) of column 16*ct + n, stored as code - 128
+// (two's complement), i.e. exactly the B operand of v_mfma_i32_16x16x64_i8.
+// Padding is stored as 0 (it only ever meets zero activation digits).
+// ---------------------------------------------------------------------------
+template <bool PACK>
+__global__ void __launch_bounds__(256)
+pack_m16_kernel(uint8_t *__restrict__ codes, int64_t stride, int64_t n_in, int64_t n_out,
+                uint8_t *__restrict__ packed, int64_t n_kb, int64_t n_chunks) {
+    const int64_t gidx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gidx >= n_chunks) return;
+    const int lane = (int)(gidx & 63);
+    const int64_t blk = gidx >> 6;
+    const int64_t kb = blk % n_kb, ct = blk / n_kb;
+    const int g = lane >> 4, n = lane & 15;
+    const int64_t col = ct * 16 + n;
+    uint8_t *p = packed + gidx * 16;
+    if (PACK) {
+        uint32_t d[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            uint32_t v = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int64_t row = kb * 64 + 16 * g + 4 * q + e;
+                const uint32_t b = (row < n_in && col < n_out) ? (uint32_t)(codes[row * stride + col] ^ 0x80u) : 0u;
+                v |= b << (8 * e);
+            }
+            d[q] = v;
+        }
+        *reinterpret_cast<uint4 *>(p) = make_uint4(d[0], d[1], d[2], d[3]);
+    } else {
+        const uint4 v = *reinterpret_cast<const uint4 *>(p);
+        const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int64_t row = kb * 64 + 16 * g + 4 * q + e;
+                if (row < n_in && col < n_out) codes[row * stride + col] = (uint8_t)((d[q] >> (8 * e)) ^ 0x80u);
+            }
+    }
+}
+
 }  // namespace rwkv
 
 using namespace rwkv;
@@ -202,6 +249,39 @@ int rwkv_dequant_packed(rwkv_stream_t stream, const uint8_t *packed, const float
                        (hipStream_t)stream, packed, range, offset, n_in, n_out,
                        ceil_div(n_in, kBlockRows), dq);
     RWKV_CHECK_LAUNCH("dequant_packed_kernel");
+    return RWKV_OK;
+}
+
+size_t rwkv_packed_m16_bytes(int64_t n_in, int64_t n_out) {
+    if (n_in <= 0 || n_out <= 0) return 0;
+    return (size_t)(ceil_div(n_out, 16) * ceil_div(n_in, 64) * 1024);
+}
+
+int rwkv_pack_m16(rwkv_stream_t stream, const uint8_t *codes, int64_t codes_stride,
+                  int64_t n_in, int64_t n_out, uint8_t *packed) {
+    RWKV_CHECK_ARG(codes && packed, "rwkv_pack_m16: null pointer");
+    RWKV_CHECK_ARG(n_in > 0 && n_out > 0 && codes_stride >= n_out, "rwkv_pack_m16: bad sizes");
+    RWKV_CHECK_ALIGN(packed, 16);
+    const int64_t n_kb = ceil_div(n_in, 64);
+    const int64_t n_chunks = ceil_div(n_out, 16) * n_kb * 64;
+    hipLaunchKernelGGL(pack_m16_kernel<true>, dim3((unsigned)ceil_div(n_chunks, 256)), dim3(256), 0,
+                       (hipStream_t)stream, const_cast<uint8_t *>(codes), codes_stride, n_in, n_out,
+                       packed, n_kb, n_chunks);
+    RWKV_CHECK_LAUNCH("pack_m16_kernel");
+    return RWKV_OK;
+}
+
+int rwkv_unpack_m16(rwkv_stream_t stream, const uint8_t *packed, int64_t n_in, int64_t n_out,
+                    uint8_t *codes, int64_t codes_stride) {
+    RWKV_CHECK_ARG(codes && packed, "rwkv_unpack_m16: null pointer");
+    RWKV_CHECK_ARG(n_in > 0 && n_out > 0 && codes_stride >= n_out, "rwkv_unpack_m16: bad sizes");
+    RWKV_CHECK_ALIGN(packed, 16);
+    const int64_t n_kb = ceil_div(n_in, 64);
+    const int64_t n_chunks = ceil_div(n_out, 16) * n_kb * 64;
+    hipLaunchKernelGGL(pack_m16_kernel<false>, dim3((unsigned)ceil_div(n_chunks, 256)), dim3(256), 0,
+                       (hipStream_t)stream, codes, codes_stride, n_in, n_out,
+                       const_cast<uint8_t *>(packed), n_kb, n_chunks);
+    RWKV_CHECK_LAUNCH("unpack_m16_kernel");
     return RWKV_OK;
 }
 

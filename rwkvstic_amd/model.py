@@ -21,17 +21,18 @@ from . import ops
 class QuantMatrix:
     """Device-resident quantised matrix: packed codes + per-input-channel range/offset."""
 
-    def __init__(self, packed: torch.Tensor, rng: torch.Tensor, off: torch.Tensor, n_in: int, n_out: int):
+    def __init__(self, packed: torch.Tensor, rng: torch.Tensor, off: torch.Tensor, n_in: int, n_out: int,
+                 packed16: Optional[torch.Tensor] = None):
         self.packed, self.range, self.offset, self.n_in, self.n_out = packed, rng, off, n_in, n_out
+        self.packed16 = packed16
 
     @classmethod
-    def from_weight(cls, weight: torch.Tensor, device) -> "QuantMatrix":
+    def from_weight(cls, weight: torch.Tensor, device, m16: bool = True) -> "QuantMatrix":
         """``weight[out, in]`` in any float dtype, on any device."""
         w = weight.to(device=device, dtype=torch.float32).contiguous()
         codes, rng, off = ops.quantize(w)
         n_in, n_out = codes.shape
-        packed = ops.pack(codes)
-        return cls(packed, rng, off, n_in, n_out)
+        return cls(ops.pack(codes), rng, off, n_in, n_out, ops.pack_m16(codes) if m16 else None)
 
     @classmethod
     def from_codes(cls, codes: torch.Tensor, rng: torch.Tensor, off: torch.Tensor, device) -> "QuantMatrix":
@@ -39,13 +40,14 @@ class QuantMatrix:
         codes = codes.to(device)
         n_in, n_out = codes.shape
         return cls(ops.pack(codes), rng.to(device=device, dtype=torch.float32).contiguous(),
-                   off.to(device=device, dtype=torch.float64).contiguous(), n_in, n_out)
+                   off.to(device=device, dtype=torch.float64).contiguous(), n_in, n_out, ops.pack_m16(codes))
 
     def codes(self) -> torch.Tensor:
         return ops.unpack(self.packed, self.n_in, self.n_out)
 
     def desc(self) -> N.QMat:
-        return N.QMat(self.packed.data_ptr(), self.range.data_ptr(), self.offset.data_ptr(), self.n_in, self.n_out)
+        return N.QMat(self.packed.data_ptr(), self.packed16.data_ptr() if self.packed16 is not None else None,
+                      self.range.data_ptr(), self.offset.data_ptr(), self.n_in, self.n_out)
 
     def nbytes(self) -> int:
         return self.n_in * self.n_out
@@ -53,7 +55,9 @@ class QuantMatrix:
 
 class HipRWKV:
     def __init__(self, weights: Union[Dict[str, torch.Tensor], Iterable[Tuple[str, torch.Tensor]]],
-                 device: str = "cuda"):
+                 device: str = "cuda", fused: bool = True):
+        """``fused=False`` skips the second weight layout, so single-token steps run as one launch per
+        phase (the path every shape supports) instead of the persistent kernel."""
         if not torch.cuda.is_available():
             raise RuntimeError("HipRWKV needs a ROCm GPU (gfx950); there is no CPU path in this backend")
         N.lib()
@@ -67,7 +71,7 @@ class HipRWKV:
             if key == "emb.weight":
                 self.emb = t.to(device=self.device, dtype=torch.float32).contiguous()
             elif key.endswith(".weight") and t.dim() == 2:
-                mats[key] = QuantMatrix.from_weight(t, self.device)
+                mats[key] = QuantMatrix.from_weight(t, self.device, m16=fused)
             else:
                 vec[key] = t
         if self.emb is None:
@@ -128,6 +132,7 @@ class HipRWKV:
         with torch.cuda.device(self.device):
             N.check(L.rwkv_model_create(C.byref(desc), C.byref(handle)))
         self._handle = handle
+        self.fused_step = bool(L.rwkv_model_has_fused_step(handle))
         self._ws: Optional[torch.Tensor] = None
         self._ws_tokens = 0
 
@@ -146,6 +151,10 @@ class HipRWKV:
             self._ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
             self._ws_tokens = T
         return self._ws
+
+    def check(self) -> None:
+        """Synchronise and raise if a single-token launch gave up waiting (diagnostics)."""
+        N.check(N.lib().rwkv_model_check(self._handle))
 
     def weight_bytes(self) -> int:
         """uint8 weight bytes streamed per decoded token: L*13*C^2 + V*C."""

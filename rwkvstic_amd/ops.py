@@ -149,6 +149,28 @@ def unpack(packed: torch.Tensor, n_in: int, n_out: int) -> torch.Tensor:
     return codes
 
 
+def pack_m16(codes: torch.Tensor) -> torch.Tensor:
+    """Reference layout ``codes[in, out]`` -> 16x64 signed blocks for the matrix-core decode kernel."""
+    _req(codes, torch.uint8, "codes")
+    if codes.dim() != 2 or codes.stride(1) != 1:
+        raise ValueError("codes must be 2-D with unit inner stride")
+    n_in, n_out = codes.shape
+    L = N.lib()
+    packed = torch.empty(L.rwkv_packed_m16_bytes(n_in, n_out), dtype=torch.uint8, device=codes.device)
+    N.check(L.rwkv_pack_m16(_stream(), codes.data_ptr(), codes.stride(0), n_in, n_out, packed.data_ptr()))
+    return packed
+
+
+def unpack_m16(packed: torch.Tensor, n_in: int, n_out: int) -> torch.Tensor:
+    _req(packed, torch.uint8, "packed"); _contig(packed, "packed")
+    L = N.lib()
+    if packed.numel() < L.rwkv_packed_m16_bytes(n_in, n_out):
+        raise ValueError("packed buffer too small")
+    codes = torch.empty((n_in, n_out), dtype=torch.uint8, device=packed.device)
+    N.check(L.rwkv_unpack_m16(_stream(), packed.data_ptr(), n_in, n_out, codes.data_ptr(), n_out))
+    return codes
+
+
 def dequant_packed(packed, rng, off, n_in: int, n_out: int) -> torch.Tensor:
     _req(packed, torch.uint8, "packed"); _req(rng, torch.float32, "range"); _req(off, torch.float64, "offset")
     L = N.lib()

@@ -236,3 +236,17 @@ def test_argmax_first_maximum(ops):
     x = torch.randn(50277, dtype=torch.float64)
     x[40000] = 9.0; x[123] = 9.0
     assert int(ops.argmax(x.cuda())) == 123
+
+
+def test_pack_m16_round_trip(ops):
+    for n_in, n_out in [(64, 16), (130, 77), (2560, 2560)]:
+        c = torch.randint(0, 256, (n_in, n_out), dtype=torch.uint8, device="cuda")
+        p = ops.pack_m16(c)
+        assert torch.equal(ops.unpack_m16(p, n_in, n_out), c)
+    # block 0, lane 16*g + n, byte i  <->  codes[16*g + i][n] - 128
+    c = torch.arange(64 * 16, dtype=torch.int64).reshape(64, 16).remainder(256).to(torch.uint8).cuda()
+    p = ops.pack_m16(c).cpu().reshape(64, 16)
+    for lane in (0, 5, 17, 63):
+        g, n = divmod(lane, 16)
+        want = (c[16 * g:16 * g + 16, n].cpu().to(torch.int16) - 128).to(torch.int8)
+        assert torch.equal(p[lane].view(torch.int8), want)
