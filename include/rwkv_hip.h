@@ -227,6 +227,28 @@ int rwkv_model_forward(rwkv_model *m, rwkv_stream_t stream,
                        double *state, double *logits,
                        void *workspace, size_t workspace_bytes);
 
+/* Prompt / batch GEMM on the matrix cores: y[T, n_out] = x[T, n_in] x quantised
+ * matrix, the T > 1 branch of MM8.forward (matmul.py:56-57; the reference
+ * rounds to bfloat16 there, this routine keeps the single-token arithmetic:
+ * fp32(x * range) as exact 32-bit fixed point per row, integer dot products,
+ * zero-point term in float64).  x, y float64 row-major; packed16 from
+ * rwkv_pack_m16; n_in a multiple of 64. */
+size_t rwkv_gemm8_workspace_bytes(int64_t T, int64_t n_in, int64_t n_out);
+int rwkv_gemm8(rwkv_stream_t stream, int64_t T, int64_t n_in, int64_t n_out,
+               const double *x, const uint8_t *packed16, const float *range,
+               const double *offset, double *y,
+               void *workspace, size_t workspace_bytes);
+
+/* One token for each of `batch` independent sequences (the reference has no
+ * batched entry point on this path: it would call myRWKV.forward, opt.py:61-76,
+ * once per sequence).  tokens[batch]; states[batch][n_layer][5][n_embd] updated
+ * in place; logits[batch][n_vocab].  Needs the M16 layout of every matrix. */
+size_t rwkv_model_batch_workspace_bytes(const rwkv_model *m, int64_t batch);
+int rwkv_model_forward_batch(rwkv_model *m, rwkv_stream_t stream,
+                             const int64_t *tokens, int64_t batch,
+                             double *states, double *logits,
+                             void *workspace, size_t workspace_bytes);
+
 /* Greedy decode entirely on the device: for i < n:
  *   logits, state = forward(tokens[i], state); tokens[i+1] = argmax(logits).
  * tokens: int64 [n + 1] on the device, tokens[0] is the input token.  This is

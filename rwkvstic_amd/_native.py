@@ -21,6 +21,8 @@ EXPORTS = (
     "rwkv_model_create", "rwkv_model_destroy", "rwkv_model_workspace_bytes",
     "rwkv_model_has_fused_step", "rwkv_model_check",
     "rwkv_model_forward", "rwkv_model_decode_greedy", "rwkv_argmax_f64",
+    "rwkv_gemm8_workspace_bytes", "rwkv_gemm8",
+    "rwkv_model_batch_workspace_bytes", "rwkv_model_forward_batch",
 )
 
 
@@ -94,6 +96,12 @@ def lib() -> C.CDLL:
     L.rwkv_model_forward.argtypes = [vp, vp, vp, i64, vp, vp, vp, sz]
     L.rwkv_model_decode_greedy.argtypes = [vp, vp, vp, i64, vp, vp, vp, sz]
     L.rwkv_argmax_f64.argtypes = [vp, vp, i64, vp]
+    L.rwkv_gemm8_workspace_bytes.restype = sz
+    L.rwkv_gemm8_workspace_bytes.argtypes = [i64, i64, i64]
+    L.rwkv_gemm8.argtypes = [vp, i64, i64, i64, vp, vp, vp, vp, vp, vp, sz]
+    L.rwkv_model_batch_workspace_bytes.restype = sz
+    L.rwkv_model_batch_workspace_bytes.argtypes = [vp, i64]
+    L.rwkv_model_forward_batch.argtypes = [vp, vp, vp, i64, vp, vp, vp, sz]
     for name in EXPORTS:
         getattr(L, name)          # AttributeError here means header and library disagree
     _lib = L

@@ -25,6 +25,7 @@
 // max-shifted form.
 #include "rwkv_common.h"
 #include "rwkv_decode.h"
+#include "rwkv_rows.h"
 
 #include <new>
 #include <string>
@@ -488,6 +489,111 @@ int setup_fused(rwkv_model *m) {
     return RWKV_OK;
 }
 
+// ---- many-row path (prompts and batches) -----------------------------------
+constexpr int64_t kRowsChunk = 1024;   // rows per pass: bounds the workspace of long prompts
+constexpr int64_t kRowsMin = 4;        // shorter prompts go token by token
+
+struct RowsWs {
+    double *x, *mix, *kvr, *att, *h, *prev0;
+    RowsScratch s;
+};
+
+// n_wide = widest product output (n_ffn, or the vocabulary when every row needs logits)
+size_t rows_ws_bytes(int64_t R, int64_t C, int64_t F, int64_t n_wide) {
+    size_t n = 0;
+    n += round_up((size_t)R * C * 8, 256) * 8;          // x, mix[3], kvr[3], att
+    n += round_up((size_t)R * F * 8, 256);              // h
+    n += round_up((size_t)C * 8, 256);                  // prev0
+    n += round_up((size_t)R * 8, 256) * 3;              // S, qs, zp
+    n += round_up(rows_dig_bytes(R, F), 256);
+    n += round_up(rows_tot_bytes(R, n_wide), 256);
+    return n;
+}
+
+RowsWs rows_carve(void *ws, int64_t R, int64_t C, int64_t F, int64_t n_wide) {
+    unsigned char *p = static_cast<unsigned char *>(ws);
+    auto take = [&](size_t bytes) { void *q = p; p += round_up(bytes, 256); return q; };
+    RowsWs w;
+    w.x = (double *)take((size_t)R * C * 8);
+    w.mix = (double *)take((size_t)R * C * 8 * 3);
+    w.kvr = (double *)take((size_t)R * C * 8 * 3);
+    w.att = (double *)take((size_t)R * C * 8);
+    w.h = (double *)take((size_t)R * F * 8);
+    w.prev0 = (double *)take((size_t)C * 8);
+    w.s.S = (double *)take((size_t)R * 8);
+    w.s.qs = (double *)take((size_t)R * 8);
+    w.s.zp = (double *)take((size_t)R * 8);
+    w.s.dig = (signed char *)take(rows_dig_bytes(R, F));
+    w.s.tot = (long long *)take(rows_tot_bytes(R, n_wide));
+    (void)n_wide;
+    return w;
+}
+
+bool rows_supported(const rwkv_model *m) {
+    const rwkv_model_desc &d = m->d;
+    if (d.n_embd % 64 || d.n_ffn % 64 || !d.head.packed16) return false;
+    for (const rwkv_layer_desc &ld : m->layers)
+        if (!(ld.att_k.packed16 && ld.att_v.packed16 && ld.att_r.packed16 && ld.att_o.packed16 &&
+              ld.ffn_k.packed16 && ld.ffn_r.packed16 && ld.ffn_v.packed16))
+            return false;
+    return true;
+}
+
+#define RWKV_TRY(expr) do { const int rc_ = (expr); if (rc_) return rc_; } while (0)
+
+// R rows through every layer.  sequence: rows are consecutive tokens of one sequence whose state is
+// `state` [L,5,C]; otherwise row b is one token of sequence b with state at state + b * state_stride.
+int rows_layers(rwkv_model *m, hipStream_t st, const int64_t *tokens, int64_t R, bool sequence, double *state,
+                int64_t state_stride, const RowsWs &w) {
+    const rwkv_model_desc &d = m->d;
+    const int C = (int)d.n_embd, F = (int)d.n_ffn, V = (int)d.n_vocab;
+    const size_t RC = (size_t)R * C;
+    RWKV_TRY(rows_embed(st, tokens, R, V, C, d.emb, d.ln0_w, d.ln0_b, w.x));
+    for (int64_t l = 0; l < d.n_layer; ++l) {
+        const rwkv_layer_desc &L = m->layers[l];
+        double *sl = state + (size_t)l * 5 * C;
+        // TimeMix (block.py:58-80)
+        if (sequence) RWKV_CHECK_HIP(hipMemcpyAsync(w.prev0, sl, (size_t)C * 8, hipMemcpyDeviceToDevice, st));
+        RWKV_TRY(rows_ln_mix(st, 3, R, C, sequence, w.x, L.ln1_w, L.ln1_b, L.att_mix, sequence ? w.prev0 : sl, sl,
+                             state_stride, w.mix));
+        const rwkv_qmat *kvr[3] = {&L.att_k, &L.att_v, &L.att_r};
+        for (int i = 0; i < 3; ++i)
+            RWKV_TRY(rows_matmul(st, w.s, R, C, C, w.mix + i * RC, kvr[i]->packed16, kvr[i]->range, kvr[i]->offset,
+                                 ROW_STORE, w.kvr + i * RC, nullptr));
+        RWKV_TRY(rows_wkv(st, R, C, sequence, w.kvr, w.kvr + RC, w.kvr + 2 * RC, L.time_decay, L.time_first,
+                          sl + 2 * (size_t)C, state_stride, w.att));
+        RWKV_TRY(rows_matmul(st, w.s, R, C, C, w.att, L.att_o.packed16, L.att_o.range, L.att_o.offset, ROW_ADD, w.x,
+                             nullptr));
+        // ChannelMix (block.py:82-100)
+        if (sequence) RWKV_CHECK_HIP(hipMemcpyAsync(w.prev0, sl + C, (size_t)C * 8, hipMemcpyDeviceToDevice, st));
+        RWKV_TRY(rows_ln_mix(st, 2, R, C, sequence, w.x, L.ln2_w, L.ln2_b, L.ffn_mix, sequence ? w.prev0 : sl + C,
+                             sl + C, state_stride, w.mix));
+        RWKV_TRY(rows_matmul(st, w.s, R, C, F, w.mix, L.ffn_k.packed16, L.ffn_k.range, L.ffn_k.offset, ROW_RELU2, w.h,
+                             nullptr));
+        RWKV_TRY(rows_matmul(st, w.s, R, C, C, w.mix + RC, L.ffn_r.packed16, L.ffn_r.range, L.ffn_r.offset, ROW_STORE,
+                             w.kvr, nullptr));
+        RWKV_TRY(rows_matmul(st, w.s, R, F, C, w.h, L.ffn_v.packed16, L.ffn_v.range, L.ffn_v.offset, ROW_GATE_ADD, w.x,
+                             w.kvr));
+    }
+    return RWKV_OK;
+}
+
+// logits[V] of one residual row through ln_out and the head (opt.py:72-74)
+int head_logits(rwkv_model *m, hipStream_t st, const double *xrow, double *logits) {
+    const rwkv_model_desc &d = m->d;
+    const int C = (int)d.n_embd, V = (int)d.n_vocab;
+    const int c_kb = (int)ceil_div(C, kBlockRows);
+    const size_t red_bytes = 3 * kWaves * 8 + 3 * kWaves * 8 * 4;
+    LnMatArgs h;
+    h.C = C; h.mode = EPI_LOGITS; h.x = const_cast<double *>(xrow); h.ln_w = d.ln_out_w; h.ln_b = d.ln_out_b;
+    h.mix = nullptr; h.shift = nullptr; h.k = to_dev(d.head); h.r = h.k; h.out_k = logits; h.out_r = nullptr;
+    h.ln_tmp = nullptr;
+    hipLaunchKernelGGL(ln_matvec_kernel, dim3((unsigned)ceil_div(V, kTileCols)), dim3(kThreads),
+                       (size_t)c_kb * kBlockRows * 4 + red_bytes, st, h);
+    RWKV_CHECK_LAUNCH("head");
+    return RWKV_OK;
+}
+
 // One token through the persistent kernel (argument checks done by the caller).
 int fused_token(rwkv_model *m, hipStream_t st, const int64_t *token, double *state, double *logits) {
     const int rc = decode_launch(st, m->dm, m->db, m->epoch, token, state, logits);
@@ -562,7 +668,18 @@ int rwkv_model_check(rwkv_model *m) {
 
 size_t rwkv_model_workspace_bytes(const rwkv_model *m, int64_t max_tokens) {
     if (!m || max_tokens <= 0) return 0;
-    return round_up(ws_doubles(m->d.n_embd, m->d.n_ffn) * sizeof(double), 256);
+    size_t n = round_up(ws_doubles(m->d.n_embd, m->d.n_ffn) * sizeof(double), 256);
+    if (max_tokens >= kRowsMin && rows_supported(m)) {
+        const int64_t R = max_tokens < kRowsChunk ? max_tokens : kRowsChunk;
+        n += rows_ws_bytes(R, m->d.n_embd, m->d.n_ffn, m->d.n_ffn);
+    }
+    return n;
+}
+
+size_t rwkv_model_batch_workspace_bytes(const rwkv_model *m, int64_t batch) {
+    if (!m || batch <= 0 || !rows_supported(m)) return 0;
+    const int64_t wide = m->d.n_ffn > m->d.n_vocab ? m->d.n_ffn : m->d.n_vocab;
+    return rows_ws_bytes(batch, m->d.n_embd, m->d.n_ffn, wide);
 }
 
 int rwkv_model_forward(rwkv_model *m, rwkv_stream_t stream, const int64_t *tokens, int64_t T, double *state,
@@ -570,12 +687,87 @@ int rwkv_model_forward(rwkv_model *m, rwkv_stream_t stream, const int64_t *token
     int rc = check_forward_args(m, tokens, state, logits, workspace, workspace_bytes, T, "rwkv_model_forward");
     if (rc) return rc;
     const Workspace w = carve(workspace, m->d.n_embd, m->d.n_ffn);
+    if (T >= kRowsMin && rows_supported(m)) {
+        // prompt: GEMM path in chunks of kRowsChunk rows, logits from the last row only
+        const hipStream_t st = (hipStream_t)stream;
+        const int64_t C = m->d.n_embd, F = m->d.n_ffn;
+        unsigned char *rows_base = static_cast<unsigned char *>(workspace) +
+                                   round_up(ws_doubles(C, F) * sizeof(double), 256);
+        const int64_t Rmax = T < kRowsChunk ? T : kRowsChunk;
+        const RowsWs rw = rows_carve(rows_base, Rmax, C, F, F);
+        for (int64_t t0 = 0; t0 < T; t0 += kRowsChunk) {
+            const int64_t R = T - t0 < kRowsChunk ? T - t0 : kRowsChunk;
+            rc = rows_layers(m, st, tokens + t0, R, true, state, 0, rw);
+            if (rc) return rc;
+            if (t0 + R == T) rc = head_logits(m, st, rw.x + (size_t)(R - 1) * C, logits);
+            if (rc) return rc;
+        }
+        return RWKV_OK;
+    }
     for (int64_t t = 0; t < T; ++t) {
         if (m->fused) rc = fused_token(m, (hipStream_t)stream, tokens + t, state, logits);
         else rc = step_token(m, (hipStream_t)stream, tokens + t, state, logits, w, t == T - 1);
         if (rc) return rc;
     }
     return RWKV_OK;
+}
+
+int rwkv_model_forward_batch(rwkv_model *m, rwkv_stream_t stream, const int64_t *tokens, int64_t batch,
+                             double *states, double *logits, void *workspace, size_t workspace_bytes) {
+    if (!m || !tokens || !states || !logits || !workspace)
+        return set_error(RWKV_ERR_ARG, "rwkv_model_forward_batch: null pointer");
+    if (batch <= 0) return set_error(RWKV_ERR_ARG, "rwkv_model_forward_batch: batch must be positive");
+    if (!rows_supported(m))
+        return set_error(RWKV_ERR_SIZE, "rwkv_model_forward_batch: needs the M16 layout of every matrix and "
+                                        "n_embd, n_ffn multiples of 64");
+    if (reinterpret_cast<uintptr_t>(tokens) % 8 || reinterpret_cast<uintptr_t>(states) % 8 ||
+        reinterpret_cast<uintptr_t>(logits) % 8 || reinterpret_cast<uintptr_t>(workspace) % 16)
+        return set_error(RWKV_ERR_ALIGN, "rwkv_model_forward_batch: tokens/states/logits need 8-byte, workspace "
+                                         "16-byte alignment");
+    const size_t need = rwkv_model_batch_workspace_bytes(m, batch);
+    if (workspace_bytes < need)
+        return set_error(RWKV_ERR_WORKSPACE, "rwkv_model_forward_batch: workspace of %zu bytes needed, %zu given",
+                         need, workspace_bytes);
+    const hipStream_t st = (hipStream_t)stream;
+    const rwkv_model_desc &d = m->d;
+    const int64_t C = d.n_embd, F = d.n_ffn, V = d.n_vocab;
+    const RowsWs rw = rows_carve(workspace, batch, C, F, F > V ? F : V);
+    int rc = rows_layers(m, st, tokens, batch, false, states, d.n_layer * 5 * C, rw);
+    if (rc) return rc;
+    rc = rows_ln_mix(st, 0, batch, (int)C, false, rw.x, d.ln_out_w, d.ln_out_b, nullptr, nullptr, nullptr, 0, rw.mix);
+    if (rc) return rc;
+    return rows_matmul(st, rw.s, batch, C, V, rw.mix, d.head.packed16, d.head.range, d.head.offset, ROW_STORE, logits,
+                       nullptr);
+}
+
+int rwkv_gemm8(rwkv_stream_t stream, int64_t T, int64_t n_in, int64_t n_out, const double *x,
+               const uint8_t *packed16, const float *range, const double *offset, double *y,
+               void *workspace, size_t workspace_bytes) {
+    RWKV_CHECK_ARG(x && packed16 && range && offset && y && workspace, "rwkv_gemm8: null pointer");
+    RWKV_CHECK_ARG(T > 0 && n_in > 0 && n_out > 0, "rwkv_gemm8: sizes must be positive");
+    if (n_in % 64) return set_error(RWKV_ERR_SIZE, "rwkv_gemm8: n_in must be a multiple of 64");
+    RWKV_CHECK_ALIGN(packed16, 16);
+    RWKV_CHECK_ALIGN(workspace, 16);
+    RWKV_CHECK_ALIGN(x, 8);
+    RWKV_CHECK_ALIGN(y, 8);
+    const size_t need = rwkv_gemm8_workspace_bytes(T, n_in, n_out);
+    if (workspace_bytes < need)
+        return set_error(RWKV_ERR_WORKSPACE, "rwkv_gemm8: workspace of %zu bytes needed, %zu given", need,
+                         workspace_bytes);
+    unsigned char *p = static_cast<unsigned char *>(workspace);
+    RowsScratch s;
+    s.S = (double *)p; p += round_up((size_t)T * 8, 256);
+    s.qs = (double *)p; p += round_up((size_t)T * 8, 256);
+    s.zp = (double *)p; p += round_up((size_t)T * 8, 256);
+    s.dig = (signed char *)p; p += round_up(rows_dig_bytes(T, n_in), 256);
+    s.tot = (long long *)p;
+    return rows_matmul((hipStream_t)stream, s, T, n_in, n_out, x, packed16, range, offset, ROW_STORE, y, nullptr);
+}
+
+size_t rwkv_gemm8_workspace_bytes(int64_t T, int64_t n_in, int64_t n_out) {
+    if (T <= 0 || n_in <= 0 || n_out <= 0) return 0;
+    return round_up((size_t)T * 8, 256) * 3 + round_up(rows_dig_bytes(T, n_in), 256) +
+           round_up(rows_tot_bytes(T, n_out), 256);
 }
 
 int rwkv_model_decode_greedy(rwkv_model *m, rwkv_stream_t stream, int64_t *tokens, int64_t n, double *state,

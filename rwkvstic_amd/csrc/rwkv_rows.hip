@@ -1,0 +1,445 @@
+// Many-row path of the FASTQUANT RWKV-4 forward pass: a prompt (T tokens of one
+// sequence; reference agnostic/backends/opt.py:61-76 with T > 1,
+// modules/matmul.py:56-57,86-94) or a batch (B independent sequences, one token
+// each).  Rows are tokens; every matrix product is a GEMM on the matrix cores.
+//
+// Arithmetic.  Exactly the single-token kernel's: each row of
+// xs = fp32(x * range) is rewritten as 32-bit fixed point q = round(xs / S),
+// S a power of two chosen per row so that |q| <= 2^30, and split into four
+// signed base-256 digits.  The digit rows (4 per token) are the A operand and
+// the weights, stored as code - 128 in 1 KiB blocks of 16 columns x 64 rows
+// ("M16"), the B operand of v_mfma_i32_16x16x64_i8.  Integer sums are exact and
+// independent of tiling and of any split of the contraction, so a prompt
+// processed here gives the same products as the same tokens fed one at a time.
+// (The reference rounds this product to bfloat16, matmul.py:57; nothing here
+// is rounded below float32 class.)
+//
+// Digit rows are stored in fragment order: for M-tile mt (tokens 4mt..4mt+3) and
+// contraction block kb (rows 64kb..64kb+63) one 1 KiB fragment whose lane
+// 16g + m holds bytes k = 64kb + 16g + i (i < 16) of digit row m = 4*(t % 4) + d;
+// a wavefront loads a fragment with one coalesced 16-byte-per-lane request and
+// hands it to the matrix instruction unchanged.
+#include "rwkv_rows.h"
+
+namespace rwkv {
+
+namespace {
+
+constexpr int kRT = 256;           // threads of the row kernels
+constexpr int kRW = kRT / 64;
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ double wsum(double v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ float wmaxf(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// Sum of N values per thread over the workgroup (fixed order), broadcast.
+template <int N>
+__device__ __forceinline__ void rsum(double (&v)[N], double *red /*[N*kRW]*/) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        const double s = wsum(v[i]);
+        if (lane == 0) red[i * kRW + wave] = s;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        double s = 0.0;
+#pragma unroll
+        for (int w = 0; w < kRW; ++w) s += red[i * kRW + w];
+        v[i] = s;
+    }
+    __syncthreads();
+}
+
+// ---------------------------------------------------------------------------
+// x[t] = ln0(emb[token[t]])          (emb.py:9, opt.py:63-64)
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(kRT)
+rows_embed_kernel(const int64_t *__restrict__ tokens, int V, int C, const float *__restrict__ emb,
+                  const double *__restrict__ w, const double *__restrict__ b, double *__restrict__ x) {
+    __shared__ double red[2 * kRW];
+    const int t = blockIdx.x;
+    int64_t tok = tokens[t];
+    if (tok < 0) tok = 0;
+    if (tok >= V) tok = V - 1;
+    const float *e = emb + (size_t)tok * C;
+    double s[1] = {0.0};
+    for (int c = threadIdx.x; c < C; c += kRT) s[0] += (double)e[c];
+    rsum<1>(s, red);
+    const double mean = s[0] / (double)C;
+    double q[1] = {0.0};
+    for (int c = threadIdx.x; c < C; c += kRT) { const double d = (double)e[c] - mean; q[0] += d * d; }
+    rsum<1>(q, red);
+    const double sd = sqrt(q[0] / (double)C + 1e-5);
+    for (int c = threadIdx.x; c < C; c += kRT) x[(size_t)t * C + c] = w[c] * (((double)e[c] - mean) / sd) + b[c];
+}
+
+// ---------------------------------------------------------------------------
+// LayerNorm + token shift + time mix      (layernorm.py:15-20, block.py:58-67,82-91)
+//   xy = ln(x[t]);  prev = sequence ? (t == 0 ? prev0 : ln(x[t-1])) : prev0[t];
+//   mix_m[t] = xy * mu_m + prev * (1 - mu_m);  the newest xy becomes the shift state.
+// NM == 0: LayerNorm only, written to mix_0 (the head's ln_out).
+// ---------------------------------------------------------------------------
+struct LnMixArgs {
+    int C, R, sequence;
+    const double *x;            // [R, C]
+    const double *ln_w, *ln_b;  // [C]
+    const double *mu;           // [NM, C]
+    const double *prev0;        // sequence: [C]; batch: row t at prev0 + t * prev_stride
+    double *shift_dst;          // sequence: [C] (written by row R-1); batch: row t at shift_dst + t * prev_stride
+    int64_t prev_stride;
+    double *mix;                // [max(NM,1), R, C]
+};
+
+template <int NM>
+__global__ void __launch_bounds__(kRT) rows_ln_mix_kernel(const LnMixArgs a) {
+    __shared__ double red[4 * kRW];
+    const int t = blockIdx.x, C = a.C;
+    const bool need_prev = NM > 0 && a.sequence && t > 0;
+    const double *xr = a.x + (size_t)t * C;
+    const double *xp = need_prev ? xr - C : xr;
+    double s[2] = {0.0, 0.0};
+    for (int c = threadIdx.x; c < C; c += kRT) { s[0] += xr[c]; s[1] += xp[c]; }
+    rsum<2>(s, red);
+    const double mean = s[0] / (double)C, meanp = s[1] / (double)C;
+    double q[2] = {0.0, 0.0};
+    for (int c = threadIdx.x; c < C; c += kRT) {
+        const double d = xr[c] - mean, dp = xp[c] - meanp;
+        q[0] += d * d; q[1] += dp * dp;
+    }
+    rsum<2>(q, red);
+    const double sd = sqrt(q[0] / (double)C + 1e-5), sdp = sqrt(q[1] / (double)C + 1e-5);
+    const size_t RC = (size_t)a.R * C;
+    for (int c = threadIdx.x; c < C; c += kRT) {
+        const double w = a.ln_w[c], b = a.ln_b[c];
+        const double xy = w * ((xr[c] - mean) / sd) + b;
+        if (NM == 0) { a.mix[(size_t)t * C + c] = xy; continue; }
+        double prev;
+        if (need_prev) prev = w * ((xp[c] - meanp) / sdp) + b;
+        else prev = a.sequence ? a.prev0[c] : a.prev0[(size_t)t * a.prev_stride + c];
+#pragma unroll
+        for (int m = 0; m < NM; ++m) {
+            const double mu = a.mu[(size_t)m * C + c];
+            a.mix[m * RC + (size_t)t * C + c] = xy * mu + prev * (1.0 - mu);
+        }
+        if (!a.sequence) a.shift_dst[(size_t)t * a.prev_stride + c] = xy;
+        else if (t == a.R - 1) a.shift_dst[c] = xy;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Row quantiser: xs = fp32(v * range), S from the row's max |xs|, digits in
+// fragment order, zero-point term sum v * offset and sum q   (matmul.py:59-62,131-133).
+// ---------------------------------------------------------------------------
+struct QuantArgs {
+    int K;                      // contraction length, multiple of 64
+    const double *in;           // [R, K]
+    const float *range;         // [K]
+    const double *offset;       // [K]
+    signed char *dig;           // fragments [ceil(R/4)][K/64][1024]
+    double *S, *qs, *zp;        // [R]
+};
+
+__global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
+    __shared__ double red[2 * kRW];
+    __shared__ float redf[kRW];
+    const int t = blockIdx.x, K = a.K;
+    const double *row = a.in + (size_t)t * K;
+    float amax = 0.f;
+    double z[1] = {0.0};
+    for (int c = threadIdx.x; c < K; c += kRT) {
+        const double v = row[c];
+        amax = fmaxf(amax, fabsf((float)(v * (double)a.range[c])));
+        z[0] += v * a.offset[c];
+    }
+    amax = wmaxf(amax);
+    if ((threadIdx.x & 63) == 0) redf[threadIdx.x >> 6] = amax;
+    rsum<1>(z, red);                       // (its barriers also publish redf)
+    amax = redf[0];
+#pragma unroll
+    for (int w = 1; w < kRW; ++w) amax = fmaxf(amax, redf[w]);
+    double S = 0.0, invS = 0.0;
+    if (amax > 0.f && amax < INFINITY) {
+        int e;
+        frexpf(amax, &e);                  // amax = f * 2^e, f in [0.5, 1)  =>  |xs| < 2^e
+        S = ldexp(1.0, e - 30);
+        invS = ldexp(1.0, 30 - e);
+    }
+    const int KB = K >> 6;
+    const int mt = t >> 2, m0 = (t & 3) * 4;
+    double qsum[1] = {0.0};
+    for (int c0 = threadIdx.x * 16; c0 < K; c0 += kRT * 16) {
+        unsigned pl[4][4];
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) pl[d][j] = 0u;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float xs = (float)(row[c0 + i] * (double)a.range[c0 + i]);
+            int q = __double2int_rn((double)xs * invS);
+            qsum[0] += (double)q;
+            const int d3 = (int)(signed char)(q & 0xff); q = (q - d3) >> 8;
+            const int d2 = (int)(signed char)(q & 0xff); q = (q - d2) >> 8;
+            const int d1 = (int)(signed char)(q & 0xff); q = (q - d1) >> 8;
+            const int sh = 8 * (i & 3);
+            pl[0][i >> 2] |= (unsigned)(q & 0xff) << sh;
+            pl[1][i >> 2] |= (unsigned)(d1 & 0xff) << sh;
+            pl[2][i >> 2] |= (unsigned)(d2 & 0xff) << sh;
+            pl[3][i >> 2] |= (unsigned)(d3 & 0xff) << sh;
+        }
+        const int kb = c0 >> 6, g = (c0 & 63) >> 4;
+        signed char *frag = a.dig + ((size_t)mt * KB + kb) * 1024;
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+            *reinterpret_cast<uint4 *>(frag + (16 * g + m0 + d) * 16) = make_uint4(pl[d][0], pl[d][1], pl[d][2], pl[d][3]);
+    }
+    rsum<1>(qsum, red);
+    if (threadIdx.x == 0) { a.S[t] = S; a.qs[t] = qsum[0]; a.zp[t] = z[0]; }
+}
+
+// ---------------------------------------------------------------------------
+// GEMM: tot[t, j] = sum_k q[t, k] * (code[k, j] - 128), exact in int64.
+// Workgroup = 4 wavefronts = 64 tokens x 64 columns; wavefront (wm, wn) holds
+// 8 M-tiles x 2 N-tiles of accumulators and streams fragments of both operands
+// straight from memory (software-pipelined one block ahead).  gridDim.z splits
+// the contraction; partial totals are then added with integer atomics, which
+// commute exactly.
+// ---------------------------------------------------------------------------
+struct GemmArgs {
+    const signed char *dig;     // fragments [MT][KB][1024]
+    const uint8_t *w16;         // blocks [NT][KB][1024]
+    long long *tot;             // [4*MT][ldd]
+    int MT, NT, KB, ldd, kb_per_split, atomic;
+};
+
+constexpr int kGM = 8, kGN = 2;
+
+__global__ void __launch_bounds__(256) gemm8_kernel(const GemmArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave & 1, wn = wave >> 1;
+    const int mt0 = blockIdx.y * 16 + wm * kGM, nt0 = blockIdx.x * 4 + wn * kGN;
+    const int kb0 = blockIdx.z * a.kb_per_split;
+    int kb1 = kb0 + a.kb_per_split;
+    if (kb1 > a.KB) kb1 = a.KB;
+    if (mt0 >= a.MT || nt0 >= a.NT || kb0 >= kb1) return;
+
+    const uint4 *ap[kGM];
+    const uint4 *bp[kGN];
+#pragma unroll
+    for (int i = 0; i < kGM; ++i) {
+        const int mt = mt0 + i < a.MT ? mt0 + i : a.MT - 1;       // clamped: loads stay unconditional
+        ap[i] = reinterpret_cast<const uint4 *>(a.dig + ((size_t)mt * a.KB + kb0) * 1024) + lane;
+    }
+#pragma unroll
+    for (int j = 0; j < kGN; ++j) {
+        const int nt = nt0 + j < a.NT ? nt0 + j : a.NT - 1;
+        bp[j] = reinterpret_cast<const uint4 *>(a.w16 + ((size_t)nt * a.KB + kb0) * 1024) + lane;
+    }
+    v4i acc[kGM][kGN];
+#pragma unroll
+    for (int i = 0; i < kGM; ++i)
+#pragma unroll
+        for (int j = 0; j < kGN; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+
+    uint4 A[kGM], B[kGN];
+#pragma unroll
+    for (int i = 0; i < kGM; ++i) A[i] = ap[i][0];
+#pragma unroll
+    for (int j = 0; j < kGN; ++j) B[j] = bp[j][0];
+    const int nk = kb1 - kb0;
+    for (int k = 0; k < nk; ++k) {
+        uint4 An[kGM], Bn[kGN];
+        const int kn = k + 1 < nk ? k + 1 : k;                    // last step reloads itself (unused)
+#pragma unroll
+        for (int i = 0; i < kGM; ++i) An[i] = ap[i][(size_t)kn * 64];
+#pragma unroll
+        for (int j = 0; j < kGN; ++j) Bn[j] = bp[j][(size_t)kn * 64];
+#pragma unroll
+        for (int i = 0; i < kGM; ++i) {
+            const v4i Av = {(int)A[i].x, (int)A[i].y, (int)A[i].z, (int)A[i].w};
+#pragma unroll
+            for (int j = 0; j < kGN; ++j) {
+                const v4i Bv = {(int)B[j].x, (int)B[j].y, (int)B[j].z, (int)B[j].w};
+                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Av, Bv, acc[i][j], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kGM; ++i) A[i] = An[i];
+#pragma unroll
+        for (int j = 0; j < kGN; ++j) B[j] = Bn[j];
+    }
+    // lane 16g + n, register i  <->  digit i of token 4*mt + g, column 16*nt + n
+    const int g = lane >> 4, n = lane & 15;
+#pragma unroll
+    for (int i = 0; i < kGM; ++i) {
+        if (mt0 + i >= a.MT) continue;
+#pragma unroll
+        for (int j = 0; j < kGN; ++j) {
+            if (nt0 + j >= a.NT) continue;
+            const v4i d = acc[i][j];
+            const long long tot = ((((long long)d.x * 256 + d.y) * 256 + d.z) * 256) + d.w;
+            long long *p = a.tot + (size_t)(4 * (mt0 + i) + g) * a.ldd + 16 * (nt0 + j) + n;
+            if (a.atomic) atomicAdd(reinterpret_cast<unsigned long long *>(p), (unsigned long long)tot);
+            else *p = tot;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256) rows_fill_kernel(long long *p, size_t n) {
+    const size_t i0 = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (i0 + i < n) p[i0 + i] = 0;
+}
+
+// ---------------------------------------------------------------------------
+// y[t, j] = S_t * tot + 128 * S_t * sum q_t + zp_t, then the phase's element-wise tail.
+// ---------------------------------------------------------------------------
+struct FinishArgs {
+    int R, N, ldd;
+    const long long *tot;
+    const double *S, *qs, *zp;
+    double *out;                // [R, N]
+    const double *gate;         // ROW_GATE_ADD: raw receptance [R, N]
+};
+
+template <int OP>
+__global__ void __launch_bounds__(256) rows_finish_kernel(const FinishArgs a) {
+    const int t = blockIdx.y;
+    const int j = blockIdx.x * 256 + threadIdx.x;
+    if (j >= a.N) return;
+    const double S = a.S[t];
+    const double y = S * (double)a.tot[(size_t)t * a.ldd + j] + 128.0 * (S * a.qs[t]) + a.zp[t];
+    double *o = a.out + (size_t)t * a.N + j;
+    if (OP == ROW_STORE) *o = y;
+    else if (OP == ROW_RELU2) { const double r = y > 0.0 ? y : 0.0; *o = r * r; }            // block.py:97
+    else if (OP == ROW_ADD) *o += y;                                                          // block.py:80
+    else if (OP == ROW_GATE_ADD) *o += y * (1.0 / (1.0 + exp(-a.gate[(size_t)t * a.N + j]))); // block.py:95-100
+}
+
+// ---------------------------------------------------------------------------
+// WKV + receptance gate           (block.py:69-78, wkv.py:23-39, operators.cu:6-37)
+// sequence: thread = channel, serial over the T rows; batch: thread = (row, channel).
+// ---------------------------------------------------------------------------
+struct WkvRowsArgs {
+    int C, R, sequence;
+    const double *k, *v, *r;    // [R, C]
+    const double *w, *u;        // [C]  (w = -exp(time_decay))
+    double *state;              // rows aa, bb, pp of the layer: state + 2C; batch: + row * state_stride
+    int64_t state_stride;
+    double *out;                // [R, C]  wkv * sigmoid(r)
+};
+
+__global__ void __launch_bounds__(64) wkv_rows_kernel(const WkvRowsArgs a) {
+    const int c = blockIdx.x * 64 + threadIdx.x;
+    if (c >= a.C) return;
+    const int C = a.C;
+    const double w = a.w[c], u = a.u[c];
+    const int t0 = a.sequence ? 0 : blockIdx.y, t1 = a.sequence ? a.R : blockIdx.y + 1;
+    double *st = a.state + (a.sequence ? 0 : (size_t)blockIdx.y * a.state_stride);
+    double aa = st[c], bb = st[C + c], pp = st[2 * C + c];
+    for (int t = t0; t < t1; ++t) {
+        const size_t i = (size_t)t * C + c;
+        const double y = wkv_step<double>(w, u, a.k[i], a.v[i], aa, bb, pp);
+        a.out[i] = y * (1.0 / (1.0 + exp(-a.r[i])));
+    }
+    st[c] = aa; st[C + c] = bb; st[2 * C + c] = pp;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+size_t rows_dig_bytes(int64_t R, int64_t K) { return (size_t)(ceil_div(R, 4) * (K / 64) * 1024); }
+size_t rows_tot_bytes(int64_t R, int64_t N) { return (size_t)(ceil_div(R, 4) * 4 * round_up(N, 16) * 8); }
+
+int rows_embed(hipStream_t st, const int64_t *tokens, int64_t R, int V, int C, const float *emb, const double *w,
+               const double *b, double *x) {
+    hipLaunchKernelGGL(rows_embed_kernel, dim3((unsigned)R), dim3(kRT), 0, st, tokens, V, C, emb, w, b, x);
+    RWKV_CHECK_LAUNCH("rows_embed_kernel");
+    return RWKV_OK;
+}
+
+int rows_ln_mix(hipStream_t st, int n_mix, int64_t R, int C, bool sequence, const double *x, const double *ln_w,
+                const double *ln_b, const double *mu, const double *prev0, double *shift_dst, int64_t prev_stride,
+                double *mix) {
+    LnMixArgs a;
+    a.C = C; a.R = (int)R; a.sequence = sequence ? 1 : 0; a.x = x; a.ln_w = ln_w; a.ln_b = ln_b; a.mu = mu;
+    a.prev0 = prev0; a.shift_dst = shift_dst; a.prev_stride = prev_stride; a.mix = mix;
+    const dim3 grid((unsigned)R), block(kRT);
+    switch (n_mix) {
+        case 0: hipLaunchKernelGGL(rows_ln_mix_kernel<0>, grid, block, 0, st, a); break;
+        case 2: hipLaunchKernelGGL(rows_ln_mix_kernel<2>, grid, block, 0, st, a); break;
+        case 3: hipLaunchKernelGGL(rows_ln_mix_kernel<3>, grid, block, 0, st, a); break;
+        default: return set_error(RWKV_ERR_ARG, "rows_ln_mix: unsupported mix count %d", n_mix);
+    }
+    RWKV_CHECK_LAUNCH("rows_ln_mix_kernel");
+    return RWKV_OK;
+}
+
+int rows_matmul(hipStream_t st, const RowsScratch &s, int64_t R, int64_t K, int64_t N, const double *in,
+                const uint8_t *w16, const float *range, const double *offset, int op, double *out,
+                const double *gate) {
+    if (K % 64 != 0) return set_error(RWKV_ERR_SIZE, "rows_matmul: contraction length %lld is not a multiple of 64",
+                                      (long long)K);
+    QuantArgs q;
+    q.K = (int)K; q.in = in; q.range = range; q.offset = offset; q.dig = s.dig; q.S = s.S; q.qs = s.qs; q.zp = s.zp;
+    hipLaunchKernelGGL(rows_quant_kernel, dim3((unsigned)R), dim3(kRT), 0, st, q);
+    RWKV_CHECK_LAUNCH("rows_quant_kernel");
+
+    GemmArgs g;
+    g.dig = s.dig; g.w16 = w16; g.tot = s.tot;
+    g.MT = (int)ceil_div(R, 4); g.NT = (int)ceil_div(N, 16); g.KB = (int)(K / 64); g.ldd = g.NT * 16;
+    const int gx = (int)ceil_div(g.NT, 4), gy = (int)ceil_div(g.MT, 16);
+    // Split the contraction until the grid has a few workgroups per compute unit.
+    int split = 1;
+    while (gx * gy * split < 512 && g.KB / (split * 2) >= 8) split *= 2;
+    g.kb_per_split = (int)ceil_div(g.KB, split);
+    g.atomic = split > 1;
+    if (g.atomic) {
+        // (a fill kernel rather than a memset node, so the sequence can be captured in a graph)
+        const size_t n = (size_t)g.MT * 4 * g.ldd;
+        hipLaunchKernelGGL(rows_fill_kernel, dim3((unsigned)ceil_div((int64_t)n, 1024)), dim3(256), 0, st, s.tot, n);
+    }
+    hipLaunchKernelGGL(gemm8_kernel, dim3(gx, gy, split), dim3(256), 0, st, g);
+    RWKV_CHECK_LAUNCH("gemm8_kernel");
+
+    FinishArgs f;
+    f.R = (int)R; f.N = (int)N; f.ldd = g.ldd; f.tot = s.tot; f.S = s.S; f.qs = s.qs; f.zp = s.zp; f.out = out;
+    f.gate = gate;
+    const dim3 fg((unsigned)ceil_div(N, 256), (unsigned)R), fb(256);
+    switch (op) {
+        case ROW_STORE: hipLaunchKernelGGL(rows_finish_kernel<ROW_STORE>, fg, fb, 0, st, f); break;
+        case ROW_RELU2: hipLaunchKernelGGL(rows_finish_kernel<ROW_RELU2>, fg, fb, 0, st, f); break;
+        case ROW_ADD: hipLaunchKernelGGL(rows_finish_kernel<ROW_ADD>, fg, fb, 0, st, f); break;
+        case ROW_GATE_ADD: hipLaunchKernelGGL(rows_finish_kernel<ROW_GATE_ADD>, fg, fb, 0, st, f); break;
+        default: return set_error(RWKV_ERR_ARG, "rows_matmul: unknown tail %d", op);
+    }
+    RWKV_CHECK_LAUNCH("rows_finish_kernel");
+    return RWKV_OK;
+}
+
+int rows_wkv(hipStream_t st, int64_t R, int C, bool sequence, const double *k, const double *v, const double *r,
+             const double *w, const double *u, double *state, int64_t state_stride, double *out) {
+    WkvRowsArgs a;
+    a.C = C; a.R = (int)R; a.sequence = sequence ? 1 : 0; a.k = k; a.v = v; a.r = r; a.w = w; a.u = u;
+    a.state = state; a.state_stride = state_stride; a.out = out;
+    hipLaunchKernelGGL(wkv_rows_kernel, dim3((unsigned)ceil_div(C, 64), sequence ? 1u : (unsigned)R), dim3(64), 0, st, a);
+    RWKV_CHECK_LAUNCH("wkv_rows_kernel");
+    return RWKV_OK;
+}
+
+}  // namespace rwkv

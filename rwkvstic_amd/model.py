@@ -135,6 +135,7 @@ class HipRWKV:
         self.fused_step = bool(L.rwkv_model_has_fused_step(handle))
         self._ws: Optional[torch.Tensor] = None
         self._ws_tokens = 0
+        self._bws: Optional[torch.Tensor] = None
 
     def __del__(self):
         h = getattr(self, "_handle", None)
@@ -186,6 +187,28 @@ class HipRWKV:
         return logits, state
 
     __call__ = forward
+
+    def forward_batch(self, tokens, states: torch.Tensor):
+        """One token for each of B independent sequences: ``tokens[B]``, ``states[B, L, 5, C]`` float64
+        (updated in place) -> ``(logits[B, V] float64, states)``."""
+        tok = torch.as_tensor(tokens, dtype=torch.int64).reshape(-1).to(self.device)
+        B = tok.numel()
+        if (not isinstance(states, torch.Tensor) or states.device.type != "cuda" or states.dtype != torch.float64
+                or tuple(states.shape) != (B, self.layers, 5, self.dims) or not states.is_contiguous()):
+            raise ValueError(f"states must be a contiguous CUDA float64 tensor of shape "
+                             f"({B}, {self.layers}, 5, {self.dims})")
+        L = N.lib()
+        nbytes = L.rwkv_model_batch_workspace_bytes(self._handle, B)
+        if nbytes == 0:
+            raise RuntimeError("forward_batch needs the model built with fused=True and n_embd, n_ffn multiples of 64")
+        if self._bws is None or self._bws.numel() < nbytes:
+            self._bws = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+        logits = torch.empty((B, self.vocab), dtype=torch.float64, device=self.device)
+        with torch.cuda.device(self.device):
+            N.check(L.rwkv_model_forward_batch(self._handle, torch.cuda.current_stream().cuda_stream,
+                                               tok.data_ptr(), B, states.data_ptr(), logits.data_ptr(),
+                                               self._bws.data_ptr(), self._bws.numel()))
+        return logits, states
 
     def decode_greedy(self, token: int, n: int, state: torch.Tensor):
         """Feed ``token`` then greedily generate: returns ``(tokens[n] int64 on device, last logits, state)``

@@ -209,6 +209,26 @@ def mm8_packed(x: torch.Tensor, packed: torch.Tensor, n_in: int, n_out: int,
     return y
 
 
+def gemm8(x: torch.Tensor, packed16: torch.Tensor, rng: torch.Tensor, off: torch.Tensor,
+          n_in: int, n_out: int) -> torch.Tensor:
+    """``y[T, n_out] = x[T, n_in] @ dequantised matrix`` with the single-token arithmetic
+    (fp32(x*range) as exact fixed point, integer dot products, float64 zero-point term);
+    the T > 1 branch of MM8.forward (matmul.py:56-57) without its bfloat16 rounding."""
+    _req(x, torch.float64, "x"); _contig(x, "x")
+    _req(packed16, torch.uint8, "packed16"); _req(rng, torch.float32, "range"); _req(off, torch.float64, "offset")
+    if x.dim() != 2 or x.shape[1] != n_in:
+        raise ValueError("gemm8: x must be [T, n_in]")
+    T = x.shape[0]
+    L = N.lib()
+    if packed16.numel() < L.rwkv_packed_m16_bytes(n_in, n_out) or rng.numel() < n_in or off.numel() < n_in:
+        raise ValueError("gemm8: matrix buffers smaller than (n_in, n_out)")
+    y = torch.empty((T, n_out), dtype=torch.float64, device=x.device)
+    ws = _workspace(L.rwkv_gemm8_workspace_bytes(T, n_in, n_out), x.device)
+    N.check(L.rwkv_gemm8(_stream(), T, n_in, n_out, x.data_ptr(), packed16.data_ptr(), rng.data_ptr(),
+                         off.data_ptr(), y.data_ptr(), ws.data_ptr(), ws.numel()))
+    return y
+
+
 def wkv_f32(w, u, k, v, aa, bb, pp) -> torch.Tensor:
     """Max-shifted float32 WKV; ``k, v`` are ``[B, T, C]``; state ``[B, C]`` updated in place."""
     for name, t in (("w", w), ("u", u), ("k", k), ("v", v), ("aa", aa), ("bb", bb), ("pp", pp)):

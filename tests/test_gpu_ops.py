@@ -250,3 +250,36 @@ def test_pack_m16_round_trip(ops):
         g, n = divmod(lane, 16)
         want = (c[16 * g:16 * g + 16, n].cpu().to(torch.int16) - 128).to(torch.int8)
         assert torch.equal(p[lane].view(torch.int8), want)
+
+
+@pytest.mark.parametrize("T,K,N", [(1, 64, 16), (5, 256, 100), (64, 2560, 2560), (130, 2560, 10240),
+                                   (33, 10240, 2560), (8, 2560, 50277)])
+def test_gemm8_matches_fp64_dense(ops, T, K, N):
+    """Prompt GEMM (matmul.py:56-57 without its bfloat16 rounding) against the float64 dense product."""
+    g = torch.Generator().manual_seed(T * 7 + K + N)
+    w = torch.randn(N, K, generator=g) * 0.02
+    codes, rng, off = O.quantize_matrix(w)
+    x = torch.randn(T, K, generator=g, dtype=torch.float64)
+    x[0, : K // 2] *= 50.0                                    # rows with very different scales
+    want = O.mm8_naive(x, codes, rng, off, dtype=torch.float64)
+    dev = "cuda"
+    p16 = ops.pack_m16(codes.to(dev))
+    got = ops.gemm8(x.to(dev), p16, rng.to(dev), off.to(dev), K, N).cpu()
+    bound = ((x.abs() * rng.double()) @ codes.double()).max(dim=1, keepdim=True).values
+    err = ((got - want).abs() / bound).max().item()
+    print(f"gemm8 T={T} K={K} N={N}: max err / sum|terms| = {err:.2e}", flush=True)
+    assert err < 2e-7                                         # float32 rounding of x*range, nothing else
+
+
+def test_gemm8_rows_do_not_depend_on_batching(ops):
+    """Integer accumulation: a row's result is bit-identical whether the contraction is split (few rows)
+    or not (many rows), and wherever the row sits in its tile."""
+    g = torch.Generator().manual_seed(3)
+    K, N = 2560, 2560
+    w = torch.randn(N, K, generator=g) * 0.02
+    codes, rng, off = O.quantize_matrix(w)
+    x = torch.randn(300, K, generator=g, dtype=torch.float64).cuda()
+    p16 = ops.pack_m16(codes.cuda())
+    full = ops.gemm8(x, p16, rng.cuda(), off.cuda(), K, N)
+    few = ops.gemm8(x[37:40].contiguous(), p16, rng.cuda(), off.cuda(), K, N)
+    assert torch.equal(full[37:40], few)
