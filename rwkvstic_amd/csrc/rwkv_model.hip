@@ -494,7 +494,7 @@ constexpr int64_t kRowsChunk = 1024;   // rows per pass: bounds the workspace of
 constexpr int64_t kRowsMin = 4;        // shorter prompts go token by token
 
 struct RowsWs {
-    double *x, *mix, *kvr, *att, *h, *prev0;
+    double *x, *mix, *kvr, *att, *h, *prev0, *wkv_scr;
     RowsScratch s;
 };
 
@@ -504,6 +504,7 @@ size_t rows_ws_bytes(int64_t R, int64_t C, int64_t F, int64_t n_wide) {
     n += round_up((size_t)R * C * 8, 256) * 8;          // x, mix[3], kvr[3], att
     n += round_up((size_t)R * F * 8, 256);              // h
     n += round_up((size_t)C * 8, 256);                  // prev0
+    n += round_up(rows_wkv_scratch_bytes(R, C), 256);
     n += round_up((size_t)R * 8, 256) * 3;              // S, qs, zp
     n += round_up(rows_dig_bytes(R, F), 256);
     n += round_up(rows_tot_bytes(R, n_wide), 256);
@@ -520,6 +521,7 @@ RowsWs rows_carve(void *ws, int64_t R, int64_t C, int64_t F, int64_t n_wide) {
     w.att = (double *)take((size_t)R * C * 8);
     w.h = (double *)take((size_t)R * F * 8);
     w.prev0 = (double *)take((size_t)C * 8);
+    w.wkv_scr = (double *)take(rows_wkv_scratch_bytes(R, C));
     w.s.S = (double *)take((size_t)R * 8);
     w.s.qs = (double *)take((size_t)R * 8);
     w.s.zp = (double *)take((size_t)R * 8);
@@ -561,7 +563,7 @@ int rows_layers(rwkv_model *m, hipStream_t st, const int64_t *tokens, int64_t R,
             RWKV_TRY(rows_matmul(st, w.s, R, C, C, w.mix + i * RC, kvr[i]->packed16, kvr[i]->range, kvr[i]->offset,
                                  ROW_STORE, w.kvr + i * RC, nullptr));
         RWKV_TRY(rows_wkv(st, R, C, sequence, w.kvr, w.kvr + RC, w.kvr + 2 * RC, L.time_decay, L.time_first,
-                          sl + 2 * (size_t)C, state_stride, w.att));
+                          sl + 2 * (size_t)C, state_stride, w.att, w.wkv_scr));
         RWKV_TRY(rows_matmul(st, w.s, R, C, C, w.att, L.att_o.packed16, L.att_o.range, L.att_o.offset, ROW_ADD, w.x,
                              nullptr));
         // ChannelMix (block.py:82-100)

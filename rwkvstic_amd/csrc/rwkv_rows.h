@@ -16,6 +16,7 @@ struct RowsScratch {
 };
 size_t rows_dig_bytes(int64_t R, int64_t K);
 size_t rows_tot_bytes(int64_t R, int64_t N);
+size_t rows_wkv_scratch_bytes(int64_t R, int64_t C);
 
 int rows_embed(hipStream_t st, const int64_t *tokens, int64_t R, int V, int C, const float *emb, const double *w,
                const double *b, double *x);
@@ -28,6 +29,7 @@ int rows_matmul(hipStream_t st, const RowsScratch &s, int64_t R, int64_t K, int6
                 const uint8_t *w16, const float *range, const double *offset, int op, double *out,
                 const double *gate);
 int rows_wkv(hipStream_t st, int64_t R, int C, bool sequence, const double *k, const double *v, const double *r,
-             const double *w, const double *u, double *state, int64_t state_stride, double *out);
+             const double *w, const double *u, double *state, int64_t state_stride, double *out,
+             double *scratch /* rows_wkv_scratch_bytes(R, C), or null: serial over the rows */);
 
 }  // namespace rwkv

@@ -358,12 +358,71 @@ __global__ void __launch_bounds__(64) wkv_rows_kernel(const WkvRowsArgs a) {
     st[c] = aa; st[C + c] = bb; st[2 * C + c] = pp;
 }
 
+
+// Long sequences: the recurrence is linear in (aa, bb), so T steps split into chunks of kWkvChunk:
+// (1) every chunk's own contribution from an empty state, in parallel; (2) a short serial pass that
+// turns them into each chunk's incoming state (a chunk decays its input by e^{n w}); (3) every chunk
+// replays its steps from that state, in parallel.  Same sums as the serial order up to float64 rounding.
+constexpr int kWkvChunk = 32;
+
+__global__ void __launch_bounds__(64) wkv_chunk_local_kernel(const WkvRowsArgs a, double *scr) {
+    const int c = blockIdx.x * 64 + threadIdx.x, j = blockIdx.y;
+    if (c >= a.C) return;
+    const int C = a.C;
+    const double w = a.w[c], u = a.u[c];
+    const int t0 = j * kWkvChunk, t1 = min(t0 + kWkvChunk, a.R);
+    double aa = 0.0, bb = 0.0, pp = -1e30;
+    for (int t = t0; t < t1; ++t) {
+        const size_t i = (size_t)t * C + c;
+        (void)wkv_step<double>(w, u, a.k[i], a.v[i], aa, bb, pp);
+    }
+    double *o = scr + (size_t)j * 3 * C;
+    o[c] = aa; o[C + c] = bb; o[2 * C + c] = pp;
+}
+
+__global__ void __launch_bounds__(64) wkv_chunk_prefix_kernel(const WkvRowsArgs a, double *scr, int n_chunks) {
+    const int c = blockIdx.x * 64 + threadIdx.x;
+    if (c >= a.C) return;
+    const int C = a.C;
+    const double w = a.w[c];
+    double aa = a.state[c], bb = a.state[C + c], pp = a.state[2 * C + c];
+    for (int j = 0; j < n_chunks; ++j) {
+        double *o = scr + (size_t)j * 3 * C;
+        const double la = o[c], lb = o[C + c], lp = o[2 * C + c];
+        o[c] = aa; o[C + c] = bb; o[2 * C + c] = pp;              // incoming state of chunk j
+        const int n = min(kWkvChunk, a.R - j * kWkvChunk);
+        const double s = pp + (double)n * w;
+        const double p = fmax(s, lp);
+        const double f1 = exp(s - p), f2 = exp(lp - p);
+        aa = f1 * aa + f2 * la;
+        bb = f1 * bb + f2 * lb;
+        pp = p;
+    }
+    a.state[c] = aa; a.state[C + c] = bb; a.state[2 * C + c] = pp;
+}
+
+__global__ void __launch_bounds__(64) wkv_chunk_replay_kernel(const WkvRowsArgs a, const double *scr) {
+    const int c = blockIdx.x * 64 + threadIdx.x, j = blockIdx.y;
+    if (c >= a.C) return;
+    const int C = a.C;
+    const double w = a.w[c], u = a.u[c];
+    const int t0 = j * kWkvChunk, t1 = min(t0 + kWkvChunk, a.R);
+    const double *in = scr + (size_t)j * 3 * C;
+    double aa = in[c], bb = in[C + c], pp = in[2 * C + c];
+    for (int t = t0; t < t1; ++t) {
+        const size_t i = (size_t)t * C + c;
+        const double y = wkv_step<double>(w, u, a.k[i], a.v[i], aa, bb, pp);
+        a.out[i] = y * (1.0 / (1.0 + exp(-a.r[i])));
+    }
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 size_t rows_dig_bytes(int64_t R, int64_t K) { return (size_t)(ceil_div(R, 4) * (K / 64) * 1024); }
+size_t rows_wkv_scratch_bytes(int64_t R, int64_t C) { return (size_t)(ceil_div(R, kWkvChunk) * 3 * C * 8); }
 size_t rows_tot_bytes(int64_t R, int64_t N) { return (size_t)(ceil_div(R, 4) * 4 * round_up(N, 16) * 8); }
 
 int rows_embed(hipStream_t st, const int64_t *tokens, int64_t R, int V, int C, const float *emb, const double *w,
@@ -433,10 +492,19 @@ int rows_matmul(hipStream_t st, const RowsScratch &s, int64_t R, int64_t K, int6
 }
 
 int rows_wkv(hipStream_t st, int64_t R, int C, bool sequence, const double *k, const double *v, const double *r,
-             const double *w, const double *u, double *state, int64_t state_stride, double *out) {
+             const double *w, const double *u, double *state, int64_t state_stride, double *out, double *scratch) {
     WkvRowsArgs a;
     a.C = C; a.R = (int)R; a.sequence = sequence ? 1 : 0; a.k = k; a.v = v; a.r = r; a.w = w; a.u = u;
     a.state = state; a.state_stride = state_stride; a.out = out;
+    if (sequence && scratch && R >= 2 * kWkvChunk) {
+        const int n_chunks = (int)ceil_div(R, kWkvChunk);
+        const dim3 grid((unsigned)ceil_div(C, 64), (unsigned)n_chunks);
+        hipLaunchKernelGGL(wkv_chunk_local_kernel, grid, dim3(64), 0, st, a, scratch);
+        hipLaunchKernelGGL(wkv_chunk_prefix_kernel, dim3(grid.x), dim3(64), 0, st, a, scratch, n_chunks);
+        hipLaunchKernelGGL(wkv_chunk_replay_kernel, grid, dim3(64), 0, st, a, (const double *)scratch);
+        RWKV_CHECK_LAUNCH("wkv_chunk kernels");
+        return RWKV_OK;
+    }
     hipLaunchKernelGGL(wkv_rows_kernel, dim3((unsigned)ceil_div(C, 64), sequence ? 1u : (unsigned)R), dim3(64), 0, st, a);
     RWKV_CHECK_LAUNCH("wkv_rows_kernel");
     return RWKV_OK;

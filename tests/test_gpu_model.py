@@ -171,11 +171,12 @@ def test_fused_step_matches_oracle_and_phase_kernels(C, L, V):
     assert torch.equal(l2, lg) and torch.equal(s2, sg)
 
 
-def test_prompt_gemm_path_matches_token_steps(tiny):
+@pytest.mark.parametrize("n_prompt", [23, 100])      # 100: the chunked WKV scan (3 full chunks + a partial one)
+def test_prompt_gemm_path_matches_token_steps(tiny, n_prompt):
     """A prompt through the GEMM path leaves the same logits and state as the same tokens fed one at a time
     (chunk-size invariance; block.py:58-67 token shift, wkv.py:23-39 recurrence)."""
     ref, hip = tiny
-    toks = synth.random_tokens(23, V=512, seed=11).tolist()
+    toks = synth.random_tokens(n_prompt, V=512, seed=11).tolist()
     lg, sg = hip.forward(toks, hip.emptyState.clone())
     s1 = hip.emptyState.clone()
     for t in toks:
