@@ -1,0 +1,164 @@
+"""User-facing shell with the reference's surface: ``RWKV(path, ...)`` returns an object that behaves like
+``RWKVMaster`` (reference src/rwkvstic/rwkvMaster.py:14-125) over the HIP FASTQUANT model
+(reference load.py:18,42-47 picks ``OptRWKV`` + the ``typical`` sampler for this mode).
+
+Kept from the reference, because callers rely on it: ``forward`` adds ``end_adj`` to logit 0 before
+sampling and stops on ``stopTokens`` / ``stopStrings``; ``lastToken`` starts at ``[187]``; ``loadContext``
+sets ``lastToken`` to the last token of ``ctx`` (not of ``newctx``) and leaves the caller's state untouched;
+``getState``/``setState`` exchange ``(state, lastToken)`` pairs.  Changed: prompts are fed in chunks of 1024
+tokens (the reference's default is 20) because they run as GEMMs here, and sampling stays on the GPU.
+"""
+from __future__ import annotations
+
+from typing import Callable, Dict, Iterable, List, Optional, Sequence, Union
+
+import torch
+
+MODE = "hip-fastquant"
+
+
+def _clone(x):
+    return x.clone() if hasattr(x, "clone") else x
+
+
+def typical(logits: torch.Tensor, temp: float = 1.0, tau: float = 0.95, generator=None, **_unused) -> int:
+    """Locally typical sampling (reference agnostic/samplers/typical.py:1-17): keep the tokens whose surprise
+    is closest to the entropy until their mass reaches ``tau``, then sample; float32, on the logits' device."""
+    probs = torch.softmax(logits.float(), dim=-1)
+    surprise = -torch.log(probs)
+    ent = torch.nansum(surprise * probs, dim=-1, keepdim=True)
+    dist = (surprise - ent).abs()
+    order = torch.argsort(dist)
+    cum = torch.cumsum(probs[order], dim=-1)
+    cutoff = int((cum < tau).sum())
+    cutoff = min(cutoff, order.numel() - 1)
+    probs = torch.where(dist > dist[order[cutoff]], torch.zeros_like(probs), probs)
+    if temp != 1.0:
+        probs = probs ** (1.0 / temp)
+    return int(torch.multinomial(probs, num_samples=1, generator=generator)[0])
+
+
+def greedy(logits: torch.Tensor, *_args, **_kw) -> int:
+    return int(torch.argmax(logits))
+
+
+class TokenIds:
+    """Stand-in tokenizer for callers that work in token ids: ``encode`` accepts a sequence of ints (or a
+    string of whitespace-separated ints), ``decode`` joins ids with spaces."""
+
+    def encode(self, x) -> List[int]:
+        if isinstance(x, str):
+            return [int(t) for t in x.split()]
+        return [int(t) for t in x]
+
+    def decode(self, ids: Iterable[int]) -> str:
+        return " ".join(str(int(i)) for i in ids)
+
+
+def load_tokenizer(spec):
+    """``None`` -> :class:`TokenIds`; a path -> a ``tokenizers`` JSON file (the reference ships the GPT-NeoX 20B
+    vocabulary, tokenizer/__init__.py:3-8); anything with ``encode``/``decode`` is used as is."""
+    if spec is None:
+        return TokenIds()
+    if isinstance(spec, str):
+        from tokenizers import Tokenizer
+        tk = Tokenizer.from_file(spec)
+
+        class _Wrap:
+            def encode(self, s):
+                return tk.encode(s).ids
+
+            def decode(self, ids):
+                return tk.decode([int(i) for i in ids])
+        return _Wrap()
+    return spec
+
+
+class RWKVMaster:
+    logging = False
+
+    def __init__(self, model, emptyState, sampler: Optional[Callable] = typical, tokenizer=None):
+        self.model = model
+        self.tokenizer = load_tokenizer(tokenizer)
+        self.emptyState = _clone(emptyState)
+        self.myState = _clone(emptyState)
+        self.lastToken = [187]                   # rwkvMaster.py:23
+        self.sampler = sampler
+
+    # ------------------------------------------------------------------ generation (rwkvMaster.py:28-56)
+    def forward(self, state=None, number: int = 1, stopStrings: Sequence[str] = ("<|endoftext|>",),
+                stopTokens: Sequence[int] = (0,), progressLambda: Callable[[Dict], None] = lambda x: x,
+                end_adj: float = -990.0, **kwargs):
+        ostate = self.myState if state is None else state
+        tokens: List[int] = []
+        logits, text = None, ""
+        for i in range(number):
+            logits, ostate = self.model.forward(self.lastToken, ostate)
+            logits[0] += end_adj
+            self.myState = ostate
+            sampled = self.sample(logits, **kwargs) if self.sampler is not None else int(torch.argmax(logits))
+            self.lastToken = [int(sampled)]
+            tokens.append(self.lastToken[0])
+            text = self.tokenizer.decode(tokens)
+            progressLambda({"logits": logits, "state": ostate, "output": text, "progress": i, "tokens": tokens,
+                            "total": number, "current": self.tokenizer.decode([tokens[-1]])})
+            if tokens[-1] in stopTokens:
+                break
+            if stopStrings and text.endswith(tuple(stopStrings)):
+                break
+        return {"logits": logits, "state": ostate, "output": text}
+
+    # ------------------------------------------------------------------ prompt (rwkvMaster.py:58-105)
+    def loadContext(self, newctx="", ctx="\n\n", statex=None, progressCallBack: Callable = lambda x: x,
+                    batch: int = 1024):
+        state = _clone(self.myState if statex is None else statex)
+        ctx_ids = self.tokenizer.encode(ctx)
+        new_ids = list(self.tokenizer.encode(newctx))
+        if ctx_ids:
+            self.lastToken = [int(ctx_ids[-1])]
+        for i in range(0, len(new_ids), max(1, batch)):
+            chunk = new_ids[i:i + max(1, batch)]
+            _, state = self.model.forward(chunk, state)
+            progressCallBack(chunk)
+        self.myState = _clone(state)
+        return new_ids, _clone(state)
+
+    # ------------------------------------------------------------------ small API (rwkvMaster.py:107-125)
+    def sample(self, logits, temp: float = 1.0, top_p_usual: float = 0.8, **kw) -> int:
+        return self.sampler(logits, temp, top_p_usual, **kw)
+
+    def decode(self, x):
+        return self.tokenizer.decode(x)
+
+    def encode(self, x):
+        return self.tokenizer.encode(x)
+
+    def setState(self, state):
+        self.myState = _clone(state[0])
+        self.lastToken = state[1]
+
+    def getState(self):
+        return _clone(self.myState), self.lastToken
+
+    def resetState(self):
+        self.myState = _clone(self.emptyState)
+        self.lastToken = [187]
+
+
+def RWKV(path: Union[str, Dict[str, torch.Tensor]], mode: str = MODE, *, tokenizer=None, device: str = "cuda",
+         sampler: Optional[Callable] = typical, **kwargs) -> RWKVMaster:
+    """``path``: a BlinkDL ``.pth`` checkpoint (loaded with ``weights_only=True``) or an already loaded state
+    dict.  Only the FASTQUANT mode exists in this backend (load.py:42-47); other modes raise."""
+    if mode != MODE:
+        raise ValueError(f"mode {mode!r} is not provided by this backend (only {MODE!r})")
+    if kwargs:
+        raise TypeError(f"unsupported options for mode {MODE!r}: {sorted(kwargs)}")
+    from .model import HipRWKV
+    if isinstance(path, str):
+        if not path.endswith(".pth"):
+            raise ValueError("only .pth checkpoints are supported")
+        weights = torch.load(path, map_location="cpu", weights_only=True)
+    else:
+        weights = path
+    model = HipRWKV(weights, device=device)
+    return RWKVMaster(model, model.emptyState.clone(), sampler, tokenizer)

@@ -227,3 +227,24 @@ def test_forward_batch_matches_per_sequence_steps(tiny):
         toks = nxt
     with pytest.raises(ValueError):
         hip.forward_batch(toks, batch_state[:2])
+
+
+def test_rwkv_shell_loads_checkpoint_file_and_generates(tmp_path, tiny):
+    """RWKV(path) -> RWKVMaster surface (load.py:18,42-47; rwkvMaster.py:28-105) over the HIP model."""
+    from rwkvstic_amd.master import RWKV, greedy
+    ref, hip = tiny
+    sd = synth.make_state_dict(layers=3, C=64, V=512, seed=5)
+    path = str(tmp_path / "tiny.pth")
+    torch.save(sd, path)
+    r = RWKV(path, sampler=greedy)
+    assert torch.equal(r.emptyState, hip.emptyState)
+    prompt = synth.random_tokens(9, V=512, seed=12).tolist()
+    ids, st = r.loadContext(newctx=prompt, ctx=[int(prompt[-1])])
+    assert ids == prompt and r.lastToken == [prompt[-1]]
+    # the reference feeds lastToken again after loadContext (rwkvMaster.py:31-33); mirror that here
+    out = r.forward(number=6, stopTokens=[], end_adj=0.0)
+    s2 = hip.emptyState.clone()
+    _, s2 = hip.forward(prompt, s2)
+    toks, _, s2 = hip.decode_greedy(prompt[-1], 6, s2)
+    assert out["output"] == " ".join(str(int(t)) for t in toks)
+    assert torch.equal(out["state"], s2)

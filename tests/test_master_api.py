@@ -1,0 +1,105 @@
+"""Behaviour of the RWKVMaster-compatible shell (reference rwkvMaster.py:14-125) with a stub model; no GPU."""
+import pytest
+import torch
+
+from rwkvstic_amd.master import RWKV, RWKVMaster, TokenIds, greedy, typical
+
+
+class StubModel:
+    """logits favour (last token + 1) mod V; the state counts the tokens it has seen."""
+    V = 16
+
+    def __init__(self):
+        self.calls = []
+
+    def forward(self, tokens, state):
+        tokens = [int(t) for t in tokens]
+        self.calls.append(tokens)
+        state += len(tokens)                       # in place, like the real model
+        logits = torch.zeros(self.V, dtype=torch.float64)
+        logits[(tokens[-1] + 1) % self.V] = 5.0
+        return logits, state
+
+
+def _master(sampler=greedy):
+    m = StubModel()
+    return m, RWKVMaster(m, torch.zeros(1, dtype=torch.float64), sampler)
+
+
+def test_defaults_and_state_api():
+    m, r = _master()
+    assert r.lastToken == [187] and float(r.myState) == 0.0
+    r.setState((torch.full((1,), 7.0, dtype=torch.float64), [3]))
+    st, last = r.getState()
+    assert float(st) == 7.0 and last == [3]
+    st += 1                                          # a clone: the master's own state is untouched
+    assert float(r.myState) == 7.0
+    r.resetState()
+    assert float(r.myState) == 0.0 and r.lastToken == [187]
+
+
+def test_forward_generates_until_number_and_updates_last_token():
+    m, r = _master()
+    r.lastToken = [2]
+    out = r.forward(number=4, stopTokens=[])
+    assert m.calls == [[2], [3], [4], [5]]
+    assert out["output"] == "3 4 5 6" and r.lastToken == [6]
+    assert float(out["state"]) == 4.0 and float(r.myState) == 4.0
+    assert out["logits"][0] == -990.0               # end_adj lands on logit 0
+
+
+def test_forward_stops_on_stop_token_and_stop_string():
+    m, r = _master()
+    r.lastToken = [2]
+    assert r.forward(number=10, stopTokens=[5])["output"] == "3 4 5"
+    m, r = _master()
+    r.lastToken = [2]
+    assert r.forward(number=10, stopTokens=[], stopStrings=["4"])["output"] == "3 4"
+    # end_adj can pull the end token up as well as push it down
+    m, r = _master()
+    r.lastToken = [2]
+    assert r.forward(number=3, end_adj=100.0)["output"] == "0"      # token 0 wins, and it is a stop token
+
+
+def test_forward_progress_callback_payload():
+    m, r = _master()
+    r.lastToken = [0]
+    seen = []
+    r.forward(number=2, stopTokens=[], progressLambda=seen.append)
+    assert [s["progress"] for s in seen] == [0, 1] and seen[1]["tokens"] == [1, 2] and seen[1]["total"] == 2
+    assert seen[1]["current"] == "2"
+
+
+def test_load_context_chunks_and_does_not_touch_callers_state():
+    m, r = _master()
+    mine = torch.full((1,), 10.0, dtype=torch.float64)
+    ids, st = r.loadContext(newctx=list(range(1, 8)), ctx=[9, 11], statex=mine, batch=3)
+    assert m.calls == [[1, 2, 3], [4, 5, 6], [7]] and ids == list(range(1, 8))
+    assert float(mine) == 10.0 and float(st) == 17.0 and float(r.myState) == 17.0
+    assert r.lastToken == [11]                       # the reference keeps the last token of ctx, not newctx
+    st += 1
+    assert float(r.myState) == 17.0
+
+
+def test_typical_sampler_stays_in_the_typical_set():
+    g = torch.Generator().manual_seed(0)
+    logits = torch.tensor([0.0, 0.1, 8.0, 0.2, -3.0], dtype=torch.float64)
+    assert all(typical(logits, 1.0, 0.5, generator=g) == 2 for _ in range(20))
+    flat = torch.zeros(50, dtype=torch.float64)
+    draws = {typical(flat, 1.0, 0.8, generator=g) for _ in range(200)}
+    assert len(draws) > 10 and all(0 <= d < 50 for d in draws)
+    assert typical(logits, 0.5, 0.95, generator=g) in range(5)
+
+
+def test_token_id_tokenizer_round_trip():
+    t = TokenIds()
+    assert t.encode("3 4 5") == [3, 4, 5] and t.decode([3, 4, 5]) == "3 4 5" and t.encode([1, 2]) == [1, 2]
+
+
+def test_rwkv_rejects_unknown_modes_and_files():
+    with pytest.raises(ValueError):
+        RWKV("model.pth", mode="jax")
+    with pytest.raises(ValueError):
+        RWKV("model.onnx")
+    with pytest.raises(TypeError):
+        RWKV({}, strategy="cuda fp16")
