@@ -1,0 +1,325 @@
+#!/usr/bin/env python3
+"""Generates rwkv_decode_back.inc: the weight-streaming ("back") waves of the single-token kernel,
+written out instruction by instruction for each supported width.
+
+    python gen_decode_back.py > rwkv_decode_back.inc
+
+Why this is not C++: the ring of in-flight weight blocks has to live in a FIXED set of registers
+that are reloaded in place, and the waits on it have to be counted by hand (loads of one wave return
+in order).  Left to the register allocator every refill gets registers of its own, the ring needs
+twice the space and spills; a spilled or copied in-flight register is silent corruption.  So the
+whole back-wave program is one asm statement with its own register map; it talks to the compiled
+front waves only through LDS and workgroup barriers.
+
+Stream of one back wave (wave wb of 8) of workgroup g, in units of 1 KiB blocks ("positions"):
+  per layer 13 jobs x KW blocks (job = one 16-column tile of a C-row matrix, or a quarter of the
+  F-row ffn value tile; wave wb owns blocks wb, wb+8, ... of the job), padded to PP positions, a
+  multiple of the ring size R, then the head tiles g, g+G, ... .  Position p lives in ring slot
+  p % R.  At every position: wait until at most R-1 loads are outstanding (then the slot's block has
+  landed), multiply, reload the slot with position p+R.  Every position issues exactly one load -
+  padding positions and positions past the end of the head load a block that stays hot in L2 - so
+  the wait count is the same everywhere.
+
+Register map (VGPR; v0..v3 are left to the compiler): v4 A-operand address (C-row digit sets), v5
+same for the F-row set, v6 park address, v7 abort-flag address, v8..v15 byte offset of block b
+inside a job, v16..v23 two accumulators, v24..v35 three A-operand buffers, v[RB..NV-1] the ring (NV = the workgroup's VGPR budget).
+SGPR: s36..s61 job base addresses of the current layer (13 pairs), s64..s89 of the next layer,
+s90..s99 scalars, vcc as a scratch pair.
+"""
+import math
+import sys
+
+V_APC, V_APF, V_PARK, V_FLAG, V_OFF, V_D, V_A = 4, 5, 6, 7, 8, 16, 24
+NA = 3            # A-operand buffers
+S_CUR, S_NXT = 36, 64
+S_L, S_T, S_JT, S_TILE, S_RT, S_RP, S_CNT, S_PAR = 90, 91, 92, 94, 95, 96, 98, 99
+NS = 4            # head tiles per barrier round (two rounds of park slots in LDS)
+PF = NA - 1       # A-operand reads run this many positions ahead
+
+
+class Emit:
+    def __init__(self):
+        self.lines = []
+        self.issued = 0          # LDS operations issued since the last full drain
+        self.ridx = [0] * NA      # issue index of the read into A buffer k
+
+    def __call__(self, s):
+        self.lines.append(s)
+
+    def drain_state(self):
+        self.issued = 0
+
+
+def gen(KW, R, NV):
+    C = 512 * KW
+    F = 4 * C
+    PS, PSF = C + 64, F + 64
+    G = 32 * KW
+    NREAL = 13 * KW
+    PP = (NREAL + R - 1) // R * R
+    RB = NV - 4 * R
+    assert RB >= V_A + 4 * NA, "ring does not fit"
+    assert R <= NREAL and R - 1 <= 63
+    TB = 8 * KW * 1024
+    DIG = max(12 * PS, 4 * PSF)
+    RED = DIG                                 # byte offset of the parked tiles from the start of LDS
+    RED_SLOTS = max(5, 2 * NS)
+    FLAG = RED + RED_SLOTS * 2048 + 32 * 8 + 32 * 8 + 2 * 4   # FLAG_ABORT word
+    LH = R * KW // math.gcd(R, KW)
+    e = Emit()
+
+    def ring(slot):
+        return f"v[{RB + 4 * slot}:{RB + 4 * slot + 3}]"
+
+    def abuf(q):
+        k = q % NA
+        return f"v[{V_A + 4 * k}:{V_A + 4 * k + 3}]"
+
+    def aread(q_layer_pos=None, head_b=None):
+        """Issue the A-operand read of a layer position (or of block head_b of a head tile)."""
+        if head_b is not None:
+            base, off, k = V_APC, 512 * head_b, head_b % NA
+        else:
+            q = q_layer_pos
+            j, b = divmod(q, KW)
+            if j <= 2:
+                base, off = V_APC, j * 4 * PS + 512 * b
+            elif j == 3:
+                base, off = V_APC, 512 * b
+            elif j == 4:
+                base, off = V_APC, 4 * PS + 512 * b
+            elif j <= 8:
+                base, off = V_APC, 512 * b
+            else:
+                base, off = V_APF, (j - 9) * C + 512 * b
+            k = q % NA
+        assert off < 65536
+        e(f"ds_read_b128 v[{V_A + 4 * k}:{V_A + 4 * k + 3}], v{base} offset:{off}")
+        e.ridx[k] = e.issued
+        e.issued += 1
+
+    def bar_check():
+        e("s_waitcnt lgkmcnt(0)")
+        e("s_barrier")
+        e(f"ds_read_b32 v{V_A}, v{V_FLAG}")
+        e("s_waitcnt lgkmcnt(0)")
+        e(f"v_readfirstlane_b32 s{S_T}, v{V_A}")
+        e(f"s_cmp_lg_u32 s{S_T}, 0")
+        e("s_cbranch_scc1 9f")
+        e.drain_state()
+
+    def park_static(dreg, slot):
+        e("s_nop 7"); e("s_nop 7"); e("s_nop 7")
+        e("s_mov_b64 exec, 0xffff")
+        e(f"ds_write_b128 v{V_PARK}, v[{dreg}:{dreg + 3}] offset:{slot * 2048}")
+        e("s_mov_b64 exec, -1")
+        e.issued += 1
+
+    # ------------------------------------------------------------------ prologue
+    e("s_mov_b64 exec, -1")
+    e(f"v_mbcnt_lo_u32_b32 v{V_A}, -1, 0")
+    e(f"v_mbcnt_hi_u32_b32 v{V_A}, -1, v{V_A}")                 # lane
+    e(f"v_and_b32 v{V_A + 1}, 3, v{V_A}")                      # n & 3
+    e(f"v_lshrrev_b32 v{V_A + 2}, 4, v{V_A}")
+    e(f"v_lshlrev_b32 v{V_A + 2}, 4, v{V_A + 2}")              # 16 * g4
+    e(f"s_lshl_b32 s{S_T}, %[wb], 6")
+    e(f"s_add_u32 s{S_T}, s{S_T}, %[lds]")
+    e(f"v_mov_b32 v{V_A + 3}, {PS}")
+    e(f"v_mul_u32_u24 v{V_APC}, v{V_A + 1}, v{V_A + 3}")
+    e(f"v_add3_u32 v{V_APC}, v{V_APC}, v{V_A + 2}, s{S_T}")
+    e(f"v_mov_b32 v{V_A + 3}, {PSF}")
+    e(f"v_mul_u32_u24 v{V_APF}, v{V_A + 1}, v{V_A + 3}")
+    e(f"v_add3_u32 v{V_APF}, v{V_APF}, v{V_A + 2}, s{S_T}")
+    e(f"s_lshl_b32 s{S_T}, %[wb], 8")
+    e(f"s_add_u32 s{S_T}, s{S_T}, %[lds]")
+    e(f"s_add_u32 s{S_T}, s{S_T}, {RED}")
+    e(f"v_lshlrev_b32 v{V_PARK}, 4, v{V_A}")
+    e(f"v_add_u32 v{V_PARK}, s{S_T}, v{V_PARK}")
+    e(f"s_add_u32 s{S_T}, %[lds], {FLAG}")
+    e(f"v_mov_b32 v{V_FLAG}, s{S_T}")
+    e(f"s_lshl_b32 s{S_T}, %[wb], 10")
+    e(f"v_lshlrev_b32 v{V_OFF}, 4, v{V_A}")
+    e(f"v_add_u32 v{V_OFF}, s{S_T}, v{V_OFF}")
+    for b in range(1, KW):
+        e(f"v_add_u32 v{V_OFF + b}, {8192 * b}, v{V_OFF}")
+    e(f"s_mov_b64 s[{S_JT}:{S_JT + 1}], %[jt]")
+    e(f"s_mov_b32 s{S_L}, %[L]")
+    for base, off in ((S_CUR, 0), (S_NXT, 128)):
+        e(f"s_load_dwordx16 s[{base}:{base + 15}], s[{S_JT}:{S_JT + 1}], {off}")
+        e(f"s_load_dwordx8 s[{base + 16}:{base + 23}], s[{S_JT}:{S_JT + 1}], {off + 64}")
+        e(f"s_load_dwordx2 s[{base + 24}:{base + 25}], s[{S_JT}:{S_JT + 1}], {off + 96}")
+    e("s_waitcnt lgkmcnt(0)")
+    for p in range(R):
+        j, b = divmod(p, KW)
+        e(f"global_load_dwordx4 {ring(p)}, v{V_OFF + b}, s[{S_CUR + 2 * j}:{S_CUR + 2 * j + 1}]")
+
+    # ------------------------------------------------------------------ layers
+    phase_start = {0: 2, 3 * KW: 1, 4 * KW: 2, 9 * KW: 1}       # position -> barriers before it
+    def phase_end(p):
+        for pe in (3 * KW, 4 * KW, 9 * KW, 13 * KW):
+            if p < pe:
+                return pe
+        return None
+
+    e("1:")
+    for p in range(PP):
+        slot = p % R
+        if p < NREAL:
+            j, b = divmod(p, KW)
+            pe = phase_end(p)
+            if p in phase_start:
+                for _ in range(phase_start[p]):
+                    bar_check()
+                for q in range(p, min(p + PF, pe)):
+                    aread(q)
+            if p + PF < pe:
+                aread(p + PF)
+            allow = e.issued - 1 - e.ridx[p % NA]
+            assert 0 <= allow <= 15
+            e(f"s_waitcnt vmcnt({R - 1}) lgkmcnt({allow})")
+            dreg = V_D + 4 * (1 if j >= 9 else j % 2)
+            first = (b == 0) and not (j > 9)
+            acc = "0" if first else f"v[{dreg}:{dreg + 3}]"
+            e(f"v_mfma_i32_16x16x64_i8 v[{dreg}:{dreg + 3}], {abuf(p)}, {ring(slot)}, {acc}")
+        else:
+            e(f"s_waitcnt vmcnt({R - 1})")
+        # reload the slot with position p + R
+        q = p + R
+        sset = S_CUR
+        if q >= PP:
+            q -= PP
+            sset = S_NXT
+        if q >= NREAL:
+            e(f"global_load_dwordx4 {ring(slot)}, v{V_OFF}, %[wh]")
+        else:
+            jq, bq = divmod(q, KW)
+            e(f"global_load_dwordx4 {ring(slot)}, v{V_OFF + bq}, s[{sset + 2 * jq}:{sset + 2 * jq + 1}]")
+        if p < NREAL:
+            if b == KW - 1 and (j < 9 or j == 12):
+                pslot = j if j <= 2 else (0 if j == 3 else (j - 4 if j <= 8 else 0))
+                park_static(dreg, pslot)
+            if p + 1 == pe:
+                e("s_waitcnt lgkmcnt(0)")
+                e("s_barrier")
+                e.drain_state()
+    # end of layer: next layer's addresses become current; fetch the layer after
+    e(f"s_add_u32 s{S_JT}, s{S_JT}, 128")
+    e(f"s_addc_u32 s{S_JT + 1}, s{S_JT + 1}, 0")
+    for i in range(13):
+        e(f"s_mov_b64 s[{S_CUR + 2 * i}:{S_CUR + 2 * i + 1}], s[{S_NXT + 2 * i}:{S_NXT + 2 * i + 1}]")
+    e(f"s_sub_u32 s{S_L}, s{S_L}, 1")
+    e(f"s_cmp_eq_u32 s{S_L}, 0")
+    e("s_cbranch_scc1 2f")
+    e(f"s_load_dwordx16 s[{S_NXT}:{S_NXT + 15}], s[{S_JT}:{S_JT + 1}], 128")
+    e(f"s_load_dwordx8 s[{S_NXT + 16}:{S_NXT + 23}], s[{S_JT}:{S_JT + 1}], 192")
+    e(f"s_load_dwordx2 s[{S_NXT + 24}:{S_NXT + 25}], s[{S_JT}:{S_JT + 1}], 224")
+    e("s_branch 1b")
+
+    # ------------------------------------------------------------------ head
+    def head_ptr():
+        """s[S_RP] = address of head tile g + G * s[S_RT], or of tile 0 when that is past the end."""
+        e(f"s_mul_i32 vcc_lo, s{S_RT}, {G}")
+        e(f"s_add_u32 vcc_lo, vcc_lo, %[g]")
+        e(f"s_cmp_ge_u32 vcc_lo, %[vt]")
+        e(f"s_cselect_b32 vcc_lo, 0, vcc_lo")
+        e(f"s_mul_hi_u32 vcc_hi, vcc_lo, {TB}")
+        e(f"s_mul_i32 vcc_lo, vcc_lo, {TB}")
+        e(f"s_add_u32 s{S_RP}, %[whlo], vcc_lo")
+        e(f"s_addc_u32 s{S_RP + 1}, %[whhi], vcc_hi")
+
+    e("2:")
+    bar_check()
+    bar_check()
+    e(f"s_mov_b32 s{S_TILE}, 0")
+    e(f"s_mov_b32 s{S_CNT}, 0")
+    e(f"s_mov_b32 s{S_PAR}, 0")
+    e(f"s_mov_b32 s{S_RT}, {R // KW - (1 if R % KW == 0 else 0)}")
+    head_ptr()
+    e("3:")
+    for q in range(LH):
+        slot = q % R
+        tq, b = divmod(q, KW)
+        dreg = V_D + 4 * (tq % 2)
+        if b == 0:
+            e(f"s_cmp_ge_u32 s{S_TILE}, %[hr]")
+            e("s_cbranch_scc1 8f")
+            e.drain_state()               # the tile before ended with a park and, at most, a barrier
+            e("s_waitcnt lgkmcnt(0)")
+            for bb in range(min(PF, KW)):
+                aread(head_b=bb)
+        if b + PF < KW:
+            aread(head_b=b + PF)
+        allow = e.issued - 1 - e.ridx[b % NA]
+        assert 0 <= allow <= 15
+        e(f"s_waitcnt vmcnt({R - 1}) lgkmcnt({allow})")
+        acc = "0" if b == 0 else f"v[{dreg}:{dreg + 3}]"
+        e(f"v_mfma_i32_16x16x64_i8 v[{dreg}:{dreg + 3}], v[{V_A + 4 * (b % NA)}:{V_A + 4 * (b % NA) + 3}], {ring(slot)}, {acc}")
+        rb = (q + R) % KW
+        if rb == 0:
+            e(f"s_add_u32 s{S_RT}, s{S_RT}, 1")
+            head_ptr()
+        e(f"global_load_dwordx4 {ring(slot)}, v{V_OFF + rb}, s[{S_RP}:{S_RP + 1}]")
+        if b == KW - 1:
+            e("s_nop 7"); e("s_nop 7"); e("s_nop 7")
+            e(f"s_add_u32 s{S_T}, s{S_CNT}, s{S_PAR}")
+            e(f"s_lshl_b32 s{S_T}, s{S_T}, 11")
+            e(f"v_add_u32 v{V_A}, s{S_T}, v{V_PARK}")
+            e("s_mov_b64 exec, 0xffff")
+            e(f"ds_write_b128 v{V_A}, v[{dreg}:{dreg + 3}]")
+            e("s_mov_b64 exec, -1")
+            e(f"s_add_u32 s{S_TILE}, s{S_TILE}, 1")
+            e(f"s_add_u32 s{S_CNT}, s{S_CNT}, 1")
+            e(f"s_cmp_eq_u32 s{S_CNT}, {NS}")
+            e("s_cbranch_scc0 7f")
+            e("s_waitcnt lgkmcnt(0)")
+            e("s_barrier")
+            e(f"s_mov_b32 s{S_CNT}, 0")
+            e(f"s_xor_b32 s{S_PAR}, s{S_PAR}, {NS}")
+            e("7:")
+    e("s_branch 3b")
+    e("8:")
+    e(f"s_cmp_eq_u32 s{S_CNT}, 0")
+    e("s_cbranch_scc1 9f")
+    e("s_waitcnt lgkmcnt(0)")
+    e("s_barrier")
+    e("9:")
+    return e.lines, dict(KW=KW, R=R, PP=PP, RB=RB, RED=RED, FLAG=FLAG, RED_SLOTS=RED_SLOTS)
+
+
+# (KW, front waves, ring size): 4 front waves -> 12 waves per workgroup, 168 VGPRs each;
+# 8 front waves -> 16 waves, 128 VGPRs each.
+CONFIGS = [(2, 4, 26), (4, 4, 26), (5, 4, 33), (8, 4, 26),
+           (2, 8, 13), (4, 8, 13), (5, 8, 22), (8, 8, 13)]
+
+
+def main():
+    out = []
+    w = out.append
+    w("// Generated by gen_decode_back.py - do not edit.  One asm statement per kernel width: the program")
+    w("// of a weight-streaming wave of the single-token kernel (see the generator for the register map).")
+    w(f"constexpr int kBackHeadSlots = {NS};   // head tiles parked per barrier round")
+    w("template <int KW, int FW> struct BackCfg;")
+    for KW, FW, R in CONFIGS:
+        NV = 168 if FW == 4 else 128
+        clob = ", ".join(f'"v{i}"' for i in range(V_APC, NV)) + ", " + ", ".join(f'"s{i}"' for i in range(S_CUR, 100))
+        lines, info = gen(KW, R, NV)
+        w(f"template <> struct BackCfg<{KW}, {FW}> {{")
+        w(f"    static constexpr int R = {R}, RED = {info['RED']}, FLAG = {info['FLAG']}, RED_SLOTS = {info['RED_SLOTS']};")
+        w("    static __device__ __forceinline__ void run(const unsigned long long *jt, const uint8_t *wh, int L, int hr, int vt,")
+        w("                                                int g, int wb, unsigned lds) {")
+        w("        const unsigned whlo = (unsigned)(unsigned long long)(uintptr_t)wh;")
+        w("        const unsigned whhi = (unsigned)((unsigned long long)(uintptr_t)wh >> 32);")
+        w("        asm volatile(")
+        for ln in lines:
+            w(f'            "{ln}\\n"')
+        w('            :')
+        w('            : [jt] "s"(jt), [wh] "s"(wh), [whlo] "s"(whlo), [whhi] "s"(whhi), [L] "s"(L), [hr] "s"(hr), [vt] "s"(vt),')
+        w('              [g] "s"(g), [wb] "s"(wb), [lds] "s"(lds)')
+        w(f'            : "memory", "scc", "vcc", {clob});')
+        w("    }")
+        w("};")
+    sys.stdout.write("\n".join(out) + "\n")
+
+
+if __name__ == "__main__":
+    main()

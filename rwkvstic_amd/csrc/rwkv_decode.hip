@@ -1,52 +1,78 @@
 // Persistent single-token kernel for the FASTQUANT RWKV-4 forward path
 // (reference agnostic/backends/opt.py:61-76, modules/block.py:56-102 at T == 1).
 //
-// One launch = one token through every layer and the head.  The grid is
-// C/16 workgroups of 512 threads, all resident at once; workgroup g owns the
-// 16 channels [16g, 16g+16) for the whole token (their residual value, WKV
-// state and receptance gate live in its registers) and the matching 16-column
-// tiles of every matrix.
+// One launch of decode_kernel = one token through every layer and the head; a
+// small launch of prep_kernel before it turns the token and the shift state
+// into the per-token constants.  The grid is C/16 workgroups, all resident at
+// once; workgroup g owns the 16 channels [16g, 16g+16) for the whole token
+// (their residual value, WKV state and receptance gate live in registers of
+// its first wave) and the matching 16-column tiles of every matrix.
 //
-// Dot products.  A matrix-vector product needs every input for every output,
-// so each of the 4 products per layer is a chip-wide dependency.  Weights are
-// streamed as 1 KiB blocks of 16 columns x 64 rows (layout "M16", stored as
-// code - 128) straight into v_mfma_i32_16x16x64_i8 as the B operand.  The
-// activation vector fp32(x * range) is rewritten once per phase as 32-bit
-// fixed point q = round(xs / S), S a power of two with |q| <= 2^30, split into
-// four signed base-256 digits; the digits are the A operand (rows 0..3), so a
-// single instruction yields the four digit sums of 16 columns over 64 rows.
-// Everything is integer: the result S * (sum_d 256^(3-d) D_d + 128 sum q) is
-// independent of summation order (deterministic) and differs from the
-// float32 sum over the same fp32(x * range) only by the |xs - S q| <= S/2
-// representation error, which is below one float32 ulp of the largest input.
+// Dot products.  Weights are streamed as 1 KiB blocks of 16 columns x 64 rows
+// (layout "M16", stored as code - 128) straight into v_mfma_i32_16x16x64_i8 as
+// the B operand.  The activation vector xs = fp32(x * range) is rewritten once
+// per product as 32-bit fixed point q = round(xs / S), S a power of two with
+// |q| <= 2^30, split into four base-256 digits; the digits are the A operand
+// (rows 0..3), so one instruction yields the four digit sums of 16 columns
+// over 64 rows.  The sums are integers: the matrix term
+// S * sum_c q_c (code_c - 128) is independent of summation order.  The rest of
+// the product, sum_c v_c (offset_c + 128 range_c) with v the unrounded input,
+// is a float64 dot product that does not depend on the output column; it is
+// computed once by the workgroups that own the channels and travels with the
+// activations.
 //
-// Exchange.  Cross-workgroup vectors (residual, wkv*r, relu^2) travel as
-// 8-byte words {epoch : 32, float32 payload : 32} written and polled with
+// Exchange.  Each of the 4 products per layer needs every channel, so each is
+// a chip-wide dependency.  Vectors travel as 8-byte words
+// {epoch : 32, float32 payload : 32} written and polled with relaxed
 // agent-scope atomics; a consumer spins until every word it needs carries the
-// epoch of the producing phase.  There is no grid barrier and no cache
-// flush.  A buffer is rewritten only after every workgroup has consumed the
-// previous contents (each rewrite is downstream of a phase that needed all
-// workgroups' outputs of the phase that read it).
+// epoch of the producing phase.  There is no grid barrier and no cache flush.
+// A buffer is rewritten only after every workgroup has consumed the previous
+// contents (each rewrite is downstream of a phase that needed all workgroups'
+// outputs of the phase that read it).  Every wait is bounded and raises an
+// abort flag that all workgroups observe, so the grid always drains.
 //
-// Weight stream.  The order in which a workgroup needs its weight blocks is
-// fixed, so each wave keeps a ring of R jobs (one job = its share of a
-// 16-column x C-row tile) in registers and refills a slot right after using
-// it: the loads for the next ~R jobs are in flight while the workgroup waits
-// for its inputs, which is what hides the exchange latency behind HBM time.
+// Roles.  Vector loads of one wave return in order, so a wave that polls would
+// first drain whatever it had prefetched.  The workgroup is therefore split:
+// "front" waves talk to the other workgroups, do the per-channel arithmetic
+// and write the digit planes to LDS; 8 "back" waves own the weight stream: each
+// keeps a ring of RJ jobs (one job = its share of a 16-column x C-row tile) in
+// registers, refills a slot right after the matrix instruction consumed it and
+// never waits on anything but LDS barriers, so several phases' worth of weight
+// loads stay in flight while the front waves wait for the other workgroups.
 #include "rwkv_decode.h"
+
+#include <type_traits>
+#include <vector>
 
 namespace rwkv {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 
-constexpr int kDT = 512;   // threads per workgroup
-constexpr int kDW = 8;     // waves per workgroup
-constexpr int kJobsPerLayer = 15;   // 13 real jobs padded to a multiple of the ring depth (3 or 5)
-constexpr int kMaxJobsPerPhase = 5;
-constexpr unsigned kSpinLimit = 1u << 21;
+constexpr int kBW = 8;                 // back (streaming) waves per workgroup
+constexpr int kRealJobs = 13;          // tile jobs per layer: k v r | o | ffn_r, 4 x ffn_k | 4 quarters of ffn_v
+constexpr unsigned kSpinLimit = 1u << 20;
+constexpr int kLnRows = 2 + 3 * 3;     // rows of the XR record table
 
-#define ALOAD(p) __hip_atomic_load((p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-#define ASTORE(p, v) __hip_atomic_store((p), (v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+// LDS flag words
+enum { FLAG_ARRIVED = 0, FLAG_SCALE = 1, FLAG_ABORT = 2, FLAG_COUNT = 4 };
+
+// Pointers that were themselves loaded from memory are "flat" to the compiler, and a flat load
+// counts against the LDS counter as well as the vector-memory counter: every wait for an LDS read
+// would then also wait for every weight load in flight.  All global accesses therefore go through
+// explicit global-address-space pointers, and the LDS flag words through LDS-address-space ones.
+#define RWKV_GLOBAL __attribute__((address_space(1)))
+#define RWKV_LDS __attribute__((address_space(3)))
+typedef RWKV_LDS volatile int lds_flag_t;
+
+template <typename T>
+__device__ __forceinline__ T gld(const T *p) { return *(const RWKV_GLOBAL T *)p; }
+template <typename T>
+__device__ __forceinline__ void gst(T *p, T v) { *(RWKV_GLOBAL T *)p = v; }
+
+#define ALOAD(p) __hip_atomic_load((RWKV_GLOBAL u64 *)(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define ASTORE(p, v) __hip_atomic_store((RWKV_GLOBAL u64 *)(p), (u64)(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define ALOAD32(p) __hip_atomic_load((RWKV_GLOBAL unsigned *)(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define ASTORE32(p, v) __hip_atomic_store((RWKV_GLOBAL unsigned *)(p), (unsigned)(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
 
 struct DArgs {
     DModel m;
@@ -57,85 +83,72 @@ struct DArgs {
     double *logits;
 };
 
-// ---- workgroup reductions (512 threads, fixed order) -----------------------
-template <int N>
-__device__ __forceinline__ void wg_sum(double (&v)[N], double *scr) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-        const double s = wave_sum(v[i]);
-        if (lane == 0) scr[i * kDW + wave] = s;
-    }
-    __syncthreads();
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-        double s = 0.0;
-#pragma unroll
-        for (int w = 0; w < kDW; ++w) s += scr[i * kDW + w];
-        v[i] = s;
-    }
-    __syncthreads();
-}
+// ---- the back (weight-streaming) waves ------------------------------------------
+// Their program is generated (gen_decode_back.py -> rwkv_decode_back.inc): one asm statement with
+// its own register map, so that the ring of in-flight weight blocks sits in fixed registers that
+// are reloaded in place.  It meets the compiled front waves only at LDS and workgroup barriers.
+#include "rwkv_decode_back.inc"
 
-template <int N>
-__device__ __forceinline__ void wg_max(float (&v)[N], float *scr) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-        float s = v[i];
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) s = fmaxf(s, __shfl_xor(s, off, 64));
-        if (lane == 0) scr[i * kDW + wave] = s;
-    }
-    __syncthreads();
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-        float s = scr[i * kDW];
-#pragma unroll
-        for (int w = 1; w < kDW; ++w) s = fmaxf(s, scr[i * kDW + w]);
-        v[i] = s;
-    }
-    __syncthreads();
+// ---- cross-lane reductions (DPP, fixed order) --------------------------------
+template <int CTRL>
+__device__ __forceinline__ int dpp_i(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false); }
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) { return __int_as_float(dpp_i<CTRL>(__float_as_int(v))); }
+template <int CTRL>
+__device__ __forceinline__ double dpp_d(double v) {
+    return __hiloint2double(dpp_i<CTRL>(__double2hiint(v)), dpp_i<CTRL>(__double2loint(v)));
 }
-
-// Per-wave partial sums parked in LDS; the epilogue adds the 8 partials in order.
-template <int N>
-__device__ __forceinline__ void park_partials(const double (&v)[N], double *part /*[kDW][8]*/, int base) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-        const double s = wave_sum(v[i]);
-        if (lane == 0) part[wave * 8 + base + i] = s;
-    }
+__device__ __forceinline__ double readlane_d(double v, int lane) {
+    return __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(v), lane),
+                            __builtin_amdgcn_readlane(__double2loint(v), lane));
 }
-__device__ __forceinline__ double sum_partials(const double *part, int idx) {
-    double s = 0.0;
-#pragma unroll
-    for (int w = 0; w < kDW; ++w) s += part[w * 8 + idx];
-    return s;
+// Sum / maximum over the 16 lanes of a DPP row (all 16 must be active); every lane gets the result.
+__device__ __forceinline__ double row16_sum(double v) {
+    v += dpp_d<0xB1>(v); v += dpp_d<0x4E>(v); v += dpp_d<0x141>(v); v += dpp_d<0x140>(v);
+    return v;
+}
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, dpp_f<0xB1>(v)); v = fmaxf(v, dpp_f<0x4E>(v));
+    v = fmaxf(v, dpp_f<0x141>(v)); v = fmaxf(v, dpp_f<0x140>(v));
+    return v;
+}
+// Over all 64 lanes (all active); the result is wave-uniform.
+__device__ __forceinline__ double wave_sum_dpp(double v) {
+    v = row16_sum(v);
+    return (readlane_d(v, 0) + readlane_d(v, 16)) + (readlane_d(v, 32) + readlane_d(v, 48));
+}
+__device__ __forceinline__ float wave_max_dpp(float v) {
+    v = row16_max(v);
+    const int i = __float_as_int(v);
+    return fmaxf(fmaxf(__int_as_float(__builtin_amdgcn_readlane(i, 0)), __int_as_float(__builtin_amdgcn_readlane(i, 16))),
+                 fmaxf(__int_as_float(__builtin_amdgcn_readlane(i, 32)), __int_as_float(__builtin_amdgcn_readlane(i, 48))));
 }
 
 // ---- fixed-point digits ------------------------------------------------------
-__device__ __forceinline__ void scale_from_amax(float amax, double &S, double &invS) {
-    if (!(amax > 0.f) || !(amax < INFINITY)) { S = 0.0; invS = 0.0; return; }
+// Scale for a vector with |xs| <= amax: S = 2^(e-30) with 2^e > amax.  Below 2^-90 the whole vector
+// is treated as zero (its products are far under any float32 ulp that matters here and 2^(30-e)
+// would leave the float range).
+__device__ __forceinline__ void scale_from_amax(float amax, double &S, float &invS) {
+    if (!(amax > 0x1p-90f) || !(amax < INFINITY)) { S = 0.0; invS = 0.f; return; }
     int e;
     frexpf(amax, &e);                 // amax = f * 2^e, f in [0.5, 1)  =>  |xs| < 2^e
     S = ldexp(1.0, e - 30);
-    invS = ldexp(1.0, 30 - e);
+    invS = ldexpf(1.f, 30 - e);
 }
 
-// q = round(xs / S) as four signed base-256 digits, most significant in plane 0.
-__device__ __forceinline__ double put_digits(signed char *dig, int plane_stride, int idx, float xs, double invS) {
-    int q = __double2int_rn((double)xs * invS);
-    const double qd = (double)q;
-    const int d3 = (int)(signed char)(q & 0xff); q = (q - d3) >> 8;
-    const int d2 = (int)(signed char)(q & 0xff); q = (q - d2) >> 8;
-    const int d1 = (int)(signed char)(q & 0xff); q = (q - d1) >> 8;
-    dig[idx] = (signed char)q;
-    dig[plane_stride + idx] = (signed char)d1;
-    dig[2 * plane_stride + idx] = (signed char)d2;
-    dig[3 * plane_stride + idx] = (signed char)d3;
-    return qd;
+// Four consecutive channels' q -> one dword per digit plane (4x4 byte transpose).  The three low
+// bytes are stored XOR 0x80, i.e. as the signed bytes b - 128; the top byte is signed as it is:
+//   q = sum_k s_k 256^k + 0x808080.
+__device__ __forceinline__ void write_digits4(signed char *dig, int plane_stride, int idx4, int q0, int q1, int q2, int q3) {
+    const unsigned u0 = (unsigned)q0 ^ 0x00808080u, u1 = (unsigned)q1 ^ 0x00808080u;
+    const unsigned u2 = (unsigned)q2 ^ 0x00808080u, u3 = (unsigned)q3 ^ 0x00808080u;
+    const unsigned x0 = __builtin_amdgcn_perm(u1, u0, 0x05010400u), x1 = __builtin_amdgcn_perm(u1, u0, 0x07030602u);
+    const unsigned y0 = __builtin_amdgcn_perm(u3, u2, 0x05010400u), y1 = __builtin_amdgcn_perm(u3, u2, 0x07030602u);
+    unsigned *d = reinterpret_cast<unsigned *>(dig + idx4);
+    d[0] = __builtin_amdgcn_perm(y1, x1, 0x07060302u);                          // most significant byte
+    d[plane_stride / 4] = __builtin_amdgcn_perm(y1, x1, 0x05040100u);
+    d[2 * (plane_stride / 4)] = __builtin_amdgcn_perm(y0, x0, 0x07060302u);
+    d[3 * (plane_stride / 4)] = __builtin_amdgcn_perm(y0, x0, 0x05040100u);      // least significant byte
 }
 
 // ---- tagged exchange ---------------------------------------------------------
@@ -143,465 +156,809 @@ __device__ __forceinline__ void put_word(u64 *dst, unsigned epoch, float v) {
     ASTORE(dst, ((u64)epoch << 32) | (u64)__float_as_uint(v));
 }
 
-// Every thread fetches words tid, tid+512, ... ; returns false if the wait ran out
-// or another workgroup raised the abort flag.
-template <int N>
-__device__ __forceinline__ bool poll_words(const u64 *src, unsigned epoch, float (&out)[N], unsigned *abort_flag) {
-    u64 w[N];
-    unsigned pending = (N >= 32) ? 0xffffffffu : ((1u << N) - 1u);
+// Values derived from the thread index are loop invariants; the compiler would compute every
+// address and predicate that depends on them once, ahead of the layer loop, and keep hundreds of
+// registers alive (or spilled).  An empty asm makes the index opaque where a phase begins, so such
+// values are recomputed next to their use.
+__device__ __forceinline__ int opaque(int v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
+struct Front {
+    int tid, wave, lane;
+    unsigned *abort_flag;
+    lds_flag_t *flags;
+    bool ok;
+    __device__ __forceinline__ void refresh() {
+        tid = opaque((int)threadIdx.x);
+        lane = tid & 63;
+        wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    }
+    __device__ __forceinline__ void fail() {
+        ok = false;
+        flags[FLAG_ABORT] = 1;
+        ASTORE32(abort_flag, 1u);
+    }
+};
+
+// A whole wave fetches NR consecutive rows of a [rows][G] record table (lane i takes workgroups
+// i, i + 64, ...), spinning until every word carries `epoch`.  Wave-uniform control flow.
+template <int NR, int NG>
+__device__ __forceinline__ void poll_rows(Front &fx, const u64 *table, int G, int row0, unsigned epoch, float (&out)[NR][NG]) {
+    u64 w[NR][NG];
     unsigned spins = 0;
-    bool ok = true;
-    while (true) {
+    while (fx.ok) {
+        bool all = true;
 #pragma unroll
-        for (int u = 0; u < N; ++u)
-            if (pending & (1u << u)) w[u] = ALOAD(src + threadIdx.x + kDT * u);
+        for (int r = 0; r < NR; ++r)
 #pragma unroll
-        for (int u = 0; u < N; ++u)
-            if ((pending & (1u << u)) && (unsigned)(w[u] >> 32) == epoch) pending &= ~(1u << u);
-        if (!pending) break;
-        ++spins;
-        if ((spins & 255u) == 0u && (spins > kSpinLimit || ALOAD(abort_flag) != 0u)) { ok = false; break; }
+            for (int i = 0; i < NG; ++i)
+                if (fx.lane + 64 * i < G) w[r][i] = ALOAD(table + (size_t)(row0 + r) * G + fx.lane + 64 * i);
+#pragma unroll
+        for (int r = 0; r < NR; ++r)
+#pragma unroll
+            for (int i = 0; i < NG; ++i)
+                if (fx.lane + 64 * i < G) all = all && ((unsigned)(w[r][i] >> 32) == epoch);
+        if (__ballot(!all) == 0ull) break;
+        __builtin_amdgcn_s_sleep(2);
+        if ((++spins & 63u) == 0u && (spins > kSpinLimit || ALOAD32(fx.abort_flag) != 0u || fx.flags[FLAG_ABORT])) fx.fail();
     }
 #pragma unroll
-    for (int u = 0; u < N; ++u) out[u] = __uint_as_float((unsigned)w[u]);
-    return ok;
+    for (int r = 0; r < NR; ++r)
+#pragma unroll
+        for (int i = 0; i < NG; ++i)
+            out[r][i] = (fx.lane + 64 * i < G) ? __uint_as_float((unsigned)w[r][i]) : 0.f;
 }
 
-// ---- weight ring ----------------------------------------------------------------
-template <int KBW>
-__device__ __forceinline__ void load_slot(uint4 (&slot)[KBW], const uint8_t *p) {
-    if (p) {
-        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-        const uint8_t *q = p + (size_t)wave * 1024 + lane * 16;
-#pragma unroll
-        for (int b = 0; b < KBW; ++b) slot[b] = *reinterpret_cast<const uint4 *>(q + (size_t)b * (kDW * 1024));
-    }
-}
-
-// D += digits(rows koff ..) x job tile.  Wave w handles blocks w, w+8, ...
-template <int KBW>
-__device__ __forceinline__ void mfma_job(const uint4 (&slot)[KBW], const signed char *dig, int plane_stride,
-                                         int koff, v4i &D) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int n = lane & 15, g4 = lane >> 4;
-    const signed char *ap = dig + n * plane_stride + koff + 64 * wave + 16 * g4;
-#pragma unroll
-    for (int b = 0; b < KBW; ++b) {
-        v4i A = {0, 0, 0, 0};
-        if (n < 4) A = *reinterpret_cast<const v4i *>(ap + b * (64 * kDW));
-        const v4i B = {(int)slot[b].x, (int)slot[b].y, (int)slot[b].z, (int)slot[b].w};
-        D = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, B, D, 0, 0, 0);
+// Spin on an LDS sequence word written by wave 0.
+__device__ __forceinline__ void wait_flag(Front &fx, int which, int seq) {
+    unsigned spins = 0;
+    while (fx.ok && fx.flags[which] < seq) {
+        __builtin_amdgcn_s_sleep(1);
+        if ((++spins & 255u) == 0u && (spins > (kSpinLimit << 4) || fx.flags[FLAG_ABORT])) fx.fail();
     }
 }
 
-// Lanes 0..15 of every wave hold the digit sums of column `lane`; park them.
-__device__ __forceinline__ void park_tile(int *red, int j, const v4i &D) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    if (lane < 16) *reinterpret_cast<v4i *>(red + ((wave * kMaxJobsPerPhase + j) * 16 + lane) * 4) = D;
+// Thread ft of FT front threads owns quads (groups of 4 consecutive words) ft, ft + FT, ...
+template <int FT, int N>
+__device__ __forceinline__ void issue_quads(const u64 *src, int ft, int first, int nq, u64 (&w)[N][4]) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        const int qi = ft + FT * (first + i);
+        if (qi < nq) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[i][e] = ALOAD(src + 4 * (size_t)qi + e);
+        }
+    }
+}
+// Re-reads until every word of the thread's quads carries the epoch (normally the first read does).
+template <int FT, int N>
+__device__ __forceinline__ void settle_quads(Front &fx, const u64 *src, int first, int nq, unsigned epoch, u64 (&w)[N][4]) {
+    unsigned spins = 0;
+    while (fx.ok) {
+        bool all = true;
+#pragma unroll
+        for (int i = 0; i < N; ++i)
+            if (fx.tid + FT * (first + i) < nq) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) all = all && ((unsigned)(w[i][e] >> 32) == epoch);
+            }
+        if (all) break;
+        __builtin_amdgcn_s_sleep(1);
+        if ((++spins & 63u) == 0u && (spins > kSpinLimit || ALOAD32(fx.abort_flag) != 0u)) { fx.fail(); break; }
+        issue_quads<FT, N>(src, fx.tid, first, nq, w);
+    }
 }
 
-__device__ __forceinline__ double finish_col(const int *red, int j, int n, double S, double qsumS, double zp) {
+// Sum of the 8 back waves' digit sums of column n of parked tile `slot`, digits recombined.
+__device__ __forceinline__ long long tile_total(const v4i *red, int slot, int n) {
     int d0 = 0, d1 = 0, d2 = 0, d3 = 0;
 #pragma unroll
-    for (int w = 0; w < kDW; ++w) {
-        const v4i v = *reinterpret_cast<const v4i *>(red + ((w * kMaxJobsPerPhase + j) * 16 + n) * 4);
+    for (int w = 0; w < kBW; ++w) {
+        const v4i v = red[(slot * kBW + w) * 16 + n];
         d0 += v.x; d1 += v.y; d2 += v.z; d3 += v.w;
     }
-    const long long tot = ((((long long)d0 * 256 + d1) * 256 + d2) * 256) + d3;
-    // codes = (code - 128) + 128:  S * (sum (code-128) q + 128 sum q)  + zero-point term
-    return S * (double)tot + 128.0 * qsumS + zp;
+    return ((((long long)d0 * 256 + d1) * 256 + d2) * 256) + d3;
+}
+// y = S (sum_c q_c (code_c - 128)) + zp,  sum_c q_c w_c = sum_k 256^k sum_c s_k,c w_c + 0x808080 sum_c w_c
+__device__ __forceinline__ double finish_col(const v4i *red, int slot, int n, double S, int colsum, double zp) {
+    return S * (double)(tile_total(red, slot, n) + 0x808080LL * (long long)colsum) + zp;
 }
 
-// ---- LayerNorm on KBW values per thread (layernorm.py:15-20) ------------------
-template <int KBW>
-__device__ __forceinline__ void layernorm_wg(double (&v)[KBW], int C, const double *__restrict__ w,
-                                             const double *__restrict__ b, double *scr) {
-    double s[2] = {0.0, 0.0};
+// LayerNorm statistics of the 16 channels a DPP row owns, and everything a consumer of x needs that
+// is linear in x: published with x itself.  P, PO: this channel's constants for the NM products the
+// normalised vector feeds.  Called by the 16 lanes of row 0 of wave 0.
+template <int NM>
+__device__ __forceinline__ void publish_ln_input(u64 *X, u64 *XR, int G, int g, int n, unsigned epoch, double x,
+                                                 const float (&P)[NM], const double (&PO)[NM]) {
+    put_word(X + 16 * g + n, epoch, (float)x);
+    const double sx = row16_sum(x), sxx = row16_sum(x * x);
+    float val = (n == 0) ? (float)sx : (float)sxx;
 #pragma unroll
-    for (int i = 0; i < KBW; ++i) { s[0] += v[i]; s[1] += v[i] * v[i]; }
-    wg_sum<2>(s, scr);
-    const double mean = s[0] / (double)C;
-    double var = s[1] / (double)C - mean * mean;
-    if (var < 0.0) var = 0.0;
-    const double rsd = 1.0 / sqrt(var + 1e-5);
-#pragma unroll
-    for (int i = 0; i < KBW; ++i) {
-        const int c = threadIdx.x + kDT * i;
-        v[i] = w[c] * ((v[i] - mean) * rsd) + b[c];
+    for (int m = 0; m < NM; ++m) {
+        const float mx = row16_max(fabsf((float)(x * (double)P[m])));
+        const double so = row16_sum(x * PO[m]);
+        const float hi = (float)so, lo = (float)(so - (double)hi);
+        if (n == 2 + 3 * m) val = mx;
+        if (n == 3 + 3 * m) val = hi;
+        if (n == 4 + 3 * m) val = lo;
     }
+    if (n < 2 + 3 * NM) put_word(XR + (size_t)n * G + g, epoch, val);
+}
+
+// ---- owner records --------------------------------------------------------------
+// Everything the owner of 16 channels needs of one layer besides its inputs sits in one 4 KiB
+// record of 8-byte slots, built at model creation (build_ownrec_kernel) in the order below.  The
+// front threads copy the next layer's record, the three WKV state rows of the channels and the
+// layer's scalars into LDS while they wait for the matrix cores, so the epilogues read LDS instead
+// of keeping dozens of prefetched values in registers across the phases.
+enum {
+    OR_DECAY = 0, OR_FIRST, OR_LN1W, OR_LN1B, OR_LN2W, OR_LN2B, OR_OFFO,      // float64 per channel
+    OR_RNGO_CSO,     // {float32 range_o, int colsum att_o}
+    OR_CSK_CSV,      // {colsum att_k, colsum att_v}
+    OR_CSR_CSFR,     // {colsum att_r, colsum ffn_r}
+    OR_CSFV,         // {colsum ffn_v, 0}
+    OR_POFK, OR_POFR,            // PO of this layer's ffn k, r
+    OR_PF,                       // {P32 ffn k, P32 ffn r}
+    OR_PON0, OR_PON1, OR_PON2,   // PO of the next LayerNorm-fed products (next layer's att k, v, r; or the head)
+    OR_PN01, OR_PN2,             // {P32 next 0, P32 next 1}, {P32 next 2, 0}
+    OR_FIELDS
+};
+constexpr int kOrOffV = OR_FIELDS * 16;          // 64 slots: float64 offset_v of the workgroup's ffn_k columns
+constexpr int kOrRngVCs = kOrOffV + 64;          // 64 slots: {float32 range_v, int colsum ffn_k}
+constexpr int kOrStatic = kOrRngVCs + 64;        // slots that come from the static record
+constexpr int kOrState = kOrStatic;              // 48 slots: aa, bb, pp of the 16 channels (per token)
+constexpr int kOrScal = kOrState + 48;           // 16 slots: the layer's DScal, byte for byte
+constexpr int kOrSlots = 512;
+static_assert(kOrScal + 16 <= kOrSlots && sizeof(DScal) == 16 * 8, "owner record");
+
+__device__ __forceinline__ double or_d(const u64 *rec, int slot) { return __longlong_as_double((long long)rec[slot]); }
+__device__ __forceinline__ unsigned or_lo(const u64 *rec, int slot) { return (unsigned)rec[slot]; }
+__device__ __forceinline__ unsigned or_hi(const u64 *rec, int slot) { return (unsigned)(rec[slot] >> 32); }
+__device__ __forceinline__ double or_sumPO(const u64 *rec, int m) { return or_d(rec, kOrScal + m); }
+__device__ __forceinline__ double or_sumQO(const u64 *rec, int m) { return or_d(rec, kOrScal + 5 + m); }
+__device__ __forceinline__ float or_maxP(const u64 *rec, int m) { return reinterpret_cast<const float *>(rec + kOrScal)[20 + m]; }
+__device__ __forceinline__ float or_maxQ(const u64 *rec, int m) { return reinterpret_cast<const float *>(rec + kOrScal)[25 + m]; }
+
+// l == L stages the head's scalars only.
+template <int FT>
+__device__ __forceinline__ void stage_owner_record(const DArgs &a, int l, int g, int G, int C, u64 *own_lds, int tid) {
+    u64 *dst = own_lds + (l & 1) * kOrSlots;
+    const bool layer = l < a.m.L;
+#pragma unroll
+    for (int i = 0; i < kOrSlots / FT; ++i) {
+        const int t = tid + FT * i;
+        u64 v = 0;
+        if (t < kOrStatic) {
+            if (layer) v = a.m.ownrec[((size_t)l * G + g) * kOrSlots + t];
+        } else if (t < kOrScal) {
+            const int k = (t - kOrState) >> 4, n = (t - kOrState) & 15;
+            if (layer) v = (u64)__double_as_longlong(a.state[((size_t)l * 5 + 2 + k) * C + 16 * g + n]);
+        } else if (t < kOrScal + 16) {
+            v = reinterpret_cast<const u64 *>(a.m.sc + l)[t - kOrScal];
+        }
+        dst[t] = v;
+    }
+}
+
+// Scale of the fixed-point digits of LayerNorm-fed product m (index in the layer's tables: m0 + m)
+// from the statistics in `stat`:  |fp32(t P + Q)| <= rsd (max |x P| + |mean| max |P|) + max |Q|.
+__device__ __forceinline__ void ln_scale(const double *stat, const u64 *rec, int m0, int m, double &S, float &invS) {
+    const double bound = stat[1] * (stat[2 + 2 * m] + fabs(stat[0]) * (double)or_maxP(rec, m0 + m)) + (double)or_maxQ(rec, m0 + m);
+    scale_from_amax((float)(bound * 1.000001) + 1e-37f, S, invS);
+}
+// sum_c mixed_c (offset_c + 128 range_c) of that product.
+__device__ __forceinline__ double ln_zp(const double *stat, const u64 *rec, int m0, int m) {
+    return stat[1] * (stat[3 + 2 * m] - stat[0] * or_sumPO(rec, m0 + m)) + or_sumQO(rec, m0 + m);
+}
+
+// Front side of a LayerNorm-fed product group (NM matrices sharing the normalised input):
+// waits for x and its records, leaves mean, rsd and the per-product sums in stat[0..7], writes NM
+// sets of digit planes.  Contains one workgroup barrier (statistics) and ends with the "digits
+// ready" barrier.  rec: the LDS owner record of the layer (scalars).
+template <int KW, int FW, int NM>
+__device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, const float *P32, const float *Q32,
+                                         const u64 *rec, int m0, unsigned epoch, signed char *dig, double *stat,
+                                         long long *tr) {
+    constexpr int C = 512 * KW, G = 32 * KW, NG = (G + 63) / 64, FT = 64 * FW, NQ = C / 4, NQT = (NQ + FT - 1) / FT;
+    constexpr int PS = C + 64;
+    static_assert(FW >= 4, "one front wave per product plus wave 0");
+    fx.refresh();
+    // this thread's constants, requested before any waiting
+    float4 P[NQT][NM], Q[NQT][NM];
+#pragma unroll
+    for (int i = 0; i < NQT; ++i) {
+        const int qi = fx.tid + FT * i;
+        if (qi < NQ) {
+#pragma unroll
+            for (int m = 0; m < NM; ++m) {
+                P[i][m] = *reinterpret_cast<const float4 *>(P32 + (size_t)(m0 + m) * C + 4 * qi);
+                Q[i][m] = *reinterpret_cast<const float4 *>(Q32 + (size_t)(m0 + m) * C + 4 * qi);
+            }
+        }
+    }
+    ++seq;
+    u64 w[NQT][4];
+    if (fx.wave == 0) {
+        float r[2][NG];
+        poll_rows<2, NG>(fx, a.b.XR, G, 0, epoch, r);
+        if (fx.lane == 0) fx.flags[FLAG_ARRIVED] = seq;
+        issue_quads<FT, NQT>(a.b.X, fx.tid, 0, NQ, w);
+        double s0 = 0.0, s1 = 0.0;
+#pragma unroll
+        for (int i = 0; i < NG; ++i) { s0 += (double)r[0][i]; s1 += (double)r[1][i]; }
+        s0 = wave_sum_dpp(s0); s1 = wave_sum_dpp(s1);
+        const double mean = s0 * (1.0 / (double)C);
+        double var = s1 * (1.0 / (double)C) - mean * mean;
+        if (var < 0.0) var = 0.0;
+        const double rsd = 1.0 / sqrt(var + 1e-5);                 // layernorm.py:15-20
+        if (fx.lane == 0) { stat[0] = mean; stat[1] = rsd; }
+    } else {
+        wait_flag(fx, FLAG_ARRIVED, seq);
+        issue_quads<FT, NQT>(a.b.X, fx.tid, 0, NQ, w);
+        const int m = fx.wave - 1;
+        if (m < NM) {
+            float r[3][NG];
+            poll_rows<3, NG>(fx, a.b.XR, G, 2 + 3 * m, epoch, r);
+            float mx = 0.f;
+            double so = 0.0;
+#pragma unroll
+            for (int i = 0; i < NG; ++i) { mx = fmaxf(mx, r[0][i]); so += (double)r[1][i] + (double)r[2][i]; }
+            mx = wave_max_dpp(mx); so = wave_sum_dpp(so);
+            if (fx.lane == 0) { stat[2 + 2 * m] = (double)mx; stat[3 + 2 * m] = so; }
+        }
+    }
+    __syncthreads();                                               // statistics
+    if (tr) tr[0] = wall_clock64();
+    if (fx.flags[FLAG_ABORT]) { fx.ok = false; return; }
+    const double mean = stat[0], rsd = stat[1];
+    float invS[NM];
+#pragma unroll
+    for (int m = 0; m < NM; ++m) {
+        double S;
+        ln_scale(stat, rec, m0, m, S, invS[m]);
+    }
+    settle_quads<FT, NQT>(fx, a.b.X, 0, NQ, epoch, w);
+#pragma unroll
+    for (int i = 0; i < NQT; ++i) {
+        const int qi = fx.tid + FT * i;
+        if (qi < NQ) {
+            float t[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                t[e] = (float)(((double)__uint_as_float((unsigned)w[i][e]) - mean) * rsd);
+#pragma unroll
+            for (int m = 0; m < NM; ++m) {
+                const float p[4] = {P[i][m].x, P[i][m].y, P[i][m].z, P[i][m].w};
+                const float qq[4] = {Q[i][m].x, Q[i][m].y, Q[i][m].z, Q[i][m].w};
+                int q[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) q[e] = __float2int_rn(fmaf(t[e], p[e], qq[e]) * invS[m]);   // matmul.py:131
+                write_digits4(dig + m * 4 * PS, PS, 4 * qi, q[0], q[1], q[2], q[3]);
+            }
+        }
+    }
+    __syncthreads();                                               // digits ready
+    if (tr) tr[1] = wall_clock64();
+    if (fx.flags[FLAG_ABORT]) fx.ok = false;
+}
+
+// Front side of a product whose input was scaled by its producers (att output, ffn value):
+// the records carry max |xs| and the shares of the zero-point sum.  Leaves the scale in stat[16],
+// the zero-point sum in stat[18].  Ends with the "digits ready" barrier.
+template <int KW, int FW, int NQT>
+__device__ __forceinline__ void vec_front(Front &fx, int &seq, const u64 *src, const u64 *rec, int nq, unsigned epoch,
+                                          signed char *dig, int plane_stride, double *stat, long long *tr) {
+    constexpr int G = 32 * KW, NG = (G + 63) / 64, FT = 64 * FW;
+    constexpr int CH = NQT <= 5 ? NQT : 3, NCH = (NQT + CH - 1) / CH;
+    fx.refresh();
+    ++seq;
+    u64 w[NCH > 1 ? 2 : 1][CH][4];
+    float invS;
+    if (fx.wave == 0) {
+        float r[3][NG];
+        poll_rows<3, NG>(fx, rec, G, 0, epoch, r);
+        if (fx.lane == 0) fx.flags[FLAG_ARRIVED] = seq;
+        issue_quads<FT, CH>(src, fx.tid, 0, nq, w[0]);
+        float mx = 0.f;
+        double so = 0.0;
+#pragma unroll
+        for (int i = 0; i < NG; ++i) { mx = fmaxf(mx, r[0][i]); so += (double)r[1][i] + (double)r[2][i]; }
+        mx = wave_max_dpp(mx);
+        so = wave_sum_dpp(so);
+        double S;
+        scale_from_amax(mx, S, invS);
+        if (fx.lane == 0) { stat[16] = S; stat[17] = (double)invS; stat[18] = so; fx.flags[FLAG_SCALE] = seq; }
+    } else {
+        wait_flag(fx, FLAG_ARRIVED, seq);
+        issue_quads<FT, CH>(src, fx.tid, 0, nq, w[0]);
+        wait_flag(fx, FLAG_SCALE, seq);
+        invS = (float)stat[17];
+    }
+    if (tr) tr[0] = wall_clock64();
+#pragma unroll
+    for (int ch = 0; ch < NCH; ++ch) {
+        if (ch + 1 < NCH) issue_quads<FT, CH>(src, fx.tid, (ch + 1) * CH, nq, w[(ch + 1) & 1]);
+        settle_quads<FT, CH>(fx, src, ch * CH, nq, epoch, w[ch & 1]);
+#pragma unroll
+        for (int i = 0; i < CH; ++i) {
+            const int qi = fx.tid + FT * (ch * CH + i);
+            if (ch * CH + i < NQT && qi < nq) {
+                int q[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) q[e] = __float2int_rn(__uint_as_float((unsigned)w[ch & 1][i][e]) * invS);
+                write_digits4(dig, plane_stride, 4 * qi, q[0], q[1], q[2], q[3]);
+            }
+        }
+    }
+    __syncthreads();                                               // digits ready
+    if (tr) tr[1] = wall_clock64();
+    if (fx.flags[FLAG_ABORT]) fx.ok = false;
 }
 
 // =============================================================================
-template <int KBW>
-__global__ void __launch_bounds__(kDT) decode_kernel(const DArgs a) {
-    constexpr int C = KBW * kDT, F = 4 * C, NKB = C / 64;
-    constexpr int R = 3;                           // ring depth in jobs
-    constexpr int JPL = kJobsPerLayer;
-    constexpr int PS = C + 64, PSF = F + 64;        // digit plane strides (+64: conflict-free A reads)
-    constexpr size_t kTileBytes = (size_t)NKB * 1024;
-    static_assert(JPL % R == 0, "ring depth must divide the padded job count");
+template <int KW, int FW, bool TRACE>
+__device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, const v4i *red, double *stat, double *rf_lds,
+                                           lds_flag_t *flags, u64 *own_lds) {
+    constexpr int C = 512 * KW, F = 4 * C, G = 32 * KW, FT = 64 * FW;
+    constexpr int PS = C + 64, PSF = F + 64;
+    constexpr int NQH = F / 4, NQTH = (NQH + FT - 1) / FT, NQC = C / 4, NQTC = (NQC + FT - 1) / FT;
+    Front fx;
+    fx.abort_flag = a.b.abort_flag; fx.flags = flags; fx.ok = true;
+    fx.refresh();
+    const int g = blockIdx.x, L = a.m.L, V = a.m.V;
+    const bool fin = fx.wave == 0;                       // wave 0 owns the workgroup's 16 channels
+    long long *trace = (TRACE && g == 0 && threadIdx.x == 0) ? a.b.trace : nullptr;
+    int seq = 0;
+    int lane, n, row, c_own;                             // recomputed at the start of every phase
+#define RWKV_IDS() do { fx.refresh(); lane = fx.lane; n = lane & 15; row = lane >> 4; c_own = 16 * g + n; } while (0)
+    RWKV_IDS();
 
-    extern __shared__ __align__(16) unsigned char smem[];
-    constexpr int DIG_BYTES = (3 * 4 * PS > 4 * PSF) ? 3 * 4 * PS : 4 * PSF;
-    signed char *dig = reinterpret_cast<signed char *>(smem);
-    int *red = reinterpret_cast<int *>(smem + DIG_BYTES);                           // [2][8][5][16][4]
-    constexpr int RED_INTS = kDW * kMaxJobsPerPhase * 16 * 4;
-    double *part = reinterpret_cast<double *>(red + 2 * RED_INTS);                  // [2][8][8]
-    double *scr = part + 2 * kDW * 8;                                               // [4*8]
-    double *own_x = scr + 4 * kDW;                                                  // [16]
-    double *own_ln1 = own_x + 16;                                                   // [16]
-    double *own_ln2 = own_ln1 + 16;                                                 // [16]
+    stage_owner_record<FT>(a, 0, g, G, C, own_lds, fx.tid);   // read after the first barriers below
+    // the residual value of the own channels lives in LDS between the epilogues (rf_lds[16 + n])
+    double *x_lds = rf_lds + 16;
+    if (fin && row == 0) x_lds[n] = a.m.X0[c_own];
 
-    const int g = blockIdx.x, G = gridDim.x;
-    const int tid = threadIdx.x;
-    const int L = a.m.L, V = a.m.V;
-    const int v_tiles = (V + 15) / 16;
-    const int head_jobs = (((v_tiles + G - 1) / G + R - 1) / R) * R;
-    unsigned *abort_flag = a.b.abort_flag;
-
-    auto layer_job = [&](int l, int j) -> const uint8_t * {
-        const DLayer &Ly = a.m.layers[l];
-        if (j == 0) return Ly.att_k.w16 + (size_t)g * kTileBytes;
-        if (j == 1) return Ly.att_v.w16 + (size_t)g * kTileBytes;
-        if (j == 2) return Ly.att_r.w16 + (size_t)g * kTileBytes;
-        if (j == 3) return Ly.att_o.w16 + (size_t)g * kTileBytes;
-        if (j == 4) return Ly.ffn_r.w16 + (size_t)g * kTileBytes;
-        if (j <= 8) return Ly.ffn_k.w16 + (size_t)(g + G * (j - 5)) * kTileBytes;
-        if (j <= 12) return Ly.ffn_v.w16 + ((size_t)g * 4 + (j - 9)) * kTileBytes;
-        return nullptr;
-    };
-    auto head_job = [&](int hj) -> const uint8_t * {
-        const int tile = g + G * hj;
-        return (hj < head_jobs && tile < v_tiles) ? a.m.head.w16 + (size_t)tile * kTileBytes : nullptr;
-    };
-    auto flat_job = [&](int l, int j) -> const uint8_t * {   // j may run past the layer
-        if (j == 13 || j == 14) j += R;     // padding jobs own no data: their slot goes to its next user
-        if (j < JPL) return layer_job(l, j);
-        if (l + 1 < L) return layer_job(l + 1, j - JPL);
-        return head_job(j - JPL);
-    };
-
-    uint4 ring[R][KBW];
-#pragma unroll
-    for (int s = 0; s < R; ++s) load_slot<KBW>(ring[s], layer_job(0, s));
-
-    int64_t tok = a.token[0];
-    if (tok < 0) tok = 0;
-    if (tok >= V) tok = V - 1;
-
-    double x_own = 0.0;       // residual value of channel 16g + tid (threads 0..15)
-    unsigned parity = 0;      // LDS double buffering of red/part
-
-    for (int l = 0; l < L; ++l) {
-        const DLayer &Ly = a.m.layers[l];
+    for (int l = 0; l < L && fx.ok; ++l) {
+        const u64 *rec = own_lds + (l & 1) * kOrSlots;
         double *sl = a.state + (size_t)l * 5 * C;
-        const unsigned e_base = a.epoch0 + 4u * (unsigned)l;
-        const int c_own = 16 * g + tid;     // meaningful for tid < 16
-
-        // per-channel scalars the epilogues need; fetched early, off the critical path
-        double td = 0, tf = 0, st_aa = 0, st_bb = 0, st_pp = 0;
-        if (tid < 16) {
-            td = Ly.time_decay[c_own]; tf = Ly.time_first[c_own];
-            st_aa = sl[2 * (size_t)C + c_own]; st_bb = sl[3 * (size_t)C + c_own]; st_pp = sl[4 * (size_t)C + c_own];
-        }
+        const unsigned e = a.epoch0 + 4u * (unsigned)l;
+        long long *tr = trace ? trace + (size_t)l * kTraceStampsPerLayer : nullptr;
+        const float *P32 = a.m.P32 + (size_t)l * kLnMats * C, *Q32 = a.m.Q32 + (size_t)l * kLnMats * C;
+        if (tr) tr[0] = wall_clock64();
 
         // ===================== phase 1: att k, v, r ============================
-        {
-            double xv[KBW];
-            if (l == 0) {
-#pragma unroll
-                for (int i = 0; i < KBW; ++i) xv[i] = (double)a.m.emb[(size_t)tok * C + tid + kDT * i];
-                layernorm_wg<KBW>(xv, C, a.m.ln0_w, a.m.ln0_b, scr);     // opt.py:64
-#pragma unroll
-                for (int i = 0; i < KBW; ++i) {
-                    const int c = tid + kDT * i;
-                    if ((c >> 4) == g) own_x[c & 15] = xv[i];
-                }
-            } else {
-                float xf[KBW];
-                const bool ok = poll_words<KBW>(a.b.X, e_base, xf, abort_flag);
-                if (__syncthreads_or(!ok)) { if (tid == 0) ASTORE(abort_flag, 1u); return; }
-#pragma unroll
-                for (int i = 0; i < KBW; ++i) xv[i] = (double)xf[i];
-            }
-            layernorm_wg<KBW>(xv, C, Ly.ln1_w, Ly.ln1_b, scr);           // block.py:58
-            float xs[3][KBW];
-            double zq[6] = {0, 0, 0, 0, 0, 0};                            // zp[3], qsum[3]
-            float amax[3] = {0.f, 0.f, 0.f};
-            const DQ *mats[3] = {&Ly.att_k, &Ly.att_v, &Ly.att_r};
-#pragma unroll
-            for (int i = 0; i < KBW; ++i) {
-                const int c = tid + kDT * i;
-                const double xy = xv[i];
-                if ((c >> 4) == g) own_ln1[c & 15] = xy;
-                const double sh = sl[c];                                   // block.py:61-64
-#pragma unroll
-                for (int m = 0; m < 3; ++m) {
-                    const double mu = Ly.att_mix[(size_t)m * C + c];
-                    const double mixed = xy * mu + sh * (1.0 - mu);       // block.py:67
-                    xs[m][i] = (float)(mixed * (double)mats[m]->range[c]); // matmul.py:131
-                    zq[m] += mixed * mats[m]->offset[c];
-                    amax[m] = fmaxf(amax[m], fabsf(xs[m][i]));
-                }
-            }
-            wg_max<3>(amax, reinterpret_cast<float *>(scr));
-            double S[3], invS[3];
-#pragma unroll
-            for (int m = 0; m < 3; ++m) scale_from_amax(amax[m], S[m], invS[m]);
-#pragma unroll
-            for (int i = 0; i < KBW; ++i)
-#pragma unroll
-                for (int m = 0; m < 3; ++m)
-                    zq[3 + m] += put_digits(dig + m * 4 * PS, PS, tid + kDT * i, xs[m][i], invS[m]);
-            double *pp_ = part + parity * (kDW * 8);
-            park_partials<6>(zq, pp_, 0);
-            __syncthreads();
-
-            v4i D[3];
-#pragma unroll
-            for (int j = 0; j < 3; ++j) {
-                D[j] = v4i{0, 0, 0, 0};
-                mfma_job<KBW>(ring[j % R], dig + j * 4 * PS, PS, 0, D[j]);
-                load_slot<KBW>(ring[j % R], flat_job(l, j + R));
-            }
-            int *rd = red + parity * RED_INTS;
-#pragma unroll
-            for (int j = 0; j < 3; ++j) park_tile(rd, j, D[j]);
-            __syncthreads();
-            if (tid < 16) {
-                double y[3];
-#pragma unroll
-                for (int j = 0; j < 3; ++j)
-                    y[j] = finish_col(rd, j, tid, S[j], S[j] * sum_partials(pp_, 3 + j), sum_partials(pp_, j));
-                const float r = sigmoid_f32((float)y[2]);                 // block.py:72
-                float aa = (float)st_aa, bb = (float)st_bb;
-                double pp = st_pp;
-                const float wkv = wkv_step_f32(td, tf, (float)y[0], (float)y[1], aa, bb, pp);
-                put_word(a.b.A + c_own, e_base + 1u, wkv * r);            // block.py:78
+        ln_front<KW, FW, 3>(fx, seq, a, P32, Q32, rec, 0, e, dig, stat, tr ? tr + 1 : nullptr);
+        if (!fx.ok) break;
+        __syncthreads();                                                         // tile sums parked
+        if (tr) tr[3] = wall_clock64();
+        RWKV_IDS();
+        double xy1 = 0.0;
+        if (fin) {
+            const int j = row < 3 ? row : 0;
+            const int cs1 = (int)(j == 0 ? or_lo(rec, OR_CSK_CSV * 16 + n) : (j == 1 ? or_hi(rec, OR_CSK_CSV * 16 + n) : or_lo(rec, OR_CSR_CSFR * 16 + n)));
+            double Sj;
+            float invSj;
+            ln_scale(stat, rec, 0, j, Sj, invSj);
+            const double y = finish_col(red, j, n, Sj, cs1, ln_zp(stat, rec, 0, j));
+            const double yv = __shfl(y, n + 16, 64), yr = __shfl(y, n + 32, 64);
+            if (row == 0) {
+                const double td = or_d(rec, OR_DECAY * 16 + n), tf = or_d(rec, OR_FIRST * 16 + n);
+                const float r = sigmoid_f32((float)yr);                          // block.py:72
+                float aa = (float)or_d(rec, kOrState + n), bb = (float)or_d(rec, kOrState + 16 + n);
+                double pp = or_d(rec, kOrState + 32 + n);
+                const float wkv = wkv_step_f32(td, tf, (float)y, (float)yv, aa, bb, pp);
+                const double av = (double)(wkv * r);                             // block.py:78
+                const float xs = (float)(av * (double)__uint_as_float(or_lo(rec, OR_RNGO_CSO * 16 + n)));   // matmul.py:131
+                put_word(a.b.A + c_own, e + 1u, xs);
+                const float mx = row16_max(fabsf(xs));
+                const double so = row16_sum(av * or_d(rec, OR_OFFO * 16 + n) + 128.0 * (double)xs);
+                const float hi = (float)so, lo = (float)(so - (double)hi);
+                if (n < 3) put_word(a.b.AR + (size_t)n * G + g, e + 1u, n == 0 ? mx : (n == 1 ? hi : lo));
                 sl[2 * (size_t)C + c_own] = (double)aa;
                 sl[3 * (size_t)C + c_own] = (double)bb;
                 sl[4 * (size_t)C + c_own] = pp;
-                if (l == 0) x_own = own_x[tid];
+                xy1 = or_d(rec, OR_LN1W * 16 + n) * ((x_lds[n] - stat[0]) * stat[1]) + or_d(rec, OR_LN1B * 16 + n);   // block.py:58
+                sl[c_own] = xy1;                                                 // block.py:63-64
             }
-            parity ^= 1u;
         }
+        if (tr) tr[4] = wall_clock64();
 
         // ===================== phase 2: att output =============================
-        {
-            float af[KBW];
-            const bool ok = poll_words<KBW>(a.b.A, e_base + 1u, af, abort_flag);
-            if (__syncthreads_or(!ok)) { if (tid == 0) ASTORE(abort_flag, 1u); return; }
-            float xs[KBW];
-            double zq[2] = {0, 0};
-            float amax[1] = {0.f};
-#pragma unroll
-            for (int i = 0; i < KBW; ++i) {
-                const int c = tid + kDT * i;
-                const double v = (double)af[i];
-                xs[i] = (float)(v * (double)Ly.att_o.range[c]);
-                zq[0] += v * Ly.att_o.offset[c];
-                amax[0] = fmaxf(amax[0], fabsf(xs[i]));
-            }
-            wg_max<1>(amax, reinterpret_cast<float *>(scr));
-            double S, invS;
-            scale_from_amax(amax[0], S, invS);
-#pragma unroll
-            for (int i = 0; i < KBW; ++i) zq[1] += put_digits(dig, PS, tid + kDT * i, xs[i], invS);
-            double *pp_ = part + parity * (kDW * 8);
-            park_partials<2>(zq, pp_, 0);
-            __syncthreads();
-            v4i D = {0, 0, 0, 0};
-            mfma_job<KBW>(ring[3 % R], dig, PS, 0, D);
-            load_slot<KBW>(ring[3 % R], flat_job(l, 3 + R));
-            int *rd = red + parity * RED_INTS;
-            park_tile(rd, 0, D);
-            __syncthreads();
-            if (tid < 16) {
-                const double y = finish_col(rd, 0, tid, S, S * sum_partials(pp_, 1), sum_partials(pp_, 0));
-                x_own = x_own + y;                                        // block.py:80
-                put_word(a.b.X + c_own, e_base + 2u, (float)x_own);
-                sl[c_own] = own_ln1[tid];                                 // block.py:63-64
-            }
-            parity ^= 1u;
+        vec_front<KW, FW, NQTC>(fx, seq, a.b.A, a.b.AR, NQC, e + 1u, dig, PS, stat, tr ? tr + 5 : nullptr);
+        if (!fx.ok) break;
+        __syncthreads();
+        if (tr) tr[7] = wall_clock64();
+        RWKV_IDS();
+        if (fin && row == 0) {
+            const double x_own = x_lds[n] + finish_col(red, 0, n, stat[16], (int)or_hi(rec, OR_RNGO_CSO * 16 + n), stat[18]);   // block.py:80
+            x_lds[n] = x_own;
+            const float Pf[2] = {__uint_as_float(or_lo(rec, OR_PF * 16 + n)), __uint_as_float(or_hi(rec, OR_PF * 16 + n))};
+            const double POf[2] = {or_d(rec, OR_POFK * 16 + n), or_d(rec, OR_POFR * 16 + n)};
+            publish_ln_input<2>(a.b.X, a.b.XR, G, g, n, e + 2u, x_own, Pf, POf);
         }
+        if (tr) tr[8] = wall_clock64();
 
         // ===================== phase 3: ffn receptance + key ===================
-        double rf_own = 0.0;
-        {
-            float xf[KBW];
-            const bool ok = poll_words<KBW>(a.b.X, e_base + 2u, xf, abort_flag);
-            if (__syncthreads_or(!ok)) { if (tid == 0) ASTORE(abort_flag, 1u); return; }
-            double xv[KBW];
-#pragma unroll
-            for (int i = 0; i < KBW; ++i) xv[i] = (double)xf[i];
-            layernorm_wg<KBW>(xv, C, Ly.ln2_w, Ly.ln2_b, scr);           // block.py:82
-            float xs[2][KBW];
-            double zq[4] = {0, 0, 0, 0};                                  // zp k, zp r, qsum k, qsum r
-            float amax[2] = {0.f, 0.f};
-            const DQ *mats[2] = {&Ly.ffn_k, &Ly.ffn_r};
-#pragma unroll
-            for (int i = 0; i < KBW; ++i) {
-                const int c = tid + kDT * i;
-                const double dd = xv[i];
-                if ((c >> 4) == g) own_ln2[c & 15] = dd;
-                const double sh = sl[(size_t)C + c];                      // block.py:84-88
-#pragma unroll
-                for (int m = 0; m < 2; ++m) {
-                    const double mu = Ly.ffn_mix[(size_t)m * C + c];
-                    const double mixed = dd * mu + sh * (1.0 - mu);      // block.py:91
-                    xs[m][i] = (float)(mixed * (double)mats[m]->range[c]);
-                    zq[m] += mixed * mats[m]->offset[c];
-                    amax[m] = fmaxf(amax[m], fabsf(xs[m][i]));
-                }
+        ln_front<KW, FW, 2>(fx, seq, a, P32, Q32, rec, 3, e + 2u, dig, stat, tr ? tr + 9 : nullptr);   // [0] ffn_k, [1] ffn_r
+        if (!fx.ok) break;
+        RWKV_IDS();
+        stage_owner_record<FT>(a, l + 1, g, G, C, own_lds, fx.tid);   // while the matrix cores run (l + 1 == L: the head's scalars)
+        __syncthreads();
+        if (tr) tr[11] = wall_clock64();
+        if (fin) {
+            // parked tiles: 0 = ffn_r, 1..4 = ffn_k tiles g, g+G, g+2G, g+3G
+            const int f_own = 16 * (g + G * row) + n;      // column of ffn_k tile `row`
+            double Sk;
+            float invSk;
+            ln_scale(stat, rec, 3, 0, Sk, invSk);
+            const double y = finish_col(red, 1 + row, n, Sk, (int)or_hi(rec, kOrRngVCs + lane), ln_zp(stat, rec, 3, 0));
+            const double h = y > 0.0 ? y : 0.0;                                  // block.py:97-98
+            const double hh = h * h;
+            const float xs = (float)(hh * (double)__uint_as_float(or_lo(rec, kOrRngVCs + lane)));
+            put_word(a.b.H + f_own, e + 3u, xs);
+            const float mx = wave_max_dpp(fabsf(xs));
+            const double so = wave_sum_dpp(hh * or_d(rec, kOrOffV + lane) + 128.0 * (double)xs);
+            const float hi = (float)so, lo = (float)(so - (double)hi);
+            if (lane < 3) put_word(a.b.HR + (size_t)lane * G + g, e + 3u, lane == 0 ? mx : (lane == 1 ? hi : lo));
+            if (row == 0) {                                // after H is out: the receptance gate of the own channels
+                double Sr;
+                float invSr;
+                ln_scale(stat, rec, 3, 1, Sr, invSr);
+                const double yr = finish_col(red, 0, n, Sr, (int)or_hi(rec, OR_CSR_CSFR * 16 + n), ln_zp(stat, rec, 3, 1));
+                rf_lds[n] = (double)sigmoid_f32((float)yr);                      // block.py:95
+                // the LayerNorm output of the own channel is the new ffn shift state (block.py:82,87-88)
+                sl[(size_t)C + c_own] = or_d(rec, OR_LN2W * 16 + n) * ((x_lds[n] - stat[0]) * stat[1]) + or_d(rec, OR_LN2B * 16 + n);
             }
-            wg_max<2>(amax, reinterpret_cast<float *>(scr));
-            double S[2], invS[2];
-#pragma unroll
-            for (int m = 0; m < 2; ++m) scale_from_amax(amax[m], S[m], invS[m]);
-#pragma unroll
-            for (int i = 0; i < KBW; ++i)
-#pragma unroll
-                for (int m = 0; m < 2; ++m)
-                    zq[2 + m] += put_digits(dig + m * 4 * PS, PS, tid + kDT * i, xs[m][i], invS[m]);
-            double *pp_ = part + parity * (kDW * 8);
-            park_partials<4>(zq, pp_, 0);
-            __syncthreads();
-            v4i D[5];
-#pragma unroll
-            for (int jj = 0; jj < 5; ++jj) {
-                const int j = 4 + jj;                                     // job 4: ffn_r ; 5..8: ffn_k tiles
-                D[jj] = v4i{0, 0, 0, 0};
-                mfma_job<KBW>(ring[j % R], dig + (jj == 0 ? 1 : 0) * 4 * PS, PS, 0, D[jj]);
-                load_slot<KBW>(ring[j % R], flat_job(l, j + R));
-            }
-            int *rd = red + parity * RED_INTS;
-#pragma unroll
-            for (int jj = 0; jj < 5; ++jj) park_tile(rd, jj, D[jj]);
-            __syncthreads();
-            if (tid < 80) {
-                const int jj = tid >> 4, n = tid & 15;
-                const int m = jj == 0 ? 1 : 0;
-                const double y = finish_col(rd, jj, n, S[m], S[m] * sum_partials(pp_, 2 + m), sum_partials(pp_, m));
-                if (jj == 0) {
-                    rf_own = (double)sigmoid_f32((float)y);              // block.py:95
-                } else {
-                    const double h = y > 0.0 ? y : 0.0;                  // block.py:97-98
-                    put_word(a.b.H + 16 * (g + G * (jj - 1)) + n, e_base + 3u, (float)(h * h));
-                }
-            }
-            parity ^= 1u;
         }
+        if (tr) tr[12] = wall_clock64();
 
         // ===================== phase 4: ffn value ==============================
-        {
-            float hf[4 * KBW];
-            double zq[2] = {0, 0};
-            float amax[1] = {0.f};
-            bool ok = true;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {          // a quarter (C words) at a time keeps the live set small
-                float part_h[KBW];
-                ok = poll_words<KBW>(a.b.H + (size_t)q * C, e_base + 3u, part_h, abort_flag) && ok;
-#pragma unroll
-                for (int i = 0; i < KBW; ++i) {
-                    const int f = q * C + tid + kDT * i;
-                    const double h = (double)part_h[i];
-                    const float x = (float)(h * (double)Ly.ffn_v.range[f]);
-                    zq[0] += h * Ly.ffn_v.offset[f];
-                    amax[0] = fmaxf(amax[0], fabsf(x));
-                    hf[q * KBW + i] = x;
-                }
+        vec_front<KW, FW, NQTH>(fx, seq, a.b.H, a.b.HR, NQH, e + 3u, dig, PSF, stat, tr ? tr + 13 : nullptr);
+        if (!fx.ok) break;
+        __syncthreads();
+        if (tr) tr[15] = wall_clock64();
+        RWKV_IDS();
+        if (fin && row == 0) {
+            const double y = finish_col(red, 0, n, stat[16], (int)or_lo(rec, OR_CSFV * 16 + n), stat[18]);
+            const double x_own = y * rf_lds[n] + x_lds[n];                       // block.py:100
+            x_lds[n] = x_own;
+            const float Pn[3] = {__uint_as_float(or_lo(rec, OR_PN01 * 16 + n)), __uint_as_float(or_hi(rec, OR_PN01 * 16 + n)),
+                                 __uint_as_float(or_lo(rec, OR_PN2 * 16 + n))};
+            const double POn[3] = {or_d(rec, OR_PON0 * 16 + n), or_d(rec, OR_PON1 * 16 + n), or_d(rec, OR_PON2 * 16 + n)};
+            if (l + 1 == L) {                              // the next consumer of x is the head (one product)
+                const float P1[1] = {Pn[0]};
+                const double PO1[1] = {POn[0]};
+                publish_ln_input<1>(a.b.X, a.b.XR, G, g, n, e + 4u, x_own, P1, PO1);
+            } else {
+                publish_ln_input<3>(a.b.X, a.b.XR, G, g, n, e + 4u, x_own, Pn, POn);
             }
-            if (__syncthreads_or(!ok)) { if (tid == 0) ASTORE(abort_flag, 1u); return; }
-            wg_max<1>(amax, reinterpret_cast<float *>(scr));
-            double S, invS;
-            scale_from_amax(amax[0], S, invS);
-#pragma unroll
-            for (int i = 0; i < 4 * KBW; ++i) zq[1] += put_digits(dig, PSF, tid + kDT * i, hf[i], invS);
-            double *pp_ = part + parity * (kDW * 8);
-            park_partials<2>(zq, pp_, 0);
-            __syncthreads();
-            v4i D = {0, 0, 0, 0};
-#pragma unroll
-            for (int kq = 0; kq < 4; ++kq) {
-                const int j = 9 + kq;                                     // the four C-row quarters of the tile
-                mfma_job<KBW>(ring[j % R], dig, PSF, kq * C, D);
-                load_slot<KBW>(ring[j % R], flat_job(l, j + R));
-            }
-            int *rd = red + parity * RED_INTS;
-            park_tile(rd, 0, D);
-            __syncthreads();
-            if (tid < 16) {
-                const double y = finish_col(rd, 0, tid, S, S * sum_partials(pp_, 1), sum_partials(pp_, 0));
-                x_own = y * rf_own + x_own;                               // block.py:100
-                put_word(a.b.X + c_own, e_base + 4u, (float)x_own);
-                sl[(size_t)C + c_own] = own_ln2[tid];                     // block.py:87-88
-            }
-            parity ^= 1u;
         }
     }
 
     // ========================= head (opt.py:71-73) ==============================
-    {
-        float xf[KBW];
-        const bool ok = poll_words<KBW>(a.b.X, a.epoch0 + 4u * (unsigned)L, xf, abort_flag);
-        if (__syncthreads_or(!ok)) { if (tid == 0) ASTORE(abort_flag, 1u); return; }
-        double xv[KBW];
-#pragma unroll
-        for (int i = 0; i < KBW; ++i) xv[i] = (double)xf[i];
-        layernorm_wg<KBW>(xv, C, a.m.lnout_w, a.m.lnout_b, scr);
-        float xs[KBW];
-        double zq[2] = {0, 0};
-        float amax[1] = {0.f};
-#pragma unroll
-        for (int i = 0; i < KBW; ++i) {
-            const int c = tid + kDT * i;
-            xs[i] = (float)(xv[i] * (double)a.m.head.range[c]);
-            zq[0] += xv[i] * a.m.head.offset[c];
-            amax[0] = fmaxf(amax[0], fabsf(xs[i]));
-        }
-        wg_max<1>(amax, reinterpret_cast<float *>(scr));
-        double S, invS;
-        scale_from_amax(amax[0], S, invS);
-#pragma unroll
-        for (int i = 0; i < KBW; ++i) zq[1] += put_digits(dig, PS, tid + kDT * i, xs[i], invS);
-        double *pp_ = part + parity * (kDW * 8);
-        park_partials<2>(zq, pp_, 0);
+    const int v_tiles = (V + 15) / 16, head_rounds = (v_tiles + G - 1) / G;
+    const u64 *rec_h = own_lds + (L & 1) * kOrSlots;
+    if (fx.ok)
+        ln_front<KW, FW, 1>(fx, seq, a, a.m.P32 + (size_t)L * kLnMats * C, a.m.Q32 + (size_t)L * kLnMats * C, rec_h, 0,
+                            a.epoch0 + 4u * (unsigned)L, dig, stat, nullptr);
+    if (!fx.ok) return;     // every wave leaves after the same barrier: the flag is tested after each one that follows a wait
+    RWKV_IDS();
+#undef RWKV_IDS
+    unsigned par = 0;
+    constexpr int NS = kBackHeadSlots;                   // head tiles per barrier round
+    double Sh;
+    float invSh;
+    ln_scale(stat, rec_h, 0, 0, Sh, invSh);
+    const double zph = ln_zp(stat, rec_h, 0, 0);
+    for (int h0 = 0; h0 < head_rounds; h0 += NS, par ^= 1u) {
         __syncthreads();
-        const double zp = sum_partials(pp_, 0), qsumS = S * sum_partials(pp_, 1);
-        unsigned rpar = parity;
-        for (int h0 = 0; h0 < head_jobs; h0 += R) {
-            v4i D[R];
+        const int s = fx.tid >> 4;                         // parked tile of this round
+        if (s < NS && h0 + s < head_rounds) {
+            const int v = 16 * (g + G * (h0 + s)) + n;
+            if (v < V) a.logits[v] = finish_col(red + par * (NS * kBW * 16), s, n, Sh, a.m.cs_head[v], zph);
+        }
+    }
+}
+
+template <int KW, int FW>
+struct DecodeLds {
+    static constexpr int C = 512 * KW, F = 4 * C;
+    static constexpr int PS = C + 64, PSF = F + 64;
+    static constexpr int DIG_BYTES = (3 * 4 * PS > 4 * PSF) ? 3 * 4 * PS : 4 * PSF;
+    static constexpr int RED_SLOTS = BackCfg<KW, FW>::RED_SLOTS;
+    static constexpr int RED_BYTES = RED_SLOTS * kBW * 16 * 16;
+    static constexpr int STAT_BYTES = 32 * 8, RF_BYTES = 32 * 8, FLAG_BYTES = FLAG_COUNT * 4;   // RF: gate and residual of the own channels
+    static constexpr int OWN_OFFSET = DIG_BYTES + RED_BYTES + STAT_BYTES + RF_BYTES + FLAG_BYTES;
+    static constexpr int TOTAL = OWN_OFFSET + 2 * kOrSlots * 8;
+    // the generated back-wave program addresses LDS by these offsets
+    static_assert(BackCfg<KW, FW>::RED == DIG_BYTES, "parked tiles follow the digit planes");
+    static_assert(BackCfg<KW, FW>::FLAG == DIG_BYTES + RED_BYTES + STAT_BYTES + RF_BYTES + FLAG_ABORT * 4, "abort flag offset");
+    static_assert(RED_SLOTS >= 5 && RED_SLOTS >= 2 * kBackHeadSlots, "park slots");
+};
+
+template <int KW, int FW, bool TRACE>
+__global__ void __launch_bounds__((FW + kBW) * 64) decode_kernel(const DArgs a) {
+    using Lds = DecodeLds<KW, FW>;
+    extern __shared__ __align__(16) unsigned char smem[];
+    signed char *dig = reinterpret_cast<signed char *>(smem);
+    v4i *red = reinterpret_cast<v4i *>(smem + Lds::DIG_BYTES);
+    double *stat = reinterpret_cast<double *>(smem + Lds::DIG_BYTES + Lds::RED_BYTES);
+    double *rf_lds = stat + 32;
+    lds_flag_t *flags = (lds_flag_t *)(rf_lds + 32);
+    if (threadIdx.x < FLAG_COUNT) flags[threadIdx.x] = 0;
+    __syncthreads();
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    if (wave < FW) {
+        front_path<KW, FW, TRACE>(a, dig, red, stat, rf_lds, flags, reinterpret_cast<u64 *>(smem + Lds::OWN_OFFSET));
+    } else {
+        constexpr int G = 32 * KW;
+        const int v_tiles = (a.m.V + 15) / 16, head_rounds = (v_tiles + G - 1) / G;
+        const unsigned lds = (unsigned)(uintptr_t)(RWKV_LDS unsigned char *)smem;
+        BackCfg<KW, FW>::run(a.m.jt + (size_t)blockIdx.x * (a.m.L + 1) * 16, a.m.w_head, a.m.L, head_rounds, v_tiles,
+                         (int)blockIdx.x, wave - FW, lds);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Per-token preparation: blocks 0..L-1 turn the shift rows of the state into Q32 and its scalars
+// (they change with every token); block L computes x0 = ln0(emb[token]) (emb.py:9, opt.py:63-64)
+// and publishes it, with its LayerNorm records, as the input of layer 0.
+// ---------------------------------------------------------------------------
+constexpr int kPrepThreads = 512;
+
+template <int N>
+__device__ __forceinline__ void prep_block_sum(double (&v)[N], double *scr) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();
 #pragma unroll
-            for (int s = 0; s < R; ++s) {
-                D[s] = v4i{0, 0, 0, 0};
-                if (head_job(h0 + s)) mfma_job<KBW>(ring[s], dig, PS, 0, D[s]);
-                load_slot<KBW>(ring[s], head_job(h0 + s + R));
-            }
-            int *rd = red + rpar * RED_INTS;
+    for (int i = 0; i < N; ++i) {
+        const double s = wave_sum_dpp(v[i]);
+        if (lane == 0) scr[i * (kPrepThreads / 64) + wave] = s;
+    }
+    __syncthreads();
 #pragma unroll
-            for (int s = 0; s < R; ++s) park_tile(rd, s, D[s]);
-            __syncthreads();
-            if (tid < 16 * R) {
-                const int s = tid >> 4, n = tid & 15;
-                const int v = 16 * (g + G * (h0 + s)) + n;
-                if (h0 + s < head_jobs && v < V) a.logits[v] = finish_col(rd, s, n, S, qsumS, zp);
+    for (int i = 0; i < N; ++i) {
+        double s = 0.0;
+#pragma unroll
+        for (int w = 0; w < kPrepThreads / 64; ++w) s += scr[i * (kPrepThreads / 64) + w];
+        v[i] = s;
+    }
+}
+template <int N>
+__device__ __forceinline__ void prep_block_max(float (&v)[N], float *scr) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        const float s = wave_max_dpp(v[i]);
+        if (lane == 0) scr[i * (kPrepThreads / 64) + wave] = s;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < kPrepThreads / 64; ++w) s = fmaxf(s, scr[i * (kPrepThreads / 64) + w]);
+        v[i] = s;
+    }
+}
+
+__global__ void __launch_bounds__(kPrepThreads) prep_kernel(const DArgs a) {
+    __shared__ double scr[8 * (kPrepThreads / 64)];
+    const int C = a.m.C, L = a.m.L, G = a.m.G;
+    const int l = blockIdx.x;
+    if (l < L) {
+        const DPrep &p = a.m.prep[l];
+        const double *sl = a.state + (size_t)l * 5 * C;
+        double sq[kLnMats] = {0, 0, 0, 0, 0};
+        float mq[kLnMats] = {0, 0, 0, 0, 0};
+        for (int c = threadIdx.x; c < C; c += kPrepThreads) {
+#pragma unroll
+            for (int m = 0; m < kLnMats; ++m) {
+                const bool att = m < 3;
+                const double mu = att ? p.att_mix[(size_t)m * C + c] : p.ffn_mix[(size_t)(m - 3) * C + c];
+                const double sh = att ? sl[c] : sl[(size_t)C + c];
+                const double b = att ? p.ln1_b[c] : p.ln2_b[c];
+                const double base = b * mu + sh * (1.0 - mu);                    // block.py:67,91 without the x term
+                const double rg = (double)p.range[m][c];
+                const float q = (float)(base * rg);
+                a.m.Q32[((size_t)l * kLnMats + m) * C + c] = q;
+                sq[m] += base * (p.offset[m][c] + 128.0 * rg);
+                mq[m] = fmaxf(mq[m], fabsf(q));
             }
-            rpar ^= 1u;
+        }
+        prep_block_sum<kLnMats>(sq, scr);
+        prep_block_max<kLnMats>(mq, reinterpret_cast<float *>(scr));
+        if (threadIdx.x < kLnMats) {
+            a.m.sc[l].sumQO[threadIdx.x] = sq[threadIdx.x];
+            a.m.sc[l].maxQ[threadIdx.x] = mq[threadIdx.x];
+        }
+        return;
+    }
+    // x0 = ln0(emb[token]); C is a multiple of 64 and thread t takes channels t, t + 512, ...
+    int64_t tok = a.token[0];
+    if (tok < 0) tok = 0;
+    if (tok >= a.m.V) tok = a.m.V - 1;
+    double s[2] = {0.0, 0.0};
+    for (int c = threadIdx.x; c < C; c += kPrepThreads) {
+        const double v = (double)a.m.emb[(size_t)tok * C + c];
+        s[0] += v; s[1] += v * v;
+    }
+    prep_block_sum<2>(s, scr);
+    const double mean = s[0] / (double)C;
+    double var = s[1] / (double)C - mean * mean;
+    if (var < 0.0) var = 0.0;
+    const double rsd = 1.0 / sqrt(var + 1e-5);
+    for (int c0 = 0; c0 < C; c0 += kPrepThreads) {
+        const int c = c0 + threadIdx.x;
+        if (c < C) {                                        // whole waves are in or out: C % 64 == 0
+            const double v = (double)a.m.emb[(size_t)tok * C + c];
+            const double x0 = a.m.ln0_w[c] * ((v - mean) * rsd) + a.m.ln0_b[c];
+            a.m.X0[c] = x0;
+            float P[3];
+            double PO[3];
+#pragma unroll
+            for (int m = 0; m < 3; ++m) { P[m] = a.m.P32[(size_t)m * C + c]; PO[m] = a.m.PO[(size_t)m * C + c]; }
+            publish_ln_input<3>(a.b.X, a.b.XR, G, c >> 4, c & 15, a.epoch0, x0, P, PO);
         }
     }
 }
 
 // ---------------------------------------------------------------------------
-template <int KBW>
-static size_t decode_lds_bytes() {
-    constexpr int C = KBW * kDT, F = 4 * C;
-    constexpr int PS = C + 64, PSF = F + 64;
-    constexpr int DIG_BYTES = (3 * 4 * PS > 4 * PSF) ? 3 * 4 * PS : 4 * PSF;
-    return (size_t)DIG_BYTES + 2 * (kDW * kMaxJobsPerPhase * 16 * 4) * sizeof(int) +
-           (2 * kDW * 8 + 4 * kDW + 48) * sizeof(double);
+// Model-creation kernels
+// ---------------------------------------------------------------------------
+// cs[16 t + n] = sum over rows of (code - 128) of column 16 t + n of an M16 matrix; one wave per tile.
+__global__ void __launch_bounds__(64) colsum_m16_kernel(const uint8_t *__restrict__ w16, int n_kb, int *__restrict__ cs) {
+    const int lane = threadIdx.x;
+    const uint8_t *p = w16 + (size_t)blockIdx.x * n_kb * 1024 + lane * 16;
+    int acc = 0;
+    for (int kb = 0; kb < n_kb; ++kb) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(p + (size_t)kb * 1024);
+        const unsigned d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            acc += (int)(signed char)(d[i] & 0xff) + (int)(signed char)((d[i] >> 8) & 0xff) +
+                   (int)(signed char)((d[i] >> 16) & 0xff) + (int)(signed char)(d[i] >> 24);
+    }
+    acc += __shfl_xor(acc, 16, 64);
+    acc += __shfl_xor(acc, 32, 64);
+    if (lane < 16) cs[16 * blockIdx.x + lane] = acc;
 }
 
+// Owner records (see the OR_ slots above); grid (G, L), kOrSlots threads.
+__global__ void __launch_bounds__(kOrSlots) build_ownrec_kernel(const DPrep *__restrict__ prep, const int *__restrict__ cs,
+                                                               const float *__restrict__ P32, const double *__restrict__ PO,
+                                                               int L, int C, int F, int G, u64 *__restrict__ ownrec) {
+    const int g = blockIdx.x, l = blockIdx.y, t = threadIdx.x;
+    const DPrep &p = prep[l];
+    const int *csl = cs + (size_t)l * (6 * C + F);     // k v r o ffn_r [C each], ffn_k [F], ffn_v [C]
+    const float *Pl = P32 + (size_t)l * kLnMats * C, *Pn = P32 + (size_t)(l + 1) * kLnMats * C;
+    const double *POl = PO + (size_t)l * kLnMats * C, *POn = PO + (size_t)(l + 1) * kLnMats * C;
+    const bool last = l + 1 == L;                      // the next row of the tables is the head: one product
+    auto dbl = [](double v) { return (u64)__double_as_longlong(v); };
+    auto pair = [](unsigned lo, unsigned hi) { return ((u64)hi << 32) | (u64)lo; };
+    u64 v = 0;
+    if (t < OR_FIELDS * 16) {
+        const int field = t >> 4, c = 16 * g + (t & 15);
+        switch (field) {
+            case OR_DECAY: v = dbl(p.time_decay[c]); break;
+            case OR_FIRST: v = dbl(p.time_first[c]); break;
+            case OR_LN1W: v = dbl(p.ln1_w[c]); break;
+            case OR_LN1B: v = dbl(p.ln1_b[c]); break;
+            case OR_LN2W: v = dbl(p.ln2_w[c]); break;
+            case OR_LN2B: v = dbl(p.ln2_b[c]); break;
+            case OR_OFFO: v = dbl(p.offset_o[c]); break;
+            case OR_RNGO_CSO: v = pair(__float_as_uint(p.range_o[c]), (unsigned)csl[3 * C + c]); break;
+            case OR_CSK_CSV: v = pair((unsigned)csl[c], (unsigned)csl[C + c]); break;
+            case OR_CSR_CSFR: v = pair((unsigned)csl[2 * C + c], (unsigned)csl[4 * C + c]); break;
+            case OR_CSFV: v = pair((unsigned)csl[5 * C + F + c], 0u); break;
+            case OR_POFK: v = dbl(POl[3 * C + c]); break;
+            case OR_POFR: v = dbl(POl[4 * C + c]); break;
+            case OR_PF: v = pair(__float_as_uint(Pl[3 * C + c]), __float_as_uint(Pl[4 * C + c])); break;
+            case OR_PON0: v = dbl(POn[c]); break;
+            case OR_PON1: v = last ? 0 : dbl(POn[C + c]); break;
+            case OR_PON2: v = last ? 0 : dbl(POn[2 * C + c]); break;
+            case OR_PN01: v = pair(__float_as_uint(Pn[c]), last ? 0u : __float_as_uint(Pn[C + c])); break;
+            case OR_PN2: v = pair(last ? 0u : __float_as_uint(Pn[2 * C + c]), 0u); break;
+            default: break;
+        }
+    } else if (t < kOrStatic) {
+        const int i = (t - kOrOffV) & 63;              // lane of the ffn_k epilogue: tile i / 16, column i % 16
+        const int f = 16 * (g + G * (i >> 4)) + (i & 15);
+        if (t < kOrRngVCs) v = dbl(p.offset_v[f]);
+        else v = pair(__float_as_uint(p.range_v[f]), (unsigned)csl[5 * C + f]);
+    }
+    ownrec[((size_t)l * G + g) * kOrSlots + t] = v;
+}
+
+// jt[g][l][16]: base address of job j of layer l for workgroup g (13 used); row L: the first head
+// tiles of the workgroup (tiles past the end of the vocabulary point at tile 0, whose blocks stay
+// hot in L2 and whose products are never used).  grid (G), any block size.
+__global__ void build_jobtab_kernel(const DLayer *__restrict__ layers, const uint8_t *w_head, int L, int G, int n_kb,
+                                    int v_tiles, u64 *__restrict__ jt) {
+    const int g = blockIdx.x;
+    const size_t TB = (size_t)n_kb * 1024;
+    for (int i = threadIdx.x; i < (L + 1) * 16; i += blockDim.x) {
+        const int l = i >> 4, j = i & 15;
+        const uint8_t *p = w_head;
+        if (l < L && j < kRealJobs) {
+            const DLayer &Ly = layers[l];
+            if (j <= 2) p = Ly.w[j] + (size_t)g * TB;
+            else if (j == 3) p = Ly.w[MAT_ATT_O] + (size_t)g * TB;
+            else if (j == 4) p = Ly.w[MAT_FFN_R] + (size_t)g * TB;
+            else if (j <= 8) p = Ly.w[MAT_FFN_K] + (size_t)(g + G * (j - 5)) * TB;
+            else p = Ly.w[MAT_FFN_V] + ((size_t)g * 4 + (j - 9)) * TB;
+        } else if (l == L) {
+            const int tile = g + G * j;
+            p = w_head + (size_t)(tile < v_tiles ? tile : 0) * TB;
+        }
+        jt[(size_t)g * (L + 1) * 16 + i] = (u64) reinterpret_cast<uintptr_t>(p);
+    }
+}
+
+struct ConstArgs {
+    int L, C;
+    const DPrep *prep;
+    const double *lnout_w, *lnout_b;
+    const float *range_h;
+    const double *offset_h;
+    float *P32, *Q32;
+    double *PO;
+    DScal *sc;
+};
+
+// Token-independent constants of the LayerNorm-fed products; block l < L: layer l, block L: head.
+__global__ void __launch_bounds__(kPrepThreads) build_consts_kernel(const ConstArgs a) {
+    __shared__ double scr[8 * (kPrepThreads / 64)];
+    const int C = a.C, l = blockIdx.x;
+    const bool head = l == a.L;
+    double sp[kLnMats] = {0, 0, 0, 0, 0}, sq[kLnMats] = {0, 0, 0, 0, 0};
+    float mp[kLnMats] = {0, 0, 0, 0, 0}, mq[kLnMats] = {0, 0, 0, 0, 0};
+    for (int c = threadIdx.x; c < C; c += kPrepThreads) {
+#pragma unroll
+        for (int m = 0; m < kLnMats; ++m) {
+            if (head && m > 0) continue;
+            double lw, mu, rg, of;
+            if (head) {
+                lw = a.lnout_w[c]; mu = 1.0; rg = (double)a.range_h[c]; of = a.offset_h[c];
+            } else {
+                const DPrep &p = a.prep[l];
+                const bool att = m < 3;
+                lw = att ? p.ln1_w[c] : p.ln2_w[c];
+                mu = att ? p.att_mix[(size_t)m * C + c] : p.ffn_mix[(size_t)(m - 3) * C + c];
+                rg = (double)p.range[m][c]; of = p.offset[m][c];
+            }
+            const float P = (float)(lw * mu * rg);
+            const double PO = lw * mu * (of + 128.0 * rg);
+            a.P32[((size_t)l * kLnMats + m) * C + c] = P;
+            a.PO[((size_t)l * kLnMats + m) * C + c] = PO;
+            sp[m] += PO;
+            mp[m] = fmaxf(mp[m], fabsf(P));
+            if (head) {
+                const double base = a.lnout_b[c];
+                const float Q = (float)(base * rg);
+                a.Q32[((size_t)l * kLnMats + m) * C + c] = Q;
+                sq[m] += base * (of + 128.0 * rg);
+                mq[m] = fmaxf(mq[m], fabsf(Q));
+            }
+        }
+    }
+    prep_block_sum<kLnMats>(sp, scr);
+    prep_block_sum<kLnMats>(sq, scr);
+    prep_block_max<kLnMats>(mp, reinterpret_cast<float *>(scr));
+    prep_block_max<kLnMats>(mq, reinterpret_cast<float *>(scr));
+    if (threadIdx.x < kLnMats) {
+        a.sc[l].sumPO[threadIdx.x] = sp[threadIdx.x];
+        a.sc[l].maxP[threadIdx.x] = mp[threadIdx.x];
+        if (head) { a.sc[l].sumQO[threadIdx.x] = sq[threadIdx.x]; a.sc[l].maxQ[threadIdx.x] = mq[threadIdx.x]; }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
 bool decode_supported(int64_t L, int64_t C, int64_t F, int64_t V) {
     if (L <= 0 || V <= 0 || F != 4 * C) return false;
     // one 16-column tile per workgroup, all workgroups resident: C/16 <= 256 CUs
@@ -610,16 +967,133 @@ bool decode_supported(int64_t L, int64_t C, int64_t F, int64_t V) {
 
 unsigned decode_epochs_per_token(int64_t L) { return (unsigned)(4 * L + 1); }
 
-template <int KBW>
+namespace {
+struct BlockPlan {
+    size_t layers, prep, P32, Q32, PO, sc, X0, cs, ownrec, jt, xchg, abort, total;
+    size_t cs_layer_ints;
+};
+BlockPlan plan_block(int64_t L, int64_t C, int64_t F, int64_t V) {
+    BlockPlan p;
+    size_t off = 0;
+    auto take = [&](size_t bytes) { const size_t o = off; off += (size_t)round_up((int64_t)bytes, 256); return o; };
+    const size_t G = (size_t)C / 16;
+    p.layers = take((size_t)L * sizeof(DLayer));
+    p.prep = take((size_t)L * sizeof(DPrep));
+    p.P32 = take((size_t)(L + 1) * kLnMats * C * sizeof(float));
+    p.Q32 = take((size_t)(L + 1) * kLnMats * C * sizeof(float));
+    p.PO = take((size_t)(L + 1) * kLnMats * C * sizeof(double));
+    p.sc = take((size_t)(L + 1) * sizeof(DScal));
+    p.X0 = take((size_t)C * sizeof(double));
+    p.cs_layer_ints = (size_t)(6 * C + F);
+    p.cs = take(((size_t)L * p.cs_layer_ints + (size_t)round_up(V, 16)) * sizeof(int));
+    p.ownrec = take((size_t)L * G * kOrSlots * sizeof(u64));
+    p.jt = take(G * (size_t)(L + 1) * 16 * sizeof(u64));
+    p.xchg = take(((size_t)2 * C + F + (size_t)(kLnRows + 6) * G) * sizeof(u64));
+    p.abort = take(256);
+    p.total = off;
+    return p;
+}
+}  // namespace
+
+size_t decode_block_bytes(int64_t L, int64_t C, int64_t F, int64_t V) { return plan_block(L, C, F, V).total; }
+
+int decode_setup(void *block, const DSetup &s, DModel *dm, DecodeBuffers *db) {
+    const int64_t L = s.L, C = s.C, F = s.F, V = s.V;
+    if (!decode_supported(L, C, F, V)) return set_error(RWKV_ERR_SIZE, "decode_setup: unsupported shape");
+    const BlockPlan p = plan_block(L, C, F, V);
+    unsigned char *base = static_cast<unsigned char *>(block);
+    const size_t G = (size_t)C / 16;
+    int *cs = reinterpret_cast<int *>(base + p.cs);
+    std::vector<DLayer> tab((size_t)L);
+    std::vector<DPrep> prep((size_t)L);
+    const int c_kb = (int)(C / 64), f_kb = (int)(F / 64);
+    for (int64_t l = 0; l < L; ++l) {
+        const DLayerSrc &src = s.layers[l];
+        DLayer &t = tab[(size_t)l];
+        const DQ *q[MAT_COUNT];
+        q[MAT_ATT_K] = &src.att_k; q[MAT_ATT_V] = &src.att_v; q[MAT_ATT_R] = &src.att_r; q[MAT_ATT_O] = &src.att_o;
+        q[MAT_FFN_R] = &src.ffn_r; q[MAT_FFN_K] = &src.ffn_k; q[MAT_FFN_V] = &src.ffn_v;
+        int *csl = cs + (size_t)l * p.cs_layer_ints;
+        t.pad = nullptr;
+        for (int i = 0; i < MAT_COUNT; ++i) {
+            t.w[i] = q[i]->w16;
+            const int n_out = i == MAT_FFN_K ? (int)F : (int)C;
+            const int n_kb = i == MAT_FFN_V ? f_kb : c_kb;
+            // order inside the layer's column-sum slab: k v r o ffn_r [C each], ffn_k [F], ffn_v [C]
+            int *dst = csl + (i <= MAT_FFN_R ? (size_t)i * C : (i == MAT_FFN_K ? (size_t)5 * C : (size_t)5 * C + F));
+            hipLaunchKernelGGL(colsum_m16_kernel, dim3((unsigned)(n_out / 16)), dim3(64), 0, nullptr, q[i]->w16, n_kb, dst);
+        }
+        DPrep &pr = prep[(size_t)l];
+        pr.ln1_w = src.ln1_w; pr.ln1_b = src.ln1_b; pr.ln2_w = src.ln2_w; pr.ln2_b = src.ln2_b;
+        pr.att_mix = src.att_mix; pr.ffn_mix = src.ffn_mix;
+        pr.time_decay = src.time_decay; pr.time_first = src.time_first;
+        pr.range_o = src.att_o.range; pr.offset_o = src.att_o.offset;
+        pr.range_v = src.ffn_v.range; pr.offset_v = src.ffn_v.offset;
+        const DQ *lm[kLnMats] = {&src.att_k, &src.att_v, &src.att_r, &src.ffn_k, &src.ffn_r};
+        for (int m = 0; m < kLnMats; ++m) { pr.range[m] = lm[m]->range; pr.offset[m] = lm[m]->offset; }
+    }
+    RWKV_CHECK_LAUNCH("colsum_m16_kernel");
+    int *cs_head = cs + (size_t)L * p.cs_layer_ints;
+    hipLaunchKernelGGL(colsum_m16_kernel, dim3((unsigned)ceil_div(V, 16)), dim3(64), 0, nullptr, s.head.w16, c_kb, cs_head);
+    RWKV_CHECK_LAUNCH("colsum_m16_kernel");
+    RWKV_CHECK_HIP(hipMemcpy(base + p.layers, tab.data(), (size_t)L * sizeof(DLayer), hipMemcpyHostToDevice));
+    RWKV_CHECK_HIP(hipMemcpy(base + p.prep, prep.data(), (size_t)L * sizeof(DPrep), hipMemcpyHostToDevice));
+
+    dm->L = (int)L; dm->C = (int)C; dm->F = (int)F; dm->V = (int)V; dm->G = (int)G;
+    dm->emb = s.emb; dm->ln0_w = s.ln0_w; dm->ln0_b = s.ln0_b;
+    dm->w_head = s.head.w16; dm->cs = cs; dm->cs_head = cs_head;
+    dm->ownrec = reinterpret_cast<const u64 *>(base + p.ownrec);
+    dm->layers = reinterpret_cast<const DLayer *>(base + p.layers);
+    dm->prep = reinterpret_cast<const DPrep *>(base + p.prep);
+    dm->P32 = reinterpret_cast<float *>(base + p.P32);
+    dm->Q32 = reinterpret_cast<float *>(base + p.Q32);
+    dm->PO = reinterpret_cast<double *>(base + p.PO);
+    dm->sc = reinterpret_cast<DScal *>(base + p.sc);
+    dm->X0 = reinterpret_cast<double *>(base + p.X0);
+
+    ConstArgs ca;
+    dm->jt = reinterpret_cast<const u64 *>(base + p.jt);
+    hipLaunchKernelGGL(build_jobtab_kernel, dim3((unsigned)G), dim3(256), 0, nullptr, dm->layers, s.head.w16, (int)L,
+                       (int)G, c_kb, (int)ceil_div(V, 16), reinterpret_cast<u64 *>(base + p.jt));
+    RWKV_CHECK_LAUNCH("build_jobtab_kernel");
+    ca.L = (int)L; ca.C = (int)C; ca.prep = dm->prep;
+    ca.lnout_w = s.lnout_w; ca.lnout_b = s.lnout_b; ca.range_h = s.head.range; ca.offset_h = s.head.offset;
+    ca.P32 = dm->P32; ca.Q32 = dm->Q32; ca.PO = dm->PO; ca.sc = dm->sc;
+    hipLaunchKernelGGL(build_consts_kernel, dim3((unsigned)(L + 1)), dim3(kPrepThreads), 0, nullptr, ca);
+    RWKV_CHECK_LAUNCH("build_consts_kernel");
+    hipLaunchKernelGGL(build_ownrec_kernel, dim3((unsigned)G, (unsigned)L), dim3(kOrSlots), 0, nullptr, dm->prep, dm->cs,
+                       dm->P32, dm->PO, (int)L, (int)C, (int)F, (int)G, reinterpret_cast<u64 *>(base + p.ownrec));
+    RWKV_CHECK_LAUNCH("build_ownrec_kernel");
+
+    u64 *x = reinterpret_cast<u64 *>(base + p.xchg);
+    db->X = x; x += C;
+    db->XR = x; x += (size_t)kLnRows * G;
+    db->A = x; x += C;
+    db->AR = x; x += 3 * G;
+    db->H = x; x += F;
+    db->HR = x;
+    db->abort_flag = reinterpret_cast<unsigned *>(base + p.abort);
+    db->trace = nullptr;
+    RWKV_CHECK_HIP(hipDeviceSynchronize());
+    return RWKV_OK;
+}
+
+template <int KW, int FW>
 static int launch_one(hipStream_t st, const DArgs &args) {
-    const size_t lds = decode_lds_bytes<KBW>();
+    constexpr int lds = DecodeLds<KW, FW>::TOTAL;
     static bool configured = false;
     if (!configured) {
-        RWKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_kernel<KBW>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        RWKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_kernel<KW, FW, false>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        RWKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_kernel<KW, FW, true>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         configured = true;
     }
-    hipLaunchKernelGGL(decode_kernel<KBW>, dim3(args.m.C / 16), dim3(kDT), lds, st, args);
+    hipLaunchKernelGGL(prep_kernel, dim3((unsigned)(args.m.L + 1)), dim3(kPrepThreads), 0, st, args);
+    if (args.b.trace)
+        hipLaunchKernelGGL((decode_kernel<KW, FW, true>), dim3((unsigned)args.m.G), dim3((FW + kBW) * 64), lds, st, args);
+    else
+        hipLaunchKernelGGL((decode_kernel<KW, FW, false>), dim3((unsigned)args.m.G), dim3((FW + kBW) * 64), lds, st, args);
     RWKV_CHECK_LAUNCH("decode_kernel");
     return RWKV_OK;
 }
@@ -629,10 +1103,10 @@ int decode_launch(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsig
     DArgs args;
     args.m = m; args.b = b; args.epoch0 = epoch0; args.token = token; args.state = state; args.logits = logits;
     switch (m.C) {
-        case 1024: return launch_one<2>(st, args);
-        case 2048: return launch_one<4>(st, args);
-        case 2560: return launch_one<5>(st, args);
-        case 4096: return launch_one<8>(st, args);
+        case 1024: return launch_one<2, 4>(st, args);
+        case 2048: return launch_one<4, 4>(st, args);
+        case 2560: return launch_one<5, 4>(st, args);
+        case 4096: return launch_one<8, 4>(st, args);
         default: return set_error(RWKV_ERR_SIZE, "decode kernel: n_embd %d not supported", m.C);
     }
 }

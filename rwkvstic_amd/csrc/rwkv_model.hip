@@ -460,31 +460,26 @@ int setup_fused(rwkv_model *m) {
         all16 = all16 && ld.att_k.packed16 && ld.att_v.packed16 && ld.att_r.packed16 && ld.att_o.packed16 &&
                 ld.ffn_k.packed16 && ld.ffn_r.packed16 && ld.ffn_v.packed16;
     if (!all16) return RWKV_OK;
-    const size_t L = (size_t)d.n_layer, C = (size_t)d.n_embd, F = (size_t)d.n_ffn;
-    const size_t table_bytes = round_up(L * sizeof(DLayer), 256);
-    const size_t xchg_bytes = (2 * C + F) * sizeof(u64);
-    const size_t total = table_bytes + xchg_bytes + 256;
+    const size_t total = decode_block_bytes(d.n_layer, d.n_embd, d.n_ffn, d.n_vocab);
     RWKV_CHECK_HIP(hipMalloc(&m->dev_block, total));
     RWKV_CHECK_HIP(hipMemset(m->dev_block, 0, total));
-    std::vector<DLayer> tab(L);
-    for (size_t l = 0; l < L; ++l) {
+    std::vector<DLayerSrc> src((size_t)d.n_layer);
+    for (size_t l = 0; l < src.size(); ++l) {
         const rwkv_layer_desc &ld = m->layers[l];
-        DLayer &t = tab[l];
+        DLayerSrc &t = src[l];
         t.att_k = to_dq(ld.att_k); t.att_v = to_dq(ld.att_v); t.att_r = to_dq(ld.att_r); t.att_o = to_dq(ld.att_o);
         t.ffn_k = to_dq(ld.ffn_k); t.ffn_r = to_dq(ld.ffn_r); t.ffn_v = to_dq(ld.ffn_v);
         t.ln1_w = ld.ln1_w; t.ln1_b = ld.ln1_b; t.ln2_w = ld.ln2_w; t.ln2_b = ld.ln2_b;
         t.att_mix = ld.att_mix; t.ffn_mix = ld.ffn_mix; t.time_decay = ld.time_decay; t.time_first = ld.time_first;
     }
-    RWKV_CHECK_HIP(hipMemcpy(m->dev_block, tab.data(), L * sizeof(DLayer), hipMemcpyHostToDevice));
-    unsigned char *base = static_cast<unsigned char *>(m->dev_block);
-    m->dm.L = (int)L; m->dm.C = (int)C; m->dm.F = (int)F; m->dm.V = (int)d.n_vocab;
-    m->dm.emb = d.emb; m->dm.ln0_w = d.ln0_w; m->dm.ln0_b = d.ln0_b;
-    m->dm.lnout_w = d.ln_out_w; m->dm.lnout_b = d.ln_out_b; m->dm.head = to_dq(d.head);
-    m->dm.layers = reinterpret_cast<const DLayer *>(base);
-    u64 *x = reinterpret_cast<u64 *>(base + table_bytes);
-    m->db.X = x; m->db.A = x + C; m->db.H = x + 2 * C;
-    m->db.abort_flag = reinterpret_cast<unsigned *>(base + table_bytes + xchg_bytes);
-    m->epoch = 0;
+    DSetup s;
+    s.L = d.n_layer; s.C = d.n_embd; s.F = d.n_ffn; s.V = d.n_vocab;
+    s.emb = d.emb; s.ln0_w = d.ln0_w; s.ln0_b = d.ln0_b; s.lnout_w = d.ln_out_w; s.lnout_b = d.ln_out_b;
+    s.head = to_dq(d.head);
+    s.layers = src.data();
+    const int rc = decode_setup(m->dev_block, s, &m->dm, &m->db);
+    if (rc) return rc;
+    m->epoch = 1;      // tag 0 is what the zero-filled exchange buffers hold
     m->fused = true;
     return RWKV_OK;
 }
@@ -657,6 +652,12 @@ void rwkv_model_destroy(rwkv_model *m) {
 }
 
 int rwkv_model_has_fused_step(const rwkv_model *m) { return (m && m->fused) ? 1 : 0; }
+
+int rwkv_model_set_trace(rwkv_model *m, int64_t *device_buffer) {
+    RWKV_CHECK_ARG(m, "rwkv_model_set_trace: null handle");
+    m->db.trace = reinterpret_cast<long long *>(device_buffer);
+    return RWKV_OK;
+}
 
 int rwkv_model_check(rwkv_model *m) {
     RWKV_CHECK_ARG(m, "rwkv_model_check: null handle");
