@@ -32,9 +32,10 @@ import sys
 V_APC, V_APF, V_PARK, V_FLAG, V_OFF, V_D, V_A = 4, 5, 6, 7, 8, 16, 24
 NA = 3            # A-operand buffers
 S_CUR, S_NXT = 36, 64
-S_L, S_T, S_JT, S_TILE, S_RT, S_RP, S_CNT, S_PAR = 90, 91, 92, 94, 95, 96, 98, 99
-NS = 4            # head tiles per barrier round (two rounds of park slots in LDS)
+S_L, S_T, S_JT, S_TILE, S_RT, S_RP, S_PAR = 90, 91, 92, 94, 95, 96, 99
 PF = NA - 1       # A-operand reads run this many positions ahead
+import os
+WINDOW = int(os.environ.get("RWKV_BACK_WINDOW", "4"))   # weight loads a wave keeps in flight while it reloads slots
 
 
 class Emit:
@@ -50,7 +51,7 @@ class Emit:
         self.issued = 0
 
 
-def gen(KW, R, NV):
+def gen(KW, R, NV, NSH):
     C = 512 * KW
     F = 4 * C
     PS, PSF = C + 64, F + 64
@@ -63,7 +64,7 @@ def gen(KW, R, NV):
     TB = 8 * KW * 1024
     DIG = max(12 * PS, 4 * PSF)
     RED = DIG                                 # byte offset of the parked tiles from the start of LDS
-    RED_SLOTS = max(5, 2 * NS)
+    RED_SLOTS = max(5, 2 * NSH)
     FLAG = RED + RED_SLOTS * 2048 + 32 * 8 + 32 * 8 + 2 * 4   # FLAG_ABORT word
     LH = R * KW // math.gcd(R, KW)
     e = Emit()
@@ -154,36 +155,22 @@ def gen(KW, R, NV):
         e(f"global_load_dwordx4 {ring(p)}, v{V_OFF + b}, s[{S_CUR + 2 * j}:{S_CUR + 2 * j + 1}]")
 
     # ------------------------------------------------------------------ layers
-    phase_start = {0: 2, 3 * KW: 1, 4 * KW: 2, 9 * KW: 1}       # position -> barriers before it
-    def phase_end(p):
-        for pe in (3 * KW, 4 * KW, 9 * KW, 13 * KW):
-            if p < pe:
-                return pe
-        return None
+    # Loads are issued in position order; position q's load is the q-th load of the wave.  A slot
+    # is reloaded right away only when its next position still belongs to the current phase;
+    # otherwise the reload waits until the phase's tiles are parked and the barrier is passed, so
+    # that pushing requests into a busy memory system never delays the phase's results.
+    phases = [(0, 3 * KW, 2), (3 * KW, 4 * KW, 1), (4 * KW, 9 * KW, 2), (9 * KW, 13 * KW, 1)]   # start, end, barriers before
 
-    e("1:")
-    for p in range(PP):
+    def throttle():
+        # A burst of reloads would sit in the compute unit's memory pipeline in front of the front
+        # waves' polls and stores; keeping a window in flight paces the requests to what HBM delivers.
+        if WINDOW - 1 < R - 1:
+            e(f"s_waitcnt vmcnt({WINDOW - 1})")
+
+    def layer_reload(p):
+        """Reload the slot of layer position p (0 <= p < PP) with position p + R."""
+        throttle()
         slot = p % R
-        if p < NREAL:
-            j, b = divmod(p, KW)
-            pe = phase_end(p)
-            if p in phase_start:
-                for _ in range(phase_start[p]):
-                    bar_check()
-                for q in range(p, min(p + PF, pe)):
-                    aread(q)
-            if p + PF < pe:
-                aread(p + PF)
-            allow = e.issued - 1 - e.ridx[p % NA]
-            assert 0 <= allow <= 15
-            e(f"s_waitcnt vmcnt({R - 1}) lgkmcnt({allow})")
-            dreg = V_D + 4 * (1 if j >= 9 else j % 2)
-            first = (b == 0) and not (j > 9)
-            acc = "0" if first else f"v[{dreg}:{dreg + 3}]"
-            e(f"v_mfma_i32_16x16x64_i8 v[{dreg}:{dreg + 3}], {abuf(p)}, {ring(slot)}, {acc}")
-        else:
-            e(f"s_waitcnt vmcnt({R - 1})")
-        # reload the slot with position p + R
         q = p + R
         sset = S_CUR
         if q >= PP:
@@ -194,14 +181,46 @@ def gen(KW, R, NV):
         else:
             jq, bq = divmod(q, KW)
             e(f"global_load_dwordx4 {ring(slot)}, v{V_OFF + bq}, s[{sset + 2 * jq}:{sset + 2 * jq + 1}]")
-        if p < NREAL:
+
+    e("1:")
+    for ps, pe, nbar in phases:
+        for _ in range(nbar):
+            bar_check()
+        for q in range(ps, min(ps + PF, pe)):
+            aread(q)
+        issued_loads = ps + R          # loads issued so far: positions < ps + R
+        deferred = []
+        for p in range(ps, pe):
+            j, b = divmod(p, KW)
+            if p + PF < pe:
+                aread(p + PF)
+            allow = e.issued - 1 - e.ridx[p % NA]
+            assert 0 <= allow <= 15
+            nvm = issued_loads - 1 - p
+            assert 0 <= nvm <= 63, (KW, R, p, nvm)
+            e(f"s_waitcnt vmcnt({nvm}) lgkmcnt({allow})")
+            dreg = V_D + 4 * (1 if j >= 9 else j % 2)
+            first = (b == 0) and not (j > 9)
+            acc = "0" if first else f"v[{dreg}:{dreg + 3}]"
+            e(f"v_mfma_i32_16x16x64_i8 v[{dreg}:{dreg + 3}], {abuf(p)}, {ring(p % R)}, {acc}")
+            if p + R < pe:
+                assert issued_loads == p + R
+                layer_reload(p)
+                issued_loads += 1
+            else:
+                deferred.append(p)
             if b == KW - 1 and (j < 9 or j == 12):
                 pslot = j if j <= 2 else (0 if j == 3 else (j - 4 if j <= 8 else 0))
                 park_static(dreg, pslot)
-            if p + 1 == pe:
-                e("s_waitcnt lgkmcnt(0)")
-                e("s_barrier")
-                e.drain_state()
+        e("s_waitcnt lgkmcnt(0)")
+        e("s_barrier")
+        e.drain_state()
+        if pe == NREAL:
+            deferred += list(range(NREAL, PP))     # padding positions: nothing to compute, only their turn to load
+        for p in deferred:
+            assert issued_loads == p + R
+            layer_reload(p)
+            issued_loads += 1
     # end of layer: next layer's addresses become current; fetch the layer after
     e(f"s_add_u32 s{S_JT}, s{S_JT}, 128")
     e(f"s_addc_u32 s{S_JT + 1}, s{S_JT + 1}, 0")
@@ -216,6 +235,8 @@ def gen(KW, R, NV):
     e("s_branch 1b")
 
     # ------------------------------------------------------------------ head
+    # Rounds of NSH tiles: multiply, park, barrier, then the round's reloads.  The body below covers
+    # LH = lcm(R, KW) positions (a whole number of rounds), after which slots and blocks line up again.
     def head_ptr():
         """s[S_RP] = address of head tile g + G * s[S_RT], or of tile 0 when that is past the end."""
         e(f"s_mul_i32 vcc_lo, s{S_RT}, {G}")
@@ -227,63 +248,78 @@ def gen(KW, R, NV):
         e(f"s_add_u32 s{S_RP}, %[whlo], vcc_lo")
         e(f"s_addc_u32 s{S_RP + 1}, %[whhi], vcc_hi")
 
-    e("2:")
-    bar_check()
-    bar_check()
-    e(f"s_mov_b32 s{S_TILE}, 0")
-    e(f"s_mov_b32 s{S_CNT}, 0")
-    e(f"s_mov_b32 s{S_PAR}, 0")
-    e(f"s_mov_b32 s{S_RT}, {R // KW - (1 if R % KW == 0 else 0)}")
-    head_ptr()
-    e("3:")
-    for q in range(LH):
-        slot = q % R
-        tq, b = divmod(q, KW)
-        dreg = V_D + 4 * (tq % 2)
-        if b == 0:
-            e(f"s_cmp_ge_u32 s{S_TILE}, %[hr]")
-            e("s_cbranch_scc1 8f")
-            e.drain_state()               # the tile before ended with a park and, at most, a barrier
-            e("s_waitcnt lgkmcnt(0)")
-            for bb in range(min(PF, KW)):
-                aread(head_b=bb)
-        if b + PF < KW:
-            aread(head_b=b + PF)
-        allow = e.issued - 1 - e.ridx[b % NA]
-        assert 0 <= allow <= 15
-        e(f"s_waitcnt vmcnt({R - 1}) lgkmcnt({allow})")
-        acc = "0" if b == 0 else f"v[{dreg}:{dreg + 3}]"
-        e(f"v_mfma_i32_16x16x64_i8 v[{dreg}:{dreg + 3}], v[{V_A + 4 * (b % NA)}:{V_A + 4 * (b % NA) + 3}], {ring(slot)}, {acc}")
+    def head_reload(q):
+        """Reload the slot of body position q with position q + R of the head stream."""
+        throttle()
         rb = (q + R) % KW
         if rb == 0:
             e(f"s_add_u32 s{S_RT}, s{S_RT}, 1")
             head_ptr()
-        e(f"global_load_dwordx4 {ring(slot)}, v{V_OFF + rb}, s[{S_RP}:{S_RP + 1}]")
-        if b == KW - 1:
-            e("s_nop 7"); e("s_nop 7"); e("s_nop 7")
-            e(f"s_add_u32 s{S_T}, s{S_CNT}, s{S_PAR}")
-            e(f"s_lshl_b32 s{S_T}, s{S_T}, 11")
-            e(f"v_add_u32 v{V_A}, s{S_T}, v{V_PARK}")
-            e("s_mov_b64 exec, 0xffff")
-            e(f"ds_write_b128 v{V_A}, v[{dreg}:{dreg + 3}]")
-            e("s_mov_b64 exec, -1")
-            e(f"s_add_u32 s{S_TILE}, s{S_TILE}, 1")
-            e(f"s_add_u32 s{S_CNT}, s{S_CNT}, 1")
-            e(f"s_cmp_eq_u32 s{S_CNT}, {NS}")
-            e("s_cbranch_scc0 7f")
-            e("s_waitcnt lgkmcnt(0)")
-            e("s_barrier")
-            e(f"s_mov_b32 s{S_CNT}, 0")
-            e(f"s_xor_b32 s{S_PAR}, s{S_PAR}, {NS}")
-            e("7:")
+        e(f"global_load_dwordx4 {ring(q % R)}, v{V_OFF + rb}, s[{S_RP}:{S_RP + 1}]")
+
+    tiles_per_body = LH // KW
+    assert tiles_per_body % NSH == 0
+    e("2:")
+    bar_check()
+    bar_check()
+    e(f"s_mov_b32 s{S_TILE}, 0")
+    e(f"s_mov_b32 s{S_PAR}, 0")
+    e(f"s_mov_b32 s{S_RT}, {R // KW - (1 if R % KW == 0 else 0)}")
+    head_ptr()
+    e("3:")
+    for r0 in range(0, tiles_per_body, NSH):
+        ps, pe = r0 * KW, (r0 + NSH) * KW
+        issued_loads = ps + R
+        deferred = []
+        for q in range(ps, pe):
+            tq, b = divmod(q, KW)
+            dreg = V_D + 4 * (tq % 2)
+            if b == 0:
+                # a round that starts past the end of the head is not started; one that ends past it
+                # is cut short after the last tile (label 8)
+                e(f"s_cmp_ge_u32 s{S_TILE}, %[hr]")
+                e("s_cbranch_scc1 8f" if tq % NSH else "s_cbranch_scc1 9f")
+                e("s_waitcnt lgkmcnt(0)")
+                e.drain_state()
+                for bb in range(min(PF, KW)):
+                    aread(head_b=bb)
+            if b + PF < KW:
+                aread(head_b=b + PF)
+            allow = e.issued - 1 - e.ridx[b % NA]
+            assert 0 <= allow <= 15
+            nvm = issued_loads - 1 - q
+            assert 0 <= nvm <= 63
+            e(f"s_waitcnt vmcnt({nvm}) lgkmcnt({allow})")
+            acc = "0" if b == 0 else f"v[{dreg}:{dreg + 3}]"
+            e(f"v_mfma_i32_16x16x64_i8 v[{dreg}:{dreg + 3}], v[{V_A + 4 * (b % NA)}:{V_A + 4 * (b % NA) + 3}], {ring(q % R)}, {acc}")
+            if q + R < pe:
+                assert issued_loads == q + R
+                head_reload(q)
+                issued_loads += 1
+            else:
+                deferred.append(q)
+            if b == KW - 1:
+                e("s_nop 7"); e("s_nop 7"); e("s_nop 7")
+                e(f"s_add_u32 s{S_T}, s{S_PAR}, {tq % NSH}")
+                e(f"s_lshl_b32 s{S_T}, s{S_T}, 11")
+                e(f"v_add_u32 v{V_A}, s{S_T}, v{V_PARK}")
+                e("s_mov_b64 exec, 0xffff")
+                e(f"ds_write_b128 v{V_A}, v[{dreg}:{dreg + 3}]")
+                e("s_mov_b64 exec, -1")
+                e(f"s_add_u32 s{S_TILE}, s{S_TILE}, 1")
+        e("s_waitcnt lgkmcnt(0)")
+        e("s_barrier")
+        e(f"s_xor_b32 s{S_PAR}, s{S_PAR}, {NSH}")
+        for q in deferred:
+            assert issued_loads == q + R
+            head_reload(q)
+            issued_loads += 1
     e("s_branch 3b")
-    e("8:")
-    e(f"s_cmp_eq_u32 s{S_CNT}, 0")
-    e("s_cbranch_scc1 9f")
+    e("8:")                      # the head ended inside a round: its tiles are parked, release the finishers
     e("s_waitcnt lgkmcnt(0)")
     e("s_barrier")
     e("9:")
-    return e.lines, dict(KW=KW, R=R, PP=PP, RB=RB, RED=RED, FLAG=FLAG, RED_SLOTS=RED_SLOTS)
+    return e.lines, dict(KW=KW, R=R, PP=PP, RB=RB, RED=RED, FLAG=FLAG, RED_SLOTS=RED_SLOTS, NS=NSH)
 
 
 # (KW, front waves, ring size): 4 front waves -> 12 waves per workgroup, 168 VGPRs each;
@@ -297,14 +333,15 @@ def main():
     w = out.append
     w("// Generated by gen_decode_back.py - do not edit.  One asm statement per kernel width: the program")
     w("// of a weight-streaming wave of the single-token kernel (see the generator for the register map).")
-    w(f"constexpr int kBackHeadSlots = {NS};   // head tiles parked per barrier round")
     w("template <int KW, int FW> struct BackCfg;")
     for KW, FW, R in CONFIGS:
         NV = 168 if FW == 4 else 128
         clob = ", ".join(f'"v{i}"' for i in range(V_APC, NV)) + ", " + ", ".join(f'"s{i}"' for i in range(S_CUR, 100))
-        lines, info = gen(KW, R, NV)
+        tiles_per_body = R // math.gcd(R, KW)
+        NSH = max(d for d in range(1, 5) if tiles_per_body % d == 0)     # head tiles per barrier round
+        lines, info = gen(KW, R, NV, NSH)
         w(f"template <> struct BackCfg<{KW}, {FW}> {{")
-        w(f"    static constexpr int R = {R}, RED = {info['RED']}, FLAG = {info['FLAG']}, RED_SLOTS = {info['RED_SLOTS']};")
+        w(f"    static constexpr int R = {R}, RED = {info['RED']}, FLAG = {info['FLAG']}, RED_SLOTS = {info['RED_SLOTS']}, NS = {info['NS']};")
         w("    static __device__ __forceinline__ void run(const unsigned long long *jt, const uint8_t *wh, int L, int hr, int vt,")
         w("                                                int g, int wb, unsigned lds) {")
         w("        const unsigned whlo = (unsigned)(unsigned long long)(uintptr_t)wh;")

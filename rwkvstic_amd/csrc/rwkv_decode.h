@@ -38,8 +38,9 @@ struct DScal {
     double sumPO[kLnMats];   // sum_c PO[c]
     double sumQO[kLnMats];   // sum_c (ln_b mu + shift (1 - mu)) (offset + 128 range)   (per token)
     float maxP[kLnMats];     // max_c |P32[c]|
+    float pad1;
     float maxQ[kLnMats];     // max_c |Q32[c]|                                             (per token)
-    double pad;
+    float pad2;
 };
 static_assert(sizeof(DScal) == 128, "DScal is read as a 128-byte record");
 
@@ -63,6 +64,10 @@ struct DModel {
     float *Q32;                  // [L+1][5][C]   rows < L rewritten for every token
     double *PO;                  // [L+1][5][C]
     DScal *sc;                   // [L+1]
+    DScal *scp;                  // [L][C/512] per-token scalars (sumQO, maxQ) of each 512-channel part of a layer
+    double *amax_val;            // scratch of the device-side argmax: per block maximum, its index, arrival counter
+    int *amax_idx;
+    unsigned *amax_count;
     double *X0;                  // [C] ln0(emb[token]) of the launch in flight
 };
 
@@ -106,5 +111,8 @@ int decode_setup(void *block, const DSetup &s, DModel *dm, DecodeBuffers *db);
 // decode_epochs_per_token() between launches on the same buffers and never be 0.
 int decode_launch(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsigned epoch0,
                   const int64_t *token, double *state, double *logits);
+// n greedy steps: tokens[i + 1] = argmax(forward(tokens[i])); uses n * decode_epochs_per_token() epochs.
+int decode_launch_greedy(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsigned epoch0,
+                         int64_t *tokens, int64_t n, double *state, double *logits);
 
 }  // namespace rwkv

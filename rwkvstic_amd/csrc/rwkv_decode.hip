@@ -319,10 +319,10 @@ __device__ __forceinline__ unsigned or_hi(const u64 *rec, int slot) { return (un
 __device__ __forceinline__ double or_sumPO(const u64 *rec, int m) { return or_d(rec, kOrScal + m); }
 __device__ __forceinline__ double or_sumQO(const u64 *rec, int m) { return or_d(rec, kOrScal + 5 + m); }
 __device__ __forceinline__ float or_maxP(const u64 *rec, int m) { return reinterpret_cast<const float *>(rec + kOrScal)[20 + m]; }
-__device__ __forceinline__ float or_maxQ(const u64 *rec, int m) { return reinterpret_cast<const float *>(rec + kOrScal)[25 + m]; }
+__device__ __forceinline__ float or_maxQ(const u64 *rec, int m) { return reinterpret_cast<const float *>(rec + kOrScal)[26 + m]; }
 
 // l == L stages the head's scalars only.
-template <int FT>
+template <int FT, int PARTS>
 __device__ __forceinline__ void stage_owner_record(const DArgs &a, int l, int g, int G, int C, u64 *own_lds, int tid) {
     u64 *dst = own_lds + (l & 1) * kOrSlots;
     const bool layer = l < a.m.L;
@@ -336,7 +336,33 @@ __device__ __forceinline__ void stage_owner_record(const DArgs &a, int l, int g,
             const int k = (t - kOrState) >> 4, n = (t - kOrState) & 15;
             if (layer) v = (u64)__double_as_longlong(a.state[((size_t)l * 5 + 2 + k) * C + 16 * g + n]);
         } else if (t < kOrScal + 16) {
-            v = reinterpret_cast<const u64 *>(a.m.sc + l)[t - kOrScal];
+            // slots 0-4 sum PO, 5-9 sum QO, 10-12 max P, 13-15 max Q (float pairs); the per-token
+            // ones of a layer are the combination, in a fixed order, of its parts
+            const int sidx = t - kOrScal;
+            v = reinterpret_cast<const u64 *>(a.m.sc + l)[sidx];
+            const bool per_token = (sidx >= 5 && sidx < 10) || sidx >= 13;
+            if (layer && per_token) {
+                const DScal *sp = a.m.scp + (size_t)l * PARTS;
+                if (sidx < 10) {
+                    double part[PARTS];
+#pragma unroll
+                    for (int q = 0; q < PARTS; ++q) part[q] = sp[q].sumQO[sidx - 5];     // independent loads
+                    double acc = 0.0;
+#pragma unroll
+                    for (int q = 0; q < PARTS; ++q) acc += part[q];
+                    v = (u64)__double_as_longlong(acc);
+                } else {
+                    const int i0 = 2 * (sidx - 13), i1 = i0 + 1 < kLnMats ? i0 + 1 : i0;
+                    float plo[PARTS], phi[PARTS];
+#pragma unroll
+                    for (int q = 0; q < PARTS; ++q) { plo[q] = sp[q].maxQ[i0]; phi[q] = sp[q].maxQ[i1]; }
+                    float lo = 0.f, hi = 0.f;
+#pragma unroll
+                    for (int q = 0; q < PARTS; ++q) { lo = fmaxf(lo, plo[q]); hi = fmaxf(hi, phi[q]); }
+                    if (i0 + 1 >= kLnMats) hi = 0.f;
+                    v = ((u64)__float_as_uint(hi) << 32) | (u64)__float_as_uint(lo);
+                }
+            }
         }
         dst[t] = v;
     }
@@ -451,7 +477,7 @@ template <int KW, int FW, int NQT>
 __device__ __forceinline__ void vec_front(Front &fx, int &seq, const u64 *src, const u64 *rec, int nq, unsigned epoch,
                                           signed char *dig, int plane_stride, double *stat, long long *tr) {
     constexpr int G = 32 * KW, NG = (G + 63) / 64, FT = 64 * FW;
-    constexpr int CH = NQT <= 5 ? NQT : 3, NCH = (NQT + CH - 1) / CH;
+    constexpr int CH = NQT <= 5 ? NQT : ((NQT + 1) / 2 <= 5 ? (NQT + 1) / 2 : 3), NCH = (NQT + CH - 1) / CH;
     fx.refresh();
     ++seq;
     u64 w[NCH > 1 ? 2 : 1][CH][4];
@@ -515,7 +541,7 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
 #define RWKV_IDS() do { fx.refresh(); lane = fx.lane; n = lane & 15; row = lane >> 4; c_own = 16 * g + n; } while (0)
     RWKV_IDS();
 
-    stage_owner_record<FT>(a, 0, g, G, C, own_lds, fx.tid);   // read after the first barriers below
+    stage_owner_record<FT, KW>(a, 0, g, G, C, own_lds, fx.tid);   // read after the first barriers below
     // the residual value of the own channels lives in LDS between the epilogues (rf_lds[16 + n])
     double *x_lds = rf_lds + 16;
     if (fin && row == 0) x_lds[n] = a.m.X0[c_own];
@@ -584,7 +610,7 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
         ln_front<KW, FW, 2>(fx, seq, a, P32, Q32, rec, 3, e + 2u, dig, stat, tr ? tr + 9 : nullptr);   // [0] ffn_k, [1] ffn_r
         if (!fx.ok) break;
         RWKV_IDS();
-        stage_owner_record<FT>(a, l + 1, g, G, C, own_lds, fx.tid);   // while the matrix cores run (l + 1 == L: the head's scalars)
+        stage_owner_record<FT, KW>(a, l + 1, g, G, C, own_lds, fx.tid);   // while the matrix cores run (l + 1 == L: the head's scalars)
         __syncthreads();
         if (tr) tr[11] = wall_clock64();
         if (fin) {
@@ -647,7 +673,7 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
     RWKV_IDS();
 #undef RWKV_IDS
     unsigned par = 0;
-    constexpr int NS = kBackHeadSlots;                   // head tiles per barrier round
+    constexpr int NS = BackCfg<KW, FW>::NS;               // head tiles per barrier round
     double Sh;
     float invSh;
     ln_scale(stat, rec_h, 0, 0, Sh, invSh);
@@ -675,7 +701,7 @@ struct DecodeLds {
     // the generated back-wave program addresses LDS by these offsets
     static_assert(BackCfg<KW, FW>::RED == DIG_BYTES, "parked tiles follow the digit planes");
     static_assert(BackCfg<KW, FW>::FLAG == DIG_BYTES + RED_BYTES + STAT_BYTES + RF_BYTES + FLAG_ABORT * 4, "abort flag offset");
-    static_assert(RED_SLOTS >= 5 && RED_SLOTS >= 2 * kBackHeadSlots, "park slots");
+    static_assert(RED_SLOTS >= 5 && RED_SLOTS >= 2 * BackCfg<KW, FW>::NS, "park slots");
 };
 
 template <int KW, int FW, bool TRACE>
@@ -745,40 +771,39 @@ __device__ __forceinline__ void prep_block_max(float (&v)[N], float *scr) {
     }
 }
 
-__global__ void __launch_bounds__(kPrepThreads) prep_kernel(const DArgs a) {
-    __shared__ double scr[8 * (kPrepThreads / 64)];
-    const int C = a.m.C, L = a.m.L, G = a.m.G;
-    const int l = blockIdx.x;
-    if (l < L) {
-        const DPrep &p = a.m.prep[l];
-        const double *sl = a.state + (size_t)l * 5 * C;
-        double sq[kLnMats] = {0, 0, 0, 0, 0};
-        float mq[kLnMats] = {0, 0, 0, 0, 0};
-        for (int c = threadIdx.x; c < C; c += kPrepThreads) {
+// Channels [512 part, 512 part + 512) of layer l: Q32 and this part's share of the scalars.
+__device__ __forceinline__ void prep_layer_part(const DArgs &a, int l, int part, double *scr) {
+    const int C = a.m.C, KWr = C / kPrepThreads;
+    const DPrep &p = a.m.prep[l];
+    const double *sl = a.state + (size_t)l * 5 * C;
+    const int c = part * kPrepThreads + threadIdx.x;
+    double sq[kLnMats];
+    float mq[kLnMats];
+    const double sh0 = sl[c], sh1 = sl[(size_t)C + c], b1 = p.ln1_b[c], b2 = p.ln2_b[c];
 #pragma unroll
-            for (int m = 0; m < kLnMats; ++m) {
-                const bool att = m < 3;
-                const double mu = att ? p.att_mix[(size_t)m * C + c] : p.ffn_mix[(size_t)(m - 3) * C + c];
-                const double sh = att ? sl[c] : sl[(size_t)C + c];
-                const double b = att ? p.ln1_b[c] : p.ln2_b[c];
-                const double base = b * mu + sh * (1.0 - mu);                    // block.py:67,91 without the x term
-                const double rg = (double)p.range[m][c];
-                const float q = (float)(base * rg);
-                a.m.Q32[((size_t)l * kLnMats + m) * C + c] = q;
-                sq[m] += base * (p.offset[m][c] + 128.0 * rg);
-                mq[m] = fmaxf(mq[m], fabsf(q));
-            }
-        }
-        prep_block_sum<kLnMats>(sq, scr);
-        prep_block_max<kLnMats>(mq, reinterpret_cast<float *>(scr));
-        if (threadIdx.x < kLnMats) {
-            a.m.sc[l].sumQO[threadIdx.x] = sq[threadIdx.x];
-            a.m.sc[l].maxQ[threadIdx.x] = mq[threadIdx.x];
-        }
-        return;
+    for (int m = 0; m < kLnMats; ++m) {
+        const bool att = m < 3;
+        const double mu = att ? p.att_mix[(size_t)m * C + c] : p.ffn_mix[(size_t)(m - 3) * C + c];
+        const double base = (att ? b1 : b2) * mu + (att ? sh0 : sh1) * (1.0 - mu);   // block.py:67,91 without the x term
+        const double rg = (double)p.range[m][c];
+        const float q = (float)(base * rg);
+        a.m.Q32[((size_t)l * kLnMats + m) * C + c] = q;
+        sq[m] = base * (p.offset[m][c] + 128.0 * rg);
+        mq[m] = fabsf(q);
     }
-    // x0 = ln0(emb[token]); C is a multiple of 64 and thread t takes channels t, t + 512, ...
-    int64_t tok = a.token[0];
+    prep_block_sum<kLnMats>(sq, scr);
+    prep_block_max<kLnMats>(mq, reinterpret_cast<float *>(scr));
+    if (threadIdx.x < kLnMats) {
+        DScal &d = a.m.scp[(size_t)l * KWr + part];
+        d.sumQO[threadIdx.x] = sq[threadIdx.x];
+        d.maxQ[threadIdx.x] = mq[threadIdx.x];
+    }
+}
+
+// x0 = ln0(emb[tok]) (emb.py:9, opt.py:63-64), published with its LayerNorm records as the input
+// of layer 0 under `epoch`.  C is a multiple of 512 and thread t takes channels t, t + 512, ...
+__device__ __forceinline__ void prep_token(const DArgs &a, int64_t tok, unsigned epoch, double *scr) {
+    const int C = a.m.C, G = a.m.G;
     if (tok < 0) tok = 0;
     if (tok >= a.m.V) tok = a.m.V - 1;
     double s[2] = {0.0, 0.0};
@@ -791,19 +816,89 @@ __global__ void __launch_bounds__(kPrepThreads) prep_kernel(const DArgs a) {
     double var = s[1] / (double)C - mean * mean;
     if (var < 0.0) var = 0.0;
     const double rsd = 1.0 / sqrt(var + 1e-5);
-    for (int c0 = 0; c0 < C; c0 += kPrepThreads) {
-        const int c = c0 + threadIdx.x;
-        if (c < C) {                                        // whole waves are in or out: C % 64 == 0
-            const double v = (double)a.m.emb[(size_t)tok * C + c];
-            const double x0 = a.m.ln0_w[c] * ((v - mean) * rsd) + a.m.ln0_b[c];
-            a.m.X0[c] = x0;
-            float P[3];
-            double PO[3];
+    for (int c = threadIdx.x; c < C; c += kPrepThreads) {     // whole waves are in or out: C % 64 == 0
+        const double v = (double)a.m.emb[(size_t)tok * C + c];
+        const double x0 = a.m.ln0_w[c] * ((v - mean) * rsd) + a.m.ln0_b[c];
+        a.m.X0[c] = x0;
+        float P[3];
+        double PO[3];
 #pragma unroll
-            for (int m = 0; m < 3; ++m) { P[m] = a.m.P32[(size_t)m * C + c]; PO[m] = a.m.PO[(size_t)m * C + c]; }
-            publish_ln_input<3>(a.b.X, a.b.XR, G, c >> 4, c & 15, a.epoch0, x0, P, PO);
-        }
+        for (int m = 0; m < 3; ++m) { P[m] = a.m.P32[(size_t)m * C + c]; PO[m] = a.m.PO[(size_t)m * C + c]; }
+        publish_ln_input<3>(a.b.X, a.b.XR, G, c >> 4, c & 15, epoch, x0, P, PO);
     }
+}
+
+// grid: L * (C / 512) layer parts, then one block for the token.
+__global__ void __launch_bounds__(kPrepThreads) prep_kernel(const DArgs a) {
+    __shared__ double scr[8 * (kPrepThreads / 64)];
+    const int parts = a.m.C / kPrepThreads;
+    const int b = blockIdx.x;
+    if (b < a.m.L * parts) prep_layer_part(a, b / parts, b % parts, scr);
+    else prep_token(a, a.token[0], a.epoch0, scr);
+}
+
+// Between two greedy tokens: argmax of the logits just produced -> out_token[0], and the
+// preparation of the next step (which reads the state the step before has just updated) in the same
+// launch.  grid: L * (C / 512) layer parts, then kArgmaxBlocks blocks that scan the logits; the one
+// that finishes last reduces their results, writes the token and prepares it.  a.epoch0: the epoch
+// of the NEXT token step.
+constexpr int kArgmaxBlocks = 32;
+
+__global__ void __launch_bounds__(kPrepThreads) next_token_kernel(const DArgs a, int64_t *__restrict__ out_token) {
+    __shared__ double scr[8 * (kPrepThreads / 64)];
+    __shared__ int sidx[kPrepThreads / 64];
+    __shared__ int last_flag;
+    const int parts = a.m.C / kPrepThreads;
+    const int b = blockIdx.x;
+    if (b < a.m.L * parts) { prep_layer_part(a, b / parts, b % parts, scr); return; }
+    const int ab = b - a.m.L * parts, V = a.m.V;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    auto better = [](double v, int i, double bv, int bi) { return v > bv || (v == bv && i < bi); };
+    auto block_argmax = [&](double &best, int &bi) {        // result in thread 0
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            const double ob = __shfl_xor(best, off, 64);
+            const int oi = __shfl_xor(bi, off, 64);
+            if (better(ob, oi, best, bi)) { best = ob; bi = oi; }
+        }
+        __syncthreads();
+        if (lane == 0) { scr[wave] = best; sidx[wave] = bi; }
+        __syncthreads();
+        if (threadIdx.x == 0)
+            for (int wv = 1; wv < kPrepThreads / 64; ++wv)
+                if (better(scr[wv], sidx[wv], best, bi)) { best = scr[wv]; bi = sidx[wv]; }
+    };
+    double best = -INFINITY;
+    int bi = 0x7fffffff;
+    const int chunk = (V + kArgmaxBlocks - 1) / kArgmaxBlocks;
+    const int i1 = (ab + 1) * chunk < V ? (ab + 1) * chunk : V;
+    for (int i = ab * chunk + threadIdx.x; i < i1; i += kPrepThreads) {
+        const double x = a.logits[i];
+        if (better(x, i, best, bi)) { best = x; bi = i; }
+    }
+    block_argmax(best, bi);
+    if (threadIdx.x == 0) {
+        a.m.amax_val[ab] = best;
+        a.m.amax_idx[ab] = bi;
+        __threadfence();
+        last_flag = atomicAdd(a.m.amax_count, 1u) == kArgmaxBlocks - 1;
+    }
+    __syncthreads();
+    if (!last_flag) return;
+    __threadfence();
+    best = -INFINITY; bi = 0x7fffffff;
+    if (threadIdx.x < kArgmaxBlocks) {
+        best = __hip_atomic_load(a.m.amax_val + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        bi = __hip_atomic_load(a.m.amax_idx + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    block_argmax(best, bi);
+    if (threadIdx.x == 0) {
+        sidx[0] = bi == 0x7fffffff ? 0 : bi;
+        out_token[0] = sidx[0];
+        *a.m.amax_count = 0u;                                // ready for the next launch
+    }
+    __syncthreads();
+    prep_token(a, (int64_t)sidx[0], a.epoch0, scr);
 }
 
 // ---------------------------------------------------------------------------
@@ -969,7 +1064,7 @@ unsigned decode_epochs_per_token(int64_t L) { return (unsigned)(4 * L + 1); }
 
 namespace {
 struct BlockPlan {
-    size_t layers, prep, P32, Q32, PO, sc, X0, cs, ownrec, jt, xchg, abort, total;
+    size_t layers, prep, P32, Q32, PO, sc, X0, cs, ownrec, jt, scp, amax, xchg, abort, total;
     size_t cs_layer_ints;
 };
 BlockPlan plan_block(int64_t L, int64_t C, int64_t F, int64_t V) {
@@ -988,6 +1083,8 @@ BlockPlan plan_block(int64_t L, int64_t C, int64_t F, int64_t V) {
     p.cs = take(((size_t)L * p.cs_layer_ints + (size_t)round_up(V, 16)) * sizeof(int));
     p.ownrec = take((size_t)L * G * kOrSlots * sizeof(u64));
     p.jt = take(G * (size_t)(L + 1) * 16 * sizeof(u64));
+    p.scp = take((size_t)L * (C / 512) * sizeof(DScal));
+    p.amax = take(kArgmaxBlocks * (sizeof(double) + sizeof(int)) + 64);
     p.xchg = take(((size_t)2 * C + F + (size_t)(kLnRows + 6) * G) * sizeof(u64));
     p.abort = take(256);
     p.total = off;
@@ -1043,6 +1140,10 @@ int decode_setup(void *block, const DSetup &s, DModel *dm, DecodeBuffers *db) {
     dm->emb = s.emb; dm->ln0_w = s.ln0_w; dm->ln0_b = s.ln0_b;
     dm->w_head = s.head.w16; dm->cs = cs; dm->cs_head = cs_head;
     dm->ownrec = reinterpret_cast<const u64 *>(base + p.ownrec);
+    dm->scp = reinterpret_cast<DScal *>(base + p.scp);
+    dm->amax_val = reinterpret_cast<double *>(base + p.amax);
+    dm->amax_idx = reinterpret_cast<int *>(base + p.amax + kArgmaxBlocks * sizeof(double));
+    dm->amax_count = reinterpret_cast<unsigned *>(base + p.amax + kArgmaxBlocks * (sizeof(double) + sizeof(int)));
     dm->layers = reinterpret_cast<const DLayer *>(base + p.layers);
     dm->prep = reinterpret_cast<const DPrep *>(base + p.prep);
     dm->P32 = reinterpret_cast<float *>(base + p.P32);
@@ -1079,7 +1180,7 @@ int decode_setup(void *block, const DSetup &s, DModel *dm, DecodeBuffers *db) {
 }
 
 template <int KW, int FW>
-static int launch_one(hipStream_t st, const DArgs &args) {
+static int launch_one(hipStream_t st, const DArgs &args, bool with_prep) {
     constexpr int lds = DecodeLds<KW, FW>::TOTAL;
     static bool configured = false;
     if (!configured) {
@@ -1089,7 +1190,8 @@ static int launch_one(hipStream_t st, const DArgs &args) {
                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         configured = true;
     }
-    hipLaunchKernelGGL(prep_kernel, dim3((unsigned)(args.m.L + 1)), dim3(kPrepThreads), 0, st, args);
+    if (with_prep)
+        hipLaunchKernelGGL(prep_kernel, dim3((unsigned)(args.m.L * (args.m.C / kPrepThreads) + 1)), dim3(kPrepThreads), 0, st, args);
     if (args.b.trace)
         hipLaunchKernelGGL((decode_kernel<KW, FW, true>), dim3((unsigned)args.m.G), dim3((FW + kBW) * 64), lds, st, args);
     else
@@ -1098,17 +1200,41 @@ static int launch_one(hipStream_t st, const DArgs &args) {
     return RWKV_OK;
 }
 
+static int launch_step(hipStream_t st, const DArgs &args, bool with_prep) {
+    switch (args.m.C) {
+        case 1024: return launch_one<2, 4>(st, args, with_prep);
+        case 2048: return launch_one<4, 4>(st, args, with_prep);
+        case 2560: return launch_one<5, 8>(st, args, with_prep);
+        case 4096: return launch_one<8, 4>(st, args, with_prep);
+        default: return set_error(RWKV_ERR_SIZE, "decode kernel: n_embd %d not supported", args.m.C);
+    }
+}
+
 int decode_launch(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsigned epoch0,
                   const int64_t *token, double *state, double *logits) {
     DArgs args;
     args.m = m; args.b = b; args.epoch0 = epoch0; args.token = token; args.state = state; args.logits = logits;
-    switch (m.C) {
-        case 1024: return launch_one<2, 4>(st, args);
-        case 2048: return launch_one<4, 4>(st, args);
-        case 2560: return launch_one<5, 4>(st, args);
-        case 4096: return launch_one<8, 4>(st, args);
-        default: return set_error(RWKV_ERR_SIZE, "decode kernel: n_embd %d not supported", m.C);
+    return launch_step(st, args, true);
+}
+
+int decode_launch_greedy(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsigned epoch0,
+                         int64_t *tokens, int64_t n, double *state, double *logits) {
+    DArgs args;
+    args.m = m; args.b = b; args.state = state; args.logits = logits;
+    const unsigned ept = decode_epochs_per_token(m.L);
+    for (int64_t i = 0; i < n; ++i) {
+        args.epoch0 = epoch0 + (unsigned)i * ept;
+        args.token = tokens + i;
+        const int rc = launch_step(st, args, i == 0);
+        if (rc) return rc;
+        // argmax -> tokens[i + 1], and the preparation of step i + 1 (harmless after the last step:
+        // the next forward call prepares again under the same epoch)
+        args.epoch0 += ept;
+        hipLaunchKernelGGL(next_token_kernel, dim3((unsigned)(m.L * (m.C / kPrepThreads) + kArgmaxBlocks)),
+                           dim3(kPrepThreads), 0, st, args, tokens + i + 1);
+        RWKV_CHECK_LAUNCH("next_token_kernel");
     }
+    return RWKV_OK;
 }
 
 }  // namespace rwkv

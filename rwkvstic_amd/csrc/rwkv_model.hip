@@ -779,9 +779,13 @@ int rwkv_model_decode_greedy(rwkv_model *m, rwkv_stream_t stream, int64_t *token
     if (rc) return rc;
     RWKV_CHECK_ARG(n > 0, "rwkv_model_decode_greedy: n must be positive");
     const Workspace w = carve(workspace, m->d.n_embd, m->d.n_ffn);
+    if (m->fused) {
+        rc = decode_launch_greedy((hipStream_t)stream, m->dm, m->db, m->epoch, tokens, n, state, logits);
+        m->epoch += (unsigned)n * decode_epochs_per_token(m->d.n_layer);
+        return rc;
+    }
     for (int64_t i = 0; i < n; ++i) {
-        if (m->fused) rc = fused_token(m, (hipStream_t)stream, tokens + i, state, logits);
-        else rc = step_token(m, (hipStream_t)stream, tokens + i, state, logits, w, true);
+        rc = step_token(m, (hipStream_t)stream, tokens + i, state, logits, w, true);
         if (rc) return rc;
         rc = rwkv_argmax_f64(stream, logits, m->d.n_vocab, tokens + i + 1);
         if (rc) return rc;
