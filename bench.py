@@ -71,6 +71,9 @@ def main() -> int:
     ap.add_argument("--shape", default="3B", choices=["169M", "3B", "14B"])
     ap.add_argument("--prefill", type=int, default=1024)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy-mib", type=int, default=0,
+                    help="before the workload, copy this many MiB device to device once (a kernel of known HBM "
+                         "traffic: the yardstick for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (batch-1 decode of one model replica); "
@@ -93,6 +96,15 @@ def main() -> int:
 
     stream = torch.cuda.current_stream()
     ev = lambda: torch.cuda.Event(enable_timing=True)
+
+    if args.calibrate_copy_mib > 0:
+        n = args.calibrate_copy_mib << 20
+        src = torch.full((n,), 3, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)                    # one elementwise copy kernel: reads n bytes, writes n bytes
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- prefill -------------------------------------------------------------
     prompt = synth.random_tokens(args.prefill, V=V, seed=0).cuda()

@@ -35,7 +35,9 @@ S_CUR, S_NXT = 36, 64
 S_L, S_T, S_JT, S_TILE, S_RT, S_RP, S_PAR = 90, 91, 92, 94, 95, 96, 99
 PF = NA - 1       # A-operand reads run this many positions ahead
 import os
-WINDOW = int(os.environ.get("RWKV_BACK_WINDOW", "4"))   # weight loads a wave keeps in flight while it reloads slots
+WINDOW = int(os.environ.get("RWKV_BACK_WINDOW", "4"))
+DEFER = int(os.environ.get("RWKV_BACK_DEFER", "1"))
+SLEEP = int(os.environ.get("RWKV_BACK_SLEEP", "0"))      # s_sleep units (64 cycles) between a phase's barrier and its reloads   # weight loads a wave keeps in flight while it reloads slots
 
 
 class Emit:
@@ -203,7 +205,7 @@ def gen(KW, R, NV, NSH):
             first = (b == 0) and not (j > 9)
             acc = "0" if first else f"v[{dreg}:{dreg + 3}]"
             e(f"v_mfma_i32_16x16x64_i8 v[{dreg}:{dreg + 3}], {abuf(p)}, {ring(p % R)}, {acc}")
-            if p + R < pe:
+            if p + R < pe or not DEFER:
                 assert issued_loads == p + R
                 layer_reload(p)
                 issued_loads += 1
@@ -217,6 +219,8 @@ def gen(KW, R, NV, NSH):
         e.drain_state()
         if pe == NREAL:
             deferred += list(range(NREAL, PP))     # padding positions: nothing to compute, only their turn to load
+        if SLEEP and deferred:
+            e(f"s_sleep {SLEEP}")
         for p in deferred:
             assert issued_loads == p + R
             layer_reload(p)
@@ -292,7 +296,7 @@ def gen(KW, R, NV, NSH):
             e(f"s_waitcnt vmcnt({nvm}) lgkmcnt({allow})")
             acc = "0" if b == 0 else f"v[{dreg}:{dreg + 3}]"
             e(f"v_mfma_i32_16x16x64_i8 v[{dreg}:{dreg + 3}], v[{V_A + 4 * (b % NA)}:{V_A + 4 * (b % NA) + 3}], {ring(q % R)}, {acc}")
-            if q + R < pe:
+            if q + R < pe or not DEFER:
                 assert issued_loads == q + R
                 head_reload(q)
                 issued_loads += 1

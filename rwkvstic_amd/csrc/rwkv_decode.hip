@@ -526,7 +526,7 @@ __device__ __forceinline__ void vec_front(Front &fx, int &seq, const u64 *src, c
 // =============================================================================
 template <int KW, int FW, bool TRACE>
 __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, const v4i *red, double *stat, double *rf_lds,
-                                           lds_flag_t *flags, u64 *own_lds) {
+                                           lds_flag_t *flags, u64 *own_lds, double *st_lds) {
     constexpr int C = 512 * KW, F = 4 * C, G = 32 * KW, FT = 64 * FW;
     constexpr int PS = C + 64, PSF = F + 64;
     constexpr int NQH = F / 4, NQTH = (NQH + FT - 1) / FT, NQC = C / 4, NQTC = (NQC + FT - 1) / FT;
@@ -548,7 +548,10 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
 
     for (int l = 0; l < L && fx.ok; ++l) {
         const u64 *rec = own_lds + (l & 1) * kOrSlots;
-        double *sl = a.state + (size_t)l * 5 * C;
+        // New state rows of the own channels are collected in LDS and written out once, after the
+        // head: nobody else reads them during this token, and a store issued here would queue in
+        // the compute unit's memory pipeline behind the weight stream, in front of the exchange.
+        double *sl = st_lds + (size_t)l * 5 * 16;
         const unsigned e = a.epoch0 + 4u * (unsigned)l;
         long long *tr = trace ? trace + (size_t)l * kTraceStampsPerLayer : nullptr;
         const float *P32 = a.m.P32 + (size_t)l * kLnMats * C, *Q32 = a.m.Q32 + (size_t)l * kLnMats * C;
@@ -582,11 +585,11 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
                 const double so = row16_sum(av * or_d(rec, OR_OFFO * 16 + n) + 128.0 * (double)xs);
                 const float hi = (float)so, lo = (float)(so - (double)hi);
                 if (n < 3) put_word(a.b.AR + (size_t)n * G + g, e + 1u, n == 0 ? mx : (n == 1 ? hi : lo));
-                sl[2 * (size_t)C + c_own] = (double)aa;
-                sl[3 * (size_t)C + c_own] = (double)bb;
-                sl[4 * (size_t)C + c_own] = pp;
+                sl[2 * 16 + n] = (double)aa;
+                sl[3 * 16 + n] = (double)bb;
+                sl[4 * 16 + n] = pp;
                 xy1 = or_d(rec, OR_LN1W * 16 + n) * ((x_lds[n] - stat[0]) * stat[1]) + or_d(rec, OR_LN1B * 16 + n);   // block.py:58
-                sl[c_own] = xy1;                                                 // block.py:63-64
+                sl[n] = xy1;                                                     // block.py:63-64
             }
         }
         if (tr) tr[4] = wall_clock64();
@@ -635,7 +638,7 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
                 const double yr = finish_col(red, 0, n, Sr, (int)or_hi(rec, OR_CSR_CSFR * 16 + n), ln_zp(stat, rec, 3, 1));
                 rf_lds[n] = (double)sigmoid_f32((float)yr);                      // block.py:95
                 // the LayerNorm output of the own channel is the new ffn shift state (block.py:82,87-88)
-                sl[(size_t)C + c_own] = or_d(rec, OR_LN2W * 16 + n) * ((x_lds[n] - stat[0]) * stat[1]) + or_d(rec, OR_LN2B * 16 + n);
+                sl[16 + n] = or_d(rec, OR_LN2W * 16 + n) * ((x_lds[n] - stat[0]) * stat[1]) + or_d(rec, OR_LN2B * 16 + n);
             }
         }
         if (tr) tr[12] = wall_clock64();
@@ -686,6 +689,8 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
             if (v < V) a.logits[v] = finish_col(red + par * (NS * kBW * 16), s, n, Sh, a.m.cs_head[v], zph);
         }
     }
+    // the state rows of the own channels: st_lds[l][row][n] -> state[l][row][16 g + n]
+    for (int i = fx.tid; i < L * 5 * 16; i += FT) a.state[(size_t)(i >> 4) * C + 16 * g + (i & 15)] = st_lds[i];
 }
 
 template <int KW, int FW>
@@ -697,7 +702,8 @@ struct DecodeLds {
     static constexpr int RED_BYTES = RED_SLOTS * kBW * 16 * 16;
     static constexpr int STAT_BYTES = 32 * 8, RF_BYTES = 32 * 8, FLAG_BYTES = FLAG_COUNT * 4;   // RF: gate and residual of the own channels
     static constexpr int OWN_OFFSET = DIG_BYTES + RED_BYTES + STAT_BYTES + RF_BYTES + FLAG_BYTES;
-    static constexpr int TOTAL = OWN_OFFSET + 2 * kOrSlots * 8;
+    static constexpr int STATE_OFFSET = OWN_OFFSET + 2 * kOrSlots * 8;
+    static int total(int L) { return STATE_OFFSET + L * 5 * 16 * 8; }       // + the new state rows of the own channels
     // the generated back-wave program addresses LDS by these offsets
     static_assert(BackCfg<KW, FW>::RED == DIG_BYTES, "parked tiles follow the digit planes");
     static_assert(BackCfg<KW, FW>::FLAG == DIG_BYTES + RED_BYTES + STAT_BYTES + RF_BYTES + FLAG_ABORT * 4, "abort flag offset");
@@ -717,7 +723,8 @@ __global__ void __launch_bounds__((FW + kBW) * 64) decode_kernel(const DArgs a) 
     __syncthreads();
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     if (wave < FW) {
-        front_path<KW, FW, TRACE>(a, dig, red, stat, rf_lds, flags, reinterpret_cast<u64 *>(smem + Lds::OWN_OFFSET));
+        front_path<KW, FW, TRACE>(a, dig, red, stat, rf_lds, flags, reinterpret_cast<u64 *>(smem + Lds::OWN_OFFSET),
+                                  reinterpret_cast<double *>(smem + Lds::STATE_OFFSET));
     } else {
         constexpr int G = 32 * KW;
         const int v_tiles = (a.m.V + 15) / 16, head_rounds = (v_tiles + G - 1) / G;
@@ -1181,14 +1188,15 @@ int decode_setup(void *block, const DSetup &s, DModel *dm, DecodeBuffers *db) {
 
 template <int KW, int FW>
 static int launch_one(hipStream_t st, const DArgs &args, bool with_prep) {
-    constexpr int lds = DecodeLds<KW, FW>::TOTAL;
-    static bool configured = false;
-    if (!configured) {
+    const int lds = DecodeLds<KW, FW>::total(args.m.L);
+    if (lds > 160 * 1024) return set_error(RWKV_ERR_SIZE, "decode kernel: %d layers need %d bytes of LDS", args.m.L, lds);
+    static int configured = 0;
+    if (configured < lds) {
         RWKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_kernel<KW, FW, false>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         RWKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_kernel<KW, FW, true>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        configured = true;
+        configured = lds;
     }
     if (with_prep)
         hipLaunchKernelGGL(prep_kernel, dim3((unsigned)(args.m.L * (args.m.C / kPrepThreads) + 1)), dim3(kPrepThreads), 0, st, args);

@@ -52,3 +52,26 @@ def test_host_side_validation_without_gpu(lib):
     assert lib.rwkv_mm8_one(None, 128, 8, 16, 16, 8, 16, 16, None, 0) == -4               # no workspace
     assert lib.rwkv_model_create(None, None) == -1
     assert lib.rwkv_model_workspace_bytes(None, 1) == 0
+
+
+def test_generated_back_wave_program_is_current():
+    """csrc/rwkv_decode_back.inc is generated; the committed file must be what the generator writes."""
+    import subprocess
+    import sys
+    csrc = os.path.join(ROOT, "rwkvstic_amd", "csrc")
+    env = {k: v for k, v in os.environ.items() if k != "RWKV_BACK_WINDOW"}
+    out = subprocess.run([sys.executable, os.path.join(csrc, "gen_decode_back.py")], capture_output=True, text=True,
+                         check=True, env=env).stdout
+    assert out == open(os.path.join(csrc, "rwkv_decode_back.inc")).read()
+
+
+def test_single_token_kernels_do_not_spill_ring_registers():
+    """The back-wave program reloads fixed registers in place behind the compiler's back; that is only sound while
+    the compiler neither spills nor copies them, i.e. while the asm statement owns them outright.  The check here
+    is on the source: every register of the ring is on the statement's clobber list."""
+    inc = open(os.path.join(ROOT, "rwkvstic_amd", "csrc", "rwkv_decode_back.inc")).read()
+    for block in inc.split("template <> struct BackCfg<")[1:]:
+        regs = set(int(x) for x in re.findall(r"global_load_dwordx4 v\[(\d+):", block))
+        regs |= set(r + i for r in list(regs) for i in range(4))
+        clob = set(int(x) for x in re.findall(r'"v(\d+)"', block))
+        assert regs and regs <= clob

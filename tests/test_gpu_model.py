@@ -171,6 +171,32 @@ def test_fused_step_matches_oracle_and_phase_kernels(C, L, V):
     assert torch.equal(l2, lg) and torch.equal(s2, sg)
 
 
+def test_fused_greedy_device_loop_matches_host_loop():
+    """rwkv_model_decode_greedy on the persistent kernel: argmax and the preparation of the next step run in one
+    launch between the token kernels; tokens, logits and state must equal forward() + host argmax, bit for bit
+    (rwkvMaster.py:28-56 with the sampler replaced by argmax)."""
+    from rwkvstic_amd.model import HipRWKV
+    sd = synth.make_state_dict(2, 1024, 4096, 1999, seed=77)
+    hip = HipRWKV(sd)
+    assert hip.fused_step
+    s1 = hip.emptyState.clone()
+    _, s1 = hip.forward(synth.random_tokens(3, V=1999, seed=9).tolist(), s1)      # a non-trivial starting state
+    s2 = s1.clone()
+    toks, logits, s1 = hip.decode_greedy(17, 9, s1)
+    hip.check()
+    t, out = 17, []
+    for _ in range(9):
+        l2, s2 = hip.forward([t], s2)
+        t = int(l2.argmax()); out.append(t)
+    hip.check()
+    assert toks.tolist() == out
+    assert torch.equal(logits, l2) and torch.equal(s1, s2)
+    # the loop leaves the model usable for plain steps (its last launch prepared a step that is prepared again)
+    l3, s3 = hip.forward([out[-1]], s2.clone())
+    toks4, l4, s4 = hip.decode_greedy(out[-1], 1, s1.clone())
+    assert torch.equal(l3, l4) and torch.equal(s3, s4)
+
+
 @pytest.mark.parametrize("n_prompt", [23, 100])      # 100: the chunked WKV scan (3 full chunks + a partial one)
 def test_prompt_gemm_path_matches_token_steps(tiny, n_prompt):
     """A prompt through the GEMM path leaves the same logits and state as the same tokens fed one at a time
