@@ -22,6 +22,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E vendor peak
 
+# HBM bytes per launch of the single-token kernel from rocprofv3 counters (FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB,
+# both scaled by a 1 GiB device copy in the same run): a measured constant per shape, not something this script
+# can read live.  Shapes without a counter run report null.
+PMC_TRAFFIC_BYTES = {"3B": 2_988_900_000}
+
 
 def cpu_baseline(shape, threads: int):
     """The CPU oracle (the reference's torch CPU path restated) on this box's host cores, on a
@@ -160,10 +165,12 @@ def main() -> int:
                    "weight_bytes_per_token": wbytes, "load_seconds": round(load_s, 2)},
         "prefill_tokens_per_s": round(args.prefill / (prefill_ms / 1e3), 1),
         "roofline": {"bound": "hbm",
-                     "kernel": "rwkv::decode_kernel (persistent, one launch per token)" if model.fused_step
+                     "kernel": "rwkv::decode_kernel (persistent, one launch per token; launch_us includes the prep_kernel in front of it)"
+                               if model.fused_step
                                else "decode token step (all phase kernels of one token)",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": PMC_TRAFFIC_BYTES.get(args.shape) if model.fused_step else None,
                      "launch_us": round(step_us, 2), "decode_loop_us_per_token": round(dev_ms / args.steps * 1e3, 2)},
     }
     if not args.no_cpu_baseline:

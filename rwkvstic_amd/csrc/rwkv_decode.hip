@@ -5,8 +5,8 @@
 // small launch of prep_kernel before it turns the token and the shift state
 // into the per-token constants.  The grid is C/16 workgroups, all resident at
 // once; workgroup g owns the 16 channels [16g, 16g+16) for the whole token
-// (their residual value, WKV state and receptance gate live in registers of
-// its first wave) and the matching 16-column tiles of every matrix.
+// (their residual value, WKV state and receptance gate stay in its LDS) and
+// the matching 16-column tiles of every matrix.
 //
 // Dot products.  Weights are streamed as 1 KiB blocks of 16 columns x 64 rows
 // (layout "M16", stored as code - 128) straight into v_mfma_i32_16x16x64_i8 as
@@ -33,12 +33,20 @@
 //
 // Roles.  Vector loads of one wave return in order, so a wave that polls would
 // first drain whatever it had prefetched.  The workgroup is therefore split:
-// "front" waves talk to the other workgroups, do the per-channel arithmetic
-// and write the digit planes to LDS; 8 "back" waves own the weight stream: each
-// keeps a ring of RJ jobs (one job = its share of a 16-column x C-row tile) in
-// registers, refills a slot right after the matrix instruction consumed it and
-// never waits on anything but LDS barriers, so several phases' worth of weight
-// loads stay in flight while the front waves wait for the other workgroups.
+// "front" waves talk to the other workgroups (one of them polls, the others
+// wait on LDS flags), do the per-channel arithmetic, write the digit planes to
+// LDS and finish the 16 owned columns of each product; 8 "back" waves own the
+// weight stream.  A back wave's program is one generated assembly statement
+// (gen_decode_back.py -> rwkv_decode_back.inc): the 1 KiB blocks of its share
+// of the workgroup's 13 tiles per layer form one sequence of positions,
+// position p lives in register slot p % R of a fixed ring that is reloaded in
+// place, and every wait count is known when the program is generated.  A
+// slot's reload (the block R positions ahead, possibly of a later phase or
+// layer) is issued after the barrier that hands the phase's partial sums to
+// the front waves, a few loads at a time, so the reloads do not delay the
+// products and the weight stream keeps running while the front waves wait for
+// the other workgroups.  Back waves wait on nothing but LDS barriers and
+// their own loads.
 #include "rwkv_decode.h"
 
 #include <type_traits>
