@@ -208,10 +208,10 @@ void rwkv_model_destroy(rwkv_model *m);
  * matrices have packed16 and the shape is supported), else 0. */
 int rwkv_model_has_fused_step(const rwkv_model *m);
 
-/* Diagnostics: when device_buffer is non-NULL, workgroup 0 of every following
- * single-token launch writes 100 MHz wall-clock stamps of its phase
- * boundaries (16 per layer, layers back to back) into device_buffer, which
- * must hold 16 * n_layer int64 values; NULL switches it off. */
+/* Diagnostics: when device_buffer is non-NULL, every workgroup g of every
+ * following single-token launch writes 100 MHz wall-clock stamps of its phase
+ * boundaries into device_buffer[g][layer][16], which must hold
+ * (n_embd / 16) * n_layer * 16 int64 values; NULL switches it off. */
 int rwkv_model_set_trace(rwkv_model *m, int64_t *device_buffer);
 
 /* Synchronises the device and returns RWKV_ERR_HIP if a single-token launch

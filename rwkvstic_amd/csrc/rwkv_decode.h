@@ -81,7 +81,7 @@ struct DecodeBuffers {
     u64 *H;                 // [F]       fp32(relu(k)^2 * range_v)
     u64 *HR;                // [3][G]
     unsigned *abort_flag;   // set to 1 by any workgroup whose wait ran out
-    long long *trace;       // optional: workgroup 0 writes 100 MHz timestamps here (null = off)
+    long long *trace;       // optional: [G][L][16] 100 MHz timestamps of every workgroup's phase boundaries (null = off)
 };
 
 // Host-side description from which the tables are built.

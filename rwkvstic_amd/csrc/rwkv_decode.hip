@@ -159,6 +159,13 @@ __device__ __forceinline__ void write_digits4(signed char *dig, int plane_stride
     d[3 * (plane_stride / 4)] = __builtin_amdgcn_perm(y0, x0, 0x05040100u);      // least significant byte
 }
 
+// Value of `v` in lane `src` of the wave (no lane-id arithmetic, unlike __shfl).
+__device__ __forceinline__ double lane_read_f64(double v, int src) {
+    const long long b = __double_as_longlong(v);
+    const int lo = __builtin_amdgcn_ds_bpermute(src << 2, (int)b), hi = __builtin_amdgcn_ds_bpermute(src << 2, (int)(b >> 32));
+    return __longlong_as_double(((long long)hi << 32) | (unsigned)lo);
+}
+
 // ---- tagged exchange ---------------------------------------------------------
 __device__ __forceinline__ void put_word(u64 *dst, unsigned epoch, float v) {
     ASTORE(dst, ((u64)epoch << 32) | (u64)__float_as_uint(v));
@@ -480,7 +487,7 @@ __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, co
 
 // Front side of a product whose input was scaled by its producers (att output, ffn value):
 // the records carry max |xs| and the shares of the zero-point sum.  Leaves the scale in stat[16],
-// the zero-point sum in stat[18].  Ends with the "digits ready" barrier.
+// the zero-point sum in stat[17].  Ends with the "digits ready" barrier.
 template <int KW, int FW, int NQT>
 __device__ __forceinline__ void vec_front(Front &fx, int &seq, const u64 *src, const u64 *rec, int nq, unsigned epoch,
                                           signed char *dig, int plane_stride, double *stat, long long *tr) {
@@ -503,12 +510,12 @@ __device__ __forceinline__ void vec_front(Front &fx, int &seq, const u64 *src, c
         so = wave_sum_dpp(so);
         double S;
         scale_from_amax(mx, S, invS);
-        if (fx.lane == 0) { stat[16] = S; stat[17] = (double)invS; stat[18] = so; fx.flags[FLAG_SCALE] = seq; }
+        if (fx.lane == 0) { stat[16] = S; stat[17] = so; stat[18] = (double)invS; fx.flags[FLAG_SCALE] = seq; }
     } else {
         wait_flag(fx, FLAG_ARRIVED, seq);
         issue_quads<FT, CH>(src, fx.tid, 0, nq, w[0]);
         wait_flag(fx, FLAG_SCALE, seq);
-        invS = (float)stat[17];
+        invS = (float)stat[18];
     }
     if (tr) tr[0] = wall_clock64();
 #pragma unroll
@@ -543,7 +550,7 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
     fx.refresh();
     const int g = blockIdx.x, L = a.m.L, V = a.m.V;
     const bool fin = fx.wave == 0;                       // wave 0 owns the workgroup's 16 channels
-    long long *trace = (TRACE && g == 0 && threadIdx.x == 0) ? a.b.trace : nullptr;
+    long long *trace = (TRACE && threadIdx.x == 0) ? a.b.trace + (size_t)g * L * kTraceStampsPerLayer : nullptr;
     int seq = 0;
     int lane, n, row, c_own;                             // recomputed at the start of every phase
 #define RWKV_IDS() do { fx.refresh(); lane = fx.lane; n = lane & 15; row = lane >> 4; c_own = 16 * g + n; } while (0)
@@ -579,7 +586,7 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
             float invSj;
             ln_scale(stat, rec, 0, j, Sj, invSj);
             const double y = finish_col(red, j, n, Sj, cs1, ln_zp(stat, rec, 0, j));
-            const double yv = __shfl(y, n + 16, 64), yr = __shfl(y, n + 32, 64);
+            const double yv = lane_read_f64(y, n + 16), yr = lane_read_f64(y, n + 32);
             if (row == 0) {
                 const double td = or_d(rec, OR_DECAY * 16 + n), tf = or_d(rec, OR_FIRST * 16 + n);
                 const float r = sigmoid_f32((float)yr);                          // block.py:72
@@ -609,7 +616,7 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
         if (tr) tr[7] = wall_clock64();
         RWKV_IDS();
         if (fin && row == 0) {
-            const double x_own = x_lds[n] + finish_col(red, 0, n, stat[16], (int)or_hi(rec, OR_RNGO_CSO * 16 + n), stat[18]);   // block.py:80
+            const double x_own = x_lds[n] + finish_col(red, 0, n, stat[16], (int)or_hi(rec, OR_RNGO_CSO * 16 + n), stat[17]);   // block.py:80
             x_lds[n] = x_own;
             const float Pf[2] = {__uint_as_float(or_lo(rec, OR_PF * 16 + n)), __uint_as_float(or_hi(rec, OR_PF * 16 + n))};
             const double POf[2] = {or_d(rec, OR_POFK * 16 + n), or_d(rec, OR_POFR * 16 + n)};
@@ -658,7 +665,7 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
         if (tr) tr[15] = wall_clock64();
         RWKV_IDS();
         if (fin && row == 0) {
-            const double y = finish_col(red, 0, n, stat[16], (int)or_lo(rec, OR_CSFV * 16 + n), stat[18]);
+            const double y = finish_col(red, 0, n, stat[16], (int)or_lo(rec, OR_CSFV * 16 + n), stat[17]);
             const double x_own = y * rf_lds[n] + x_lds[n];                       // block.py:100
             x_lds[n] = x_own;
             const float Pn[3] = {__uint_as_float(or_lo(rec, OR_PN01 * 16 + n)), __uint_as_float(or_hi(rec, OR_PN01 * 16 + n)),
