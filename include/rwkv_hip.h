@@ -210,8 +210,8 @@ int rwkv_model_has_fused_step(const rwkv_model *m);
 
 /* Diagnostics: when device_buffer is non-NULL, every workgroup g of every
  * following single-token launch writes 100 MHz wall-clock stamps of its phase
- * boundaries into device_buffer[g][layer][16], which must hold
- * (n_embd / 16) * n_layer * 16 int64 values; NULL switches it off. */
+ * boundaries into device_buffer[g][layer][24], which must hold
+ * (n_embd / 16) * n_layer * 24 int64 values; NULL switches it off. */
 int rwkv_model_set_trace(rwkv_model *m, int64_t *device_buffer);
 
 /* Synchronises the device and returns RWKV_ERR_HIP if a single-token launch

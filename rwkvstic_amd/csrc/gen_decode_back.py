@@ -35,8 +35,9 @@ S_CUR, S_NXT = 36, 64
 S_L, S_T, S_JT, S_TILE, S_RT, S_RP, S_PAR = 90, 91, 92, 94, 95, 96, 99
 PF = NA - 1       # A-operand reads run this many positions ahead
 import os
-WINDOW = int(os.environ.get("RWKV_BACK_WINDOW", "4"))
+WINDOW = int(os.environ.get("RWKV_BACK_WINDOW", "5"))
 DEFER = int(os.environ.get("RWKV_BACK_DEFER", "1"))
+BURST = int(os.environ.get("RWKV_BACK_BURST", "0"))      # the first BURST reloads after a phase's barrier go out back to back
 SLEEP = int(os.environ.get("RWKV_BACK_SLEEP", "0"))      # s_sleep units (64 cycles) between a phase's barrier and its reloads   # weight loads a wave keeps in flight while it reloads slots
 
 
@@ -163,15 +164,15 @@ def gen(KW, R, NV, NSH):
     # that pushing requests into a busy memory system never delays the phase's results.
     phases = [(0, 3 * KW, 2), (3 * KW, 4 * KW, 1), (4 * KW, 9 * KW, 2), (9 * KW, 13 * KW, 1)]   # start, end, barriers before
 
-    def throttle():
+    def throttle(window=WINDOW):
         # A burst of reloads would sit in the compute unit's memory pipeline in front of the front
         # waves' polls and stores; keeping a window in flight paces the requests to what HBM delivers.
-        if WINDOW - 1 < R - 1:
-            e(f"s_waitcnt vmcnt({WINDOW - 1})")
+        if window - 1 < R - 1:
+            e(f"s_waitcnt vmcnt({window - 1})")
 
-    def layer_reload(p):
+    def layer_reload(p, window=WINDOW):
         """Reload the slot of layer position p (0 <= p < PP) with position p + R."""
-        throttle()
+        throttle(window)
         slot = p % R
         q = p + R
         sset = S_CUR
@@ -221,9 +222,9 @@ def gen(KW, R, NV, NSH):
             deferred += list(range(NREAL, PP))     # padding positions: nothing to compute, only their turn to load
         if SLEEP and deferred:
             e(f"s_sleep {SLEEP}")
-        for p in deferred:
+        for i, p in enumerate(deferred):
             assert issued_loads == p + R
-            layer_reload(p)
+            layer_reload(p, max(BURST, WINDOW) if i < BURST else WINDOW)
             issued_loads += 1
     # end of layer: next layer's addresses become current; fetch the layer after
     e(f"s_add_u32 s{S_JT}, s{S_JT}, 128")

@@ -81,7 +81,7 @@ struct DecodeBuffers {
     u64 *H;                 // [F]       fp32(relu(k)^2 * range_v)
     u64 *HR;                // [3][G]
     unsigned *abort_flag;   // set to 1 by any workgroup whose wait ran out
-    long long *trace;       // optional: [G][L][16] 100 MHz timestamps of every workgroup's phase boundaries (null = off)
+    long long *trace;       // optional: [G][L][24] 100 MHz timestamps of every workgroup's phase boundaries (null = off)
 };
 
 // Host-side description from which the tables are built.
@@ -99,7 +99,7 @@ struct DSetup {
 
 bool decode_supported(int64_t L, int64_t C, int64_t F, int64_t V);
 unsigned decode_epochs_per_token(int64_t L);
-constexpr int kTraceStampsPerLayer = 16;
+constexpr int kTraceStampsPerLayer = 24;
 
 // Bytes of the single device allocation that holds tables, constants and exchange buffers.
 size_t decode_block_bytes(int64_t L, int64_t C, int64_t F, int64_t V);

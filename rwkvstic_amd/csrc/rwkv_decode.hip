@@ -266,19 +266,25 @@ __device__ __forceinline__ void settle_quads(Front &fx, const u64 *src, int firs
     }
 }
 
-// Sum of the 8 back waves' digit sums of column n of parked tile `slot`, digits recombined.
-__device__ __forceinline__ long long tile_total(const v4i *red, int slot, int n) {
+// Sum of the 8 back waves' digit sums of column n of parked tile `slot`, digits recombined:
+// sum_k 256^k sum_c s_k,c w_c.  Every digit sum is below 2^28 in magnitude and the total below 2^52,
+// so each step of the float64 Horner form is exact.
+__device__ __forceinline__ double tile_total(const v4i *red, int slot, int n) {
     int d0 = 0, d1 = 0, d2 = 0, d3 = 0;
 #pragma unroll
-    for (int w = 0; w < kBW; ++w) {
-        const v4i v = red[(slot * kBW + w) * 16 + n];
-        d0 += v.x; d1 += v.y; d2 += v.z; d3 += v.w;
+    for (int h = 0; h < kBW; h += 4) {
+        v4i v[4];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) v[w] = red[(slot * kBW + h + w) * 16 + n];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) { d0 += v[w].x; d1 += v[w].y; d2 += v[w].z; d3 += v[w].w; }
     }
-    return ((((long long)d0 * 256 + d1) * 256 + d2) * 256) + d3;
+    return fma(fma(fma((double)d0, 256.0, (double)d1), 256.0, (double)d2), 256.0, (double)d3);
 }
-// y = S (sum_c q_c (code_c - 128)) + zp,  sum_c q_c w_c = sum_k 256^k sum_c s_k,c w_c + 0x808080 sum_c w_c
+// y = S (sum_c q_c (code_c - 128)) + zp  with  sum_c q_c w_c = total + 0x808080 sum_c w_c.  S is a power
+// of two and the sum an integer below 2^53: one rounding, in the addition of zp.
 __device__ __forceinline__ double finish_col(const v4i *red, int slot, int n, double S, int colsum, double zp) {
-    return S * (double)(tile_total(red, slot, n) + 0x808080LL * (long long)colsum) + zp;
+    return fma(S, tile_total(red, slot, n) + (double)(0x808080LL * (long long)colsum), zp);
 }
 
 // LayerNorm statistics of the 16 channels a DPP row owns, and everything a consumer of x needs that
@@ -300,6 +306,26 @@ __device__ __forceinline__ void publish_ln_input(u64 *X, u64 *XR, int G, int g, 
         if (n == 4 + 3 * m) val = lo;
     }
     if (n < 2 + 3 * NM) put_word(XR + (size_t)n * G + g, epoch, val);
+}
+
+// The same for an epilogue wave whose four DPP rows all hold the same 16 channels (lane n of every
+// row: channel n, value x): row 0 publishes x and reduces sum x, sum x^2, row 1 + m the two
+// quantities of product m (Pm, POm: that product's constants of channel n), so the reductions of
+// all products run side by side.  Values and reduction order are those of publish_ln_input.
+template <int NM>
+__device__ __forceinline__ void publish_ln_input_rows(u64 *X, u64 *XR, int G, int g, int n, int row, unsigned epoch, double x,
+                                                      float Pm, double POm) {
+    static_assert(NM <= 3, "one row per product");
+    if (row == 0) put_word(X + 16 * g + n, epoch, (float)x);
+    const double sa = row16_sum(row == 0 ? x : x * POm);
+    const double sb = row16_sum(x * x);
+    const float mc = row16_max(fabsf((float)(x * (double)Pm)));
+    const float hi = (float)sa, lo = (float)(sa - (double)hi);
+    if (row == 0) {
+        if (n < 2) put_word(XR + (size_t)n * G + g, epoch, n == 0 ? (float)sa : (float)sb);
+    } else if (row <= NM) {
+        if (n < 3) put_word(XR + (size_t)(2 + 3 * (row - 1) + n) * G + g, epoch, n == 0 ? mc : (n == 1 ? hi : lo));
+    }
 }
 
 // ---- owner records --------------------------------------------------------------
@@ -395,13 +421,13 @@ __device__ __forceinline__ double ln_zp(const double *stat, const u64 *rec, int 
 }
 
 // Front side of a LayerNorm-fed product group (NM matrices sharing the normalised input):
-// waits for x and its records, leaves mean, rsd and the per-product sums in stat[0..7], writes NM
-// sets of digit planes.  Contains one workgroup barrier (statistics) and ends with the "digits
+// waits for x and its records, leaves mean, rsd and the per-product sums in stat[0..7] and each
+// product's scale and zero-point sum in stat[8 + 2m], stat[9 + 2m], writes NM sets of digit planes.  Contains one workgroup barrier (statistics) and ends with the "digits
 // ready" barrier.  rec: the LDS owner record of the layer (scalars).
 template <int KW, int FW, int NM>
 __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, const float *P32, const float *Q32,
                                          const u64 *rec, int m0, unsigned epoch, signed char *dig, double *stat,
-                                         long long *tr) {
+                                         long long *tr, long long *tp) {
     constexpr int C = 512 * KW, G = 32 * KW, NG = (G + 63) / 64, FT = 64 * FW, NQ = C / 4, NQT = (NQ + FT - 1) / FT;
     constexpr int PS = C + 64;
     static_assert(FW >= 4, "one front wave per product plus wave 0");
@@ -425,6 +451,7 @@ __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, co
         float r[2][NG];
         poll_rows<2, NG>(fx, a.b.XR, G, 0, epoch, r);
         if (fx.lane == 0) fx.flags[FLAG_ARRIVED] = seq;
+        if (tp && fx.tid == 0) tp[0] = wall_clock64();
         issue_quads<FT, NQT>(a.b.X, fx.tid, 0, NQ, w);
         double s0 = 0.0, s1 = 0.0;
 #pragma unroll
@@ -451,7 +478,7 @@ __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, co
         }
     }
     __syncthreads();                                               // statistics
-    if (tr) tr[0] = wall_clock64();
+    if (tr && fx.tid == 0) tr[0] = wall_clock64();
     if (fx.flags[FLAG_ABORT]) { fx.ok = false; return; }
     const double mean = stat[0], rsd = stat[1];
     float invS[NM];
@@ -459,6 +486,7 @@ __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, co
     for (int m = 0; m < NM; ++m) {
         double S;
         ln_scale(stat, rec, m0, m, S, invS[m]);
+        if (fx.tid == 64 * (1 + m)) { stat[8 + 2 * m] = S; stat[9 + 2 * m] = ln_zp(stat, rec, m0, m); }   // for the epilogue
     }
     settle_quads<FT, NQT>(fx, a.b.X, 0, NQ, epoch, w);
 #pragma unroll
@@ -481,7 +509,7 @@ __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, co
         }
     }
     __syncthreads();                                               // digits ready
-    if (tr) tr[1] = wall_clock64();
+    if (tr && fx.tid == 0) tr[1] = wall_clock64();
     if (fx.flags[FLAG_ABORT]) fx.ok = false;
 }
 
@@ -490,7 +518,7 @@ __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, co
 // the zero-point sum in stat[17].  Ends with the "digits ready" barrier.
 template <int KW, int FW, int NQT>
 __device__ __forceinline__ void vec_front(Front &fx, int &seq, const u64 *src, const u64 *rec, int nq, unsigned epoch,
-                                          signed char *dig, int plane_stride, double *stat, long long *tr) {
+                                          signed char *dig, int plane_stride, double *stat, long long *tr, long long *tp) {
     constexpr int G = 32 * KW, NG = (G + 63) / 64, FT = 64 * FW;
     constexpr int CH = NQT <= 5 ? NQT : ((NQT + 1) / 2 <= 5 ? (NQT + 1) / 2 : 3), NCH = (NQT + CH - 1) / CH;
     fx.refresh();
@@ -501,6 +529,7 @@ __device__ __forceinline__ void vec_front(Front &fx, int &seq, const u64 *src, c
         float r[3][NG];
         poll_rows<3, NG>(fx, rec, G, 0, epoch, r);
         if (fx.lane == 0) fx.flags[FLAG_ARRIVED] = seq;
+        if (tp && fx.tid == 0) tp[0] = wall_clock64();
         issue_quads<FT, CH>(src, fx.tid, 0, nq, w[0]);
         float mx = 0.f;
         double so = 0.0;
@@ -517,7 +546,7 @@ __device__ __forceinline__ void vec_front(Front &fx, int &seq, const u64 *src, c
         wait_flag(fx, FLAG_SCALE, seq);
         invS = (float)stat[18];
     }
-    if (tr) tr[0] = wall_clock64();
+    if (tr && fx.tid == 0) tr[0] = wall_clock64();
 #pragma unroll
     for (int ch = 0; ch < NCH; ++ch) {
         if (ch + 1 < NCH) issue_quads<FT, CH>(src, fx.tid, (ch + 1) * CH, nq, w[(ch + 1) & 1]);
@@ -534,14 +563,14 @@ __device__ __forceinline__ void vec_front(Front &fx, int &seq, const u64 *src, c
         }
     }
     __syncthreads();                                               // digits ready
-    if (tr) tr[1] = wall_clock64();
+    if (tr && fx.tid == 0) tr[1] = wall_clock64();
     if (fx.flags[FLAG_ABORT]) fx.ok = false;
 }
 
 // =============================================================================
 template <int KW, int FW, bool TRACE>
 __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, const v4i *red, double *stat, double *rf_lds,
-                                           lds_flag_t *flags, u64 *own_lds, double *st_lds) {
+                                           lds_flag_t *flags, u64 *own_lds, double *st_lds, long long *trace_lds) {
     constexpr int C = 512 * KW, F = 4 * C, G = 32 * KW, FT = 64 * FW;
     constexpr int PS = C + 64, PSF = F + 64;
     constexpr int NQH = F / 4, NQTH = (NQH + FT - 1) / FT, NQC = C / 4, NQTC = (NQC + FT - 1) / FT;
@@ -550,7 +579,8 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
     fx.refresh();
     const int g = blockIdx.x, L = a.m.L, V = a.m.V;
     const bool fin = fx.wave == 0;                       // wave 0 owns the workgroup's 16 channels
-    long long *trace = (TRACE && threadIdx.x == 0) ? a.b.trace + (size_t)g * L * kTraceStampsPerLayer : nullptr;
+    // stamps are collected in LDS and copied out after the head: a store to memory here would queue behind the weight stream
+    long long *trace = TRACE ? trace_lds : nullptr;     // uniform; thread 0 stamps
     int seq = 0;
     int lane, n, row, c_own;                             // recomputed at the start of every phase
 #define RWKV_IDS() do { fx.refresh(); lane = fx.lane; n = lane & 15; row = lane >> 4; c_own = 16 * g + n; } while (0)
@@ -570,23 +600,22 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
         const unsigned e = a.epoch0 + 4u * (unsigned)l;
         long long *tr = trace ? trace + (size_t)l * kTraceStampsPerLayer : nullptr;
         const float *P32 = a.m.P32 + (size_t)l * kLnMats * C, *Q32 = a.m.Q32 + (size_t)l * kLnMats * C;
-        if (tr) tr[0] = wall_clock64();
+        if (tr && fx.tid == 0) { tr[0] = wall_clock64(); tr[23] = clock64(); }     // [23]: shader clock, for its ratio to the wall clock
 
         // ===================== phase 1: att k, v, r ============================
-        ln_front<KW, FW, 3>(fx, seq, a, P32, Q32, rec, 0, e, dig, stat, tr ? tr + 1 : nullptr);
+        ln_front<KW, FW, 3>(fx, seq, a, P32, Q32, rec, 0, e, dig, stat, tr ? tr + 1 : nullptr, tr ? tr + 16 : nullptr);
         if (!fx.ok) break;
-        __syncthreads();                                                         // tile sums parked
-        if (tr) tr[3] = wall_clock64();
         RWKV_IDS();
-        double xy1 = 0.0;
+        // while the matrix cores run: the LayerNorm output of the own channel is the new att shift state (block.py:58,63-64)
+        if (fin && row == 0) sl[n] = or_d(rec, OR_LN1W * 16 + n) * ((x_lds[n] - stat[0]) * stat[1]) + or_d(rec, OR_LN1B * 16 + n);
+        __syncthreads();                                                         // tile sums parked
+        if (tr && fx.tid == 0) tr[3] = wall_clock64();
         if (fin) {
-            const int j = row < 3 ? row : 0;
+            const int j = row < 3 ? row : 0;             // rows 0..2: columns of k, v, r
             const int cs1 = (int)(j == 0 ? or_lo(rec, OR_CSK_CSV * 16 + n) : (j == 1 ? or_hi(rec, OR_CSK_CSV * 16 + n) : or_lo(rec, OR_CSR_CSFR * 16 + n)));
-            double Sj;
-            float invSj;
-            ln_scale(stat, rec, 0, j, Sj, invSj);
-            const double y = finish_col(red, j, n, Sj, cs1, ln_zp(stat, rec, 0, j));
+            const double y = finish_col(red, j, n, stat[8 + 2 * j], cs1, stat[9 + 2 * j]);
             const double yv = lane_read_f64(y, n + 16), yr = lane_read_f64(y, n + 32);
+            if (tr && fx.tid == 0) tr[20] = wall_clock64();
             if (row == 0) {
                 const double td = or_d(rec, OR_DECAY * 16 + n), tf = or_d(rec, OR_FIRST * 16 + n);
                 const float r = sigmoid_f32((float)yr);                          // block.py:72
@@ -603,41 +632,41 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
                 sl[2 * 16 + n] = (double)aa;
                 sl[3 * 16 + n] = (double)bb;
                 sl[4 * 16 + n] = pp;
-                xy1 = or_d(rec, OR_LN1W * 16 + n) * ((x_lds[n] - stat[0]) * stat[1]) + or_d(rec, OR_LN1B * 16 + n);   // block.py:58
-                sl[n] = xy1;                                                     // block.py:63-64
             }
         }
-        if (tr) tr[4] = wall_clock64();
+        if (tr && fx.tid == 0) tr[4] = wall_clock64();
 
         // ===================== phase 2: att output =============================
-        vec_front<KW, FW, NQTC>(fx, seq, a.b.A, a.b.AR, NQC, e + 1u, dig, PS, stat, tr ? tr + 5 : nullptr);
+        vec_front<KW, FW, NQTC>(fx, seq, a.b.A, a.b.AR, NQC, e + 1u, dig, PS, stat, tr ? tr + 5 : nullptr, tr ? tr + 17 : nullptr);
         if (!fx.ok) break;
         __syncthreads();
-        if (tr) tr[7] = wall_clock64();
+        if (tr && fx.tid == 0) tr[7] = wall_clock64();
         RWKV_IDS();
-        if (fin && row == 0) {
+        if (fin) {                                         // all four rows: the same 16 channels; row 1 + m reduces for product m
             const double x_own = x_lds[n] + finish_col(red, 0, n, stat[16], (int)or_hi(rec, OR_RNGO_CSO * 16 + n), stat[17]);   // block.py:80
-            x_lds[n] = x_own;
-            const float Pf[2] = {__uint_as_float(or_lo(rec, OR_PF * 16 + n)), __uint_as_float(or_hi(rec, OR_PF * 16 + n))};
-            const double POf[2] = {or_d(rec, OR_POFK * 16 + n), or_d(rec, OR_POFR * 16 + n)};
-            publish_ln_input<2>(a.b.X, a.b.XR, G, g, n, e + 2u, x_own, Pf, POf);
+            const int m = row == 2 ? 1 : 0;                // [0] ffn_k, [1] ffn_r
+            const u64 pf = rec[OR_PF * 16 + n];
+            const float Pm = __uint_as_float(m ? (unsigned)(pf >> 32) : (unsigned)pf);
+            const double POm = or_d(rec, (OR_POFK + m) * 16 + n);
+            if (tr && fx.tid == 0) tr[21] = wall_clock64();
+            publish_ln_input_rows<2>(a.b.X, a.b.XR, G, g, n, row, e + 2u, x_own, Pm, POm);
+            if (row == 0) x_lds[n] = x_own;                // after every row has read the old value
         }
-        if (tr) tr[8] = wall_clock64();
+        if (tr && fx.tid == 0) tr[8] = wall_clock64();
 
         // ===================== phase 3: ffn receptance + key ===================
-        ln_front<KW, FW, 2>(fx, seq, a, P32, Q32, rec, 3, e + 2u, dig, stat, tr ? tr + 9 : nullptr);   // [0] ffn_k, [1] ffn_r
+        ln_front<KW, FW, 2>(fx, seq, a, P32, Q32, rec, 3, e + 2u, dig, stat, tr ? tr + 9 : nullptr, tr ? tr + 18 : nullptr);   // [0] ffn_k, [1] ffn_r
         if (!fx.ok) break;
         RWKV_IDS();
+        // the LayerNorm output of the own channel is the new ffn shift state (block.py:82,87-88)
+        if (fin && row == 0) sl[16 + n] = or_d(rec, OR_LN2W * 16 + n) * ((x_lds[n] - stat[0]) * stat[1]) + or_d(rec, OR_LN2B * 16 + n);
         stage_owner_record<FT, KW>(a, l + 1, g, G, C, own_lds, fx.tid);   // while the matrix cores run (l + 1 == L: the head's scalars)
         __syncthreads();
-        if (tr) tr[11] = wall_clock64();
+        if (tr && fx.tid == 0) tr[11] = wall_clock64();
         if (fin) {
             // parked tiles: 0 = ffn_r, 1..4 = ffn_k tiles g, g+G, g+2G, g+3G
             const int f_own = 16 * (g + G * row) + n;      // column of ffn_k tile `row`
-            double Sk;
-            float invSk;
-            ln_scale(stat, rec, 3, 0, Sk, invSk);
-            const double y = finish_col(red, 1 + row, n, Sk, (int)or_hi(rec, kOrRngVCs + lane), ln_zp(stat, rec, 3, 0));
+            const double y = finish_col(red, 1 + row, n, stat[8], (int)or_hi(rec, kOrRngVCs + lane), stat[9]);
             const double h = y > 0.0 ? y : 0.0;                                  // block.py:97-98
             const double hh = h * h;
             const float xs = (float)(hh * (double)__uint_as_float(or_lo(rec, kOrRngVCs + lane)));
@@ -646,38 +675,30 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
             const double so = wave_sum_dpp(hh * or_d(rec, kOrOffV + lane) + 128.0 * (double)xs);
             const float hi = (float)so, lo = (float)(so - (double)hi);
             if (lane < 3) put_word(a.b.HR + (size_t)lane * G + g, e + 3u, lane == 0 ? mx : (lane == 1 ? hi : lo));
-            if (row == 0) {                                // after H is out: the receptance gate of the own channels
-                double Sr;
-                float invSr;
-                ln_scale(stat, rec, 3, 1, Sr, invSr);
-                const double yr = finish_col(red, 0, n, Sr, (int)or_hi(rec, OR_CSR_CSFR * 16 + n), ln_zp(stat, rec, 3, 1));
-                rf_lds[n] = (double)sigmoid_f32((float)yr);                      // block.py:95
-                // the LayerNorm output of the own channel is the new ffn shift state (block.py:82,87-88)
-                sl[16 + n] = or_d(rec, OR_LN2W * 16 + n) * ((x_lds[n] - stat[0]) * stat[1]) + or_d(rec, OR_LN2B * 16 + n);
+            if (row == 0) {                                // after H is out: the receptance gate of the own channels (block.py:95)
+                const double yr = finish_col(red, 0, n, stat[10], (int)or_hi(rec, OR_CSR_CSFR * 16 + n), stat[11]);
+                rf_lds[n] = (double)sigmoid_f32((float)yr);
             }
         }
-        if (tr) tr[12] = wall_clock64();
+        if (tr && fx.tid == 0) tr[12] = wall_clock64();
 
         // ===================== phase 4: ffn value ==============================
-        vec_front<KW, FW, NQTH>(fx, seq, a.b.H, a.b.HR, NQH, e + 3u, dig, PSF, stat, tr ? tr + 13 : nullptr);
+        vec_front<KW, FW, NQTH>(fx, seq, a.b.H, a.b.HR, NQH, e + 3u, dig, PSF, stat, tr ? tr + 13 : nullptr, tr ? tr + 19 : nullptr);
         if (!fx.ok) break;
         __syncthreads();
-        if (tr) tr[15] = wall_clock64();
+        if (tr && fx.tid == 0) tr[15] = wall_clock64();
         RWKV_IDS();
-        if (fin && row == 0) {
+        if (fin) {                                         // all four rows: the same 16 channels; row 1 + m reduces for product m
             const double y = finish_col(red, 0, n, stat[16], (int)or_lo(rec, OR_CSFV * 16 + n), stat[17]);
             const double x_own = y * rf_lds[n] + x_lds[n];                       // block.py:100
-            x_lds[n] = x_own;
-            const float Pn[3] = {__uint_as_float(or_lo(rec, OR_PN01 * 16 + n)), __uint_as_float(or_hi(rec, OR_PN01 * 16 + n)),
-                                 __uint_as_float(or_lo(rec, OR_PN2 * 16 + n))};
-            const double POn[3] = {or_d(rec, OR_PON0 * 16 + n), or_d(rec, OR_PON1 * 16 + n), or_d(rec, OR_PON2 * 16 + n)};
-            if (l + 1 == L) {                              // the next consumer of x is the head (one product)
-                const float P1[1] = {Pn[0]};
-                const double PO1[1] = {POn[0]};
-                publish_ln_input<1>(a.b.X, a.b.XR, G, g, n, e + 4u, x_own, P1, PO1);
-            } else {
-                publish_ln_input<3>(a.b.X, a.b.XR, G, g, n, e + 4u, x_own, Pn, POn);
-            }
+            const int m = row >= 1 ? row - 1 : 0;          // next layer's att k, v, r (or the head: one product)
+            const u64 pn = rec[(OR_PN01 + (m >> 1)) * 16 + n];
+            const float Pm = __uint_as_float((m & 1) ? (unsigned)(pn >> 32) : (unsigned)pn);
+            const double POm = or_d(rec, (OR_PON0 + m) * 16 + n);
+            if (tr && fx.tid == 0) tr[22] = wall_clock64();
+            if (l + 1 == L) publish_ln_input_rows<1>(a.b.X, a.b.XR, G, g, n, row, e + 4u, x_own, Pm, POm);
+            else publish_ln_input_rows<3>(a.b.X, a.b.XR, G, g, n, row, e + 4u, x_own, Pm, POm);
+            if (row == 0) x_lds[n] = x_own;                // after every row has read the old value
         }
     }
 
@@ -686,7 +707,7 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
     const u64 *rec_h = own_lds + (L & 1) * kOrSlots;
     if (fx.ok)
         ln_front<KW, FW, 1>(fx, seq, a, a.m.P32 + (size_t)L * kLnMats * C, a.m.Q32 + (size_t)L * kLnMats * C, rec_h, 0,
-                            a.epoch0 + 4u * (unsigned)L, dig, stat, nullptr);
+                            a.epoch0 + 4u * (unsigned)L, dig, stat, nullptr, nullptr);
     if (!fx.ok) return;     // every wave leaves after the same barrier: the flag is tested after each one that follows a wait
     RWKV_IDS();
 #undef RWKV_IDS
@@ -706,6 +727,8 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
     }
     // the state rows of the own channels: st_lds[l][row][n] -> state[l][row][16 g + n]
     for (int i = fx.tid; i < L * 5 * 16; i += FT) a.state[(size_t)(i >> 4) * C + 16 * g + (i & 15)] = st_lds[i];
+    if (TRACE)
+        for (int i = fx.tid; i < L * kTraceStampsPerLayer; i += FT) a.b.trace[(size_t)g * L * kTraceStampsPerLayer + i] = trace_lds[i];
 }
 
 template <int KW, int FW>
@@ -718,7 +741,9 @@ struct DecodeLds {
     static constexpr int STAT_BYTES = 32 * 8, RF_BYTES = 32 * 8, FLAG_BYTES = FLAG_COUNT * 4;   // RF: gate and residual of the own channels
     static constexpr int OWN_OFFSET = DIG_BYTES + RED_BYTES + STAT_BYTES + RF_BYTES + FLAG_BYTES;
     static constexpr int STATE_OFFSET = OWN_OFFSET + 2 * kOrSlots * 8;
-    static int total(int L) { return STATE_OFFSET + L * 5 * 16 * 8; }       // + the new state rows of the own channels
+    static __host__ __device__ int total(int L, bool trace = false) {                           // + the new state rows of the own channels (+ the stamps)
+        return STATE_OFFSET + L * 5 * 16 * 8 + (trace ? L * kTraceStampsPerLayer * 8 : 0);
+    }
     // the generated back-wave program addresses LDS by these offsets
     static_assert(BackCfg<KW, FW>::RED == DIG_BYTES, "parked tiles follow the digit planes");
     static_assert(BackCfg<KW, FW>::FLAG == DIG_BYTES + RED_BYTES + STAT_BYTES + RF_BYTES + FLAG_ABORT * 4, "abort flag offset");
@@ -739,7 +764,8 @@ __global__ void __launch_bounds__((FW + kBW) * 64) decode_kernel(const DArgs a) 
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     if (wave < FW) {
         front_path<KW, FW, TRACE>(a, dig, red, stat, rf_lds, flags, reinterpret_cast<u64 *>(smem + Lds::OWN_OFFSET),
-                                  reinterpret_cast<double *>(smem + Lds::STATE_OFFSET));
+                                  reinterpret_cast<double *>(smem + Lds::STATE_OFFSET),
+                                  reinterpret_cast<long long *>(smem + Lds::total(a.m.L)));
     } else {
         constexpr int G = 32 * KW;
         const int v_tiles = (a.m.V + 15) / 16, head_rounds = (v_tiles + G - 1) / G;
@@ -1203,10 +1229,11 @@ int decode_setup(void *block, const DSetup &s, DModel *dm, DecodeBuffers *db) {
 
 template <int KW, int FW>
 static int launch_one(hipStream_t st, const DArgs &args, bool with_prep) {
-    const int lds = DecodeLds<KW, FW>::total(args.m.L);
+    const bool trace = args.b.trace != nullptr;
+    const int lds = DecodeLds<KW, FW>::total(args.m.L, trace);
     if (lds > 160 * 1024) return set_error(RWKV_ERR_SIZE, "decode kernel: %d layers need %d bytes of LDS", args.m.L, lds);
     static int configured = 0;
-    if (configured < lds) {
+    if (configured < lds) {     // the attribute only ever grows
         RWKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_kernel<KW, FW, false>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         RWKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_kernel<KW, FW, true>),
@@ -1215,7 +1242,7 @@ static int launch_one(hipStream_t st, const DArgs &args, bool with_prep) {
     }
     if (with_prep)
         hipLaunchKernelGGL(prep_kernel, dim3((unsigned)(args.m.L * (args.m.C / kPrepThreads) + 1)), dim3(kPrepThreads), 0, st, args);
-    if (args.b.trace)
+    if (trace)
         hipLaunchKernelGGL((decode_kernel<KW, FW, true>), dim3((unsigned)args.m.G), dim3((FW + kBW) * 64), lds, st, args);
     else
         hipLaunchKernelGGL((decode_kernel<KW, FW, false>), dim3((unsigned)args.m.G), dim3((FW + kBW) * 64), lds, st, args);
