@@ -197,34 +197,69 @@ struct Front {
     }
 };
 
-// A whole wave fetches NR consecutive rows of a [rows][G] record table (lane i takes workgroups
-// i, i + 64, ...), spinning until every word carries `epoch`.  Wave-uniform control flow.
-template <int NR, int NG>
-__device__ __forceinline__ void poll_rows(Front &fx, const u64 *table, int G, int row0, unsigned epoch, float (&out)[NR][NG]) {
-    u64 w[NR][NG];
-    unsigned spins = 0;
-    while (fx.ok) {
-        bool all = true;
-#pragma unroll
-        for (int r = 0; r < NR; ++r)
-#pragma unroll
-            for (int i = 0; i < NG; ++i)
-                if (fx.lane + 64 * i < G) w[r][i] = ALOAD(table + (size_t)(row0 + r) * G + fx.lane + 64 * i);
-#pragma unroll
-        for (int r = 0; r < NR; ++r)
-#pragma unroll
-            for (int i = 0; i < NG; ++i)
-                if (fx.lane + 64 * i < G) all = all && ((unsigned)(w[r][i] >> 32) == epoch);
-        if (__ballot(!all) == 0ull) break;
-        __builtin_amdgcn_s_sleep(2);
-        if ((++spins & 63u) == 0u && (spins > kSpinLimit || ALOAD32(fx.abort_flag) != 0u || fx.flags[FLAG_ABORT])) fx.fail();
-    }
-#pragma unroll
-    for (int r = 0; r < NR; ++r)
-#pragma unroll
-        for (int i = 0; i < NG; ++i)
-            out[r][i] = (fx.lane + 64 * i < G) ? __uint_as_float((unsigned)w[r][i]) : 0.f;
+// Gathers read 16 bytes per lane through a raw buffer descriptor with the agent-coherent cache
+// policy: half as many memory instructions as 8-byte atomic loads of the same words.  A 16-byte
+// aligned read returns each of its two 8-byte words as some store left it (words are only ever
+// written whole).
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+typedef __amdgpu_buffer_rsrc_t xtab_t;
+__device__ __forceinline__ xtab_t make_xtab(const u64 *p, int words) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<u64 *>(p), 0, words * 8, 0x00020000);
 }
+constexpr int kAuxAgent = 16;      // cache policy bit sc1: coherent at agent scope
+
+// A whole wave fetches NR consecutive rows of a [rows][G] record table as one range of NR * G words,
+// 16 bytes (two words) per lane and read, spinning until every word carries `epoch`.  Lane l holds
+// words 2 (l + 64 k) + j (k < K, j < 2) of the range; word i belongs to row i / G.  Wave-uniform
+// control flow.
+template <int NR, int G>
+struct RowPoll {
+    static constexpr int PAIRS = NR * G / 2, K = (PAIRS + 63) / 64;
+    static_assert(G % 2 == 0, "two words per lane");
+    float v[K][2];
+    __device__ __forceinline__ void poll(Front &fx, const u64 *rows, unsigned epoch) {
+        const xtab_t t = make_xtab(rows, NR * G);
+        v4u w[K];
+        unsigned spins = 0;
+        while (fx.ok) {
+            bool all = true;
+#pragma unroll
+            for (int k = 0; k < K; ++k)
+                if (fx.lane + 64 * k < PAIRS) w[k] = __builtin_amdgcn_raw_buffer_load_b128(t, (fx.lane + 64 * k) * 16, 0, kAuxAgent);
+#pragma unroll
+            for (int k = 0; k < K; ++k)
+                if (fx.lane + 64 * k < PAIRS) all = all && w[k].y == epoch && w[k].w == epoch;
+            if (__ballot(!all) == 0ull) break;
+            __builtin_amdgcn_s_sleep(2);
+            if ((++spins & 63u) == 0u && (spins > kSpinLimit || ALOAD32(fx.abort_flag) != 0u || fx.flags[FLAG_ABORT])) fx.fail();
+        }
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const bool in = fx.lane + 64 * k < PAIRS;
+            v[k][0] = in ? __uint_as_float(w[k].x) : 0.f;
+            v[k][1] = in ? __uint_as_float(w[k].z) : 0.f;
+        }
+    }
+    // this lane's share of row r: sum (float64) and maximum of its words (0 where it holds none)
+    __device__ __forceinline__ double lane_sum(const Front &fx, int r) const {
+        double acc = 0.0;
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                if ((2 * (fx.lane + 64 * k) + j) / G == r) acc += (double)v[k][j];
+        return acc;
+    }
+    __device__ __forceinline__ float lane_max(const Front &fx, int r) const {
+        float acc = 0.f;
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                if ((2 * (fx.lane + 64 * k) + j) / G == r) acc = fmaxf(acc, v[k][j]);
+        return acc;
+    }
+};
 
 // Spin on an LDS sequence word written by wave 0.
 __device__ __forceinline__ void wait_flag(Front &fx, int which, int seq) {
@@ -237,19 +272,21 @@ __device__ __forceinline__ void wait_flag(Front &fx, int which, int seq) {
 
 // Thread ft of FT front threads owns quads (groups of 4 consecutive words) ft, ft + FT, ...
 template <int FT, int N>
-__device__ __forceinline__ void issue_quads(const u64 *src, int ft, int first, int nq, u64 (&w)[N][4]) {
+__device__ __forceinline__ void issue_quads(xtab_t src, int ft, int first, int nq, u64 (&w)[N][4]) {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
         const int qi = ft + FT * (first + i);
         if (qi < nq) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) w[i][e] = ALOAD(src + 4 * (size_t)qi + e);
+            const v4u lo = __builtin_amdgcn_raw_buffer_load_b128(src, qi * 32, 0, kAuxAgent);
+            const v4u hi = __builtin_amdgcn_raw_buffer_load_b128(src, qi * 32 + 16, 0, kAuxAgent);
+            w[i][0] = ((u64)lo.y << 32) | lo.x; w[i][1] = ((u64)lo.w << 32) | lo.z;
+            w[i][2] = ((u64)hi.y << 32) | hi.x; w[i][3] = ((u64)hi.w << 32) | hi.z;
         }
     }
 }
 // Re-reads until every word of the thread's quads carries the epoch (normally the first read does).
 template <int FT, int N>
-__device__ __forceinline__ void settle_quads(Front &fx, const u64 *src, int first, int nq, unsigned epoch, u64 (&w)[N][4]) {
+__device__ __forceinline__ void settle_quads(Front &fx, xtab_t src, int first, int nq, unsigned epoch, u64 (&w)[N][4]) {
     unsigned spins = 0;
     while (fx.ok) {
         bool all = true;
@@ -428,7 +465,7 @@ template <int KW, int FW, int NM>
 __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, const float *P32, const float *Q32,
                                          const u64 *rec, int m0, unsigned epoch, signed char *dig, double *stat,
                                          long long *tr, long long *tp) {
-    constexpr int C = 512 * KW, G = 32 * KW, NG = (G + 63) / 64, FT = 64 * FW, NQ = C / 4, NQT = (NQ + FT - 1) / FT;
+    constexpr int C = 512 * KW, G = 32 * KW, FT = 64 * FW, NQ = C / 4, NQT = (NQ + FT - 1) / FT;
     constexpr int PS = C + 64;
     static_assert(FW >= 4, "one front wave per product plus wave 0");
     fx.refresh();
@@ -447,16 +484,14 @@ __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, co
     }
     ++seq;
     u64 w[NQT][4];
+    const xtab_t xt = make_xtab(a.b.X, C);
     if (fx.wave == 0) {
-        float r[2][NG];
-        poll_rows<2, NG>(fx, a.b.XR, G, 0, epoch, r);
+        RowPoll<2, G> r;
+        r.poll(fx, a.b.XR, epoch);
         if (fx.lane == 0) fx.flags[FLAG_ARRIVED] = seq;
         if (tp && fx.tid == 0) tp[0] = wall_clock64();
-        issue_quads<FT, NQT>(a.b.X, fx.tid, 0, NQ, w);
-        double s0 = 0.0, s1 = 0.0;
-#pragma unroll
-        for (int i = 0; i < NG; ++i) { s0 += (double)r[0][i]; s1 += (double)r[1][i]; }
-        s0 = wave_sum_dpp(s0); s1 = wave_sum_dpp(s1);
+        issue_quads<FT, NQT>(xt, fx.tid, 0, NQ, w);
+        const double s0 = wave_sum_dpp(r.lane_sum(fx, 0)), s1 = wave_sum_dpp(r.lane_sum(fx, 1));
         const double mean = s0 * (1.0 / (double)C);
         double var = s1 * (1.0 / (double)C) - mean * mean;
         if (var < 0.0) var = 0.0;
@@ -464,16 +499,13 @@ __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, co
         if (fx.lane == 0) { stat[0] = mean; stat[1] = rsd; }
     } else {
         wait_flag(fx, FLAG_ARRIVED, seq);
-        issue_quads<FT, NQT>(a.b.X, fx.tid, 0, NQ, w);
+        issue_quads<FT, NQT>(xt, fx.tid, 0, NQ, w);
         const int m = fx.wave - 1;
         if (m < NM) {
-            float r[3][NG];
-            poll_rows<3, NG>(fx, a.b.XR, G, 2 + 3 * m, epoch, r);
-            float mx = 0.f;
-            double so = 0.0;
-#pragma unroll
-            for (int i = 0; i < NG; ++i) { mx = fmaxf(mx, r[0][i]); so += (double)r[1][i] + (double)r[2][i]; }
-            mx = wave_max_dpp(mx); so = wave_sum_dpp(so);
+            RowPoll<3, G> r;
+            r.poll(fx, a.b.XR + (size_t)(2 + 3 * m) * G, epoch);
+            const float mx = wave_max_dpp(r.lane_max(fx, 0));
+            const double so = wave_sum_dpp(r.lane_sum(fx, 1) + r.lane_sum(fx, 2));
             if (fx.lane == 0) { stat[2 + 2 * m] = (double)mx; stat[3 + 2 * m] = so; }
         }
     }
@@ -488,7 +520,7 @@ __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, co
         ln_scale(stat, rec, m0, m, S, invS[m]);
         if (fx.tid == 64 * (1 + m)) { stat[8 + 2 * m] = S; stat[9 + 2 * m] = ln_zp(stat, rec, m0, m); }   // for the epilogue
     }
-    settle_quads<FT, NQT>(fx, a.b.X, 0, NQ, epoch, w);
+    settle_quads<FT, NQT>(fx, xt, 0, NQ, epoch, w);
 #pragma unroll
     for (int i = 0; i < NQT; ++i) {
         const int qi = fx.tid + FT * i;
@@ -519,38 +551,35 @@ __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, co
 template <int KW, int FW, int NQT>
 __device__ __forceinline__ void vec_front(Front &fx, int &seq, const u64 *src, const u64 *rec, int nq, unsigned epoch,
                                           signed char *dig, int plane_stride, double *stat, long long *tr, long long *tp) {
-    constexpr int G = 32 * KW, NG = (G + 63) / 64, FT = 64 * FW;
+    constexpr int G = 32 * KW, FT = 64 * FW;
     constexpr int CH = NQT <= 5 ? NQT : ((NQT + 1) / 2 <= 5 ? (NQT + 1) / 2 : 3), NCH = (NQT + CH - 1) / CH;
     fx.refresh();
     ++seq;
+    const xtab_t st = make_xtab(src, 4 * nq);
     u64 w[NCH > 1 ? 2 : 1][CH][4];
     float invS;
     if (fx.wave == 0) {
-        float r[3][NG];
-        poll_rows<3, NG>(fx, rec, G, 0, epoch, r);
+        RowPoll<3, G> r;
+        r.poll(fx, rec, epoch);
         if (fx.lane == 0) fx.flags[FLAG_ARRIVED] = seq;
         if (tp && fx.tid == 0) tp[0] = wall_clock64();
-        issue_quads<FT, CH>(src, fx.tid, 0, nq, w[0]);
-        float mx = 0.f;
-        double so = 0.0;
-#pragma unroll
-        for (int i = 0; i < NG; ++i) { mx = fmaxf(mx, r[0][i]); so += (double)r[1][i] + (double)r[2][i]; }
-        mx = wave_max_dpp(mx);
-        so = wave_sum_dpp(so);
+        issue_quads<FT, CH>(st, fx.tid, 0, nq, w[0]);
+        const float mx = wave_max_dpp(r.lane_max(fx, 0));
+        const double so = wave_sum_dpp(r.lane_sum(fx, 1) + r.lane_sum(fx, 2));
         double S;
         scale_from_amax(mx, S, invS);
         if (fx.lane == 0) { stat[16] = S; stat[17] = so; stat[18] = (double)invS; fx.flags[FLAG_SCALE] = seq; }
     } else {
         wait_flag(fx, FLAG_ARRIVED, seq);
-        issue_quads<FT, CH>(src, fx.tid, 0, nq, w[0]);
+        issue_quads<FT, CH>(st, fx.tid, 0, nq, w[0]);
         wait_flag(fx, FLAG_SCALE, seq);
         invS = (float)stat[18];
     }
     if (tr && fx.tid == 0) tr[0] = wall_clock64();
 #pragma unroll
     for (int ch = 0; ch < NCH; ++ch) {
-        if (ch + 1 < NCH) issue_quads<FT, CH>(src, fx.tid, (ch + 1) * CH, nq, w[(ch + 1) & 1]);
-        settle_quads<FT, CH>(fx, src, ch * CH, nq, epoch, w[ch & 1]);
+        if (ch + 1 < NCH) issue_quads<FT, CH>(st, fx.tid, (ch + 1) * CH, nq, w[(ch + 1) & 1]);
+        settle_quads<FT, CH>(fx, st, ch * CH, nq, epoch, w[ch & 1]);
 #pragma unroll
         for (int i = 0; i < CH; ++i) {
             const int qi = fx.tid + FT * (ch * CH + i);
