@@ -346,23 +346,34 @@ __device__ __forceinline__ void publish_ln_input(u64 *X, u64 *XR, int G, int g, 
 }
 
 // The same for an epilogue wave whose four DPP rows all hold the same 16 channels (lane n of every
-// row: channel n, value x): row 0 publishes x and reduces sum x, sum x^2, row 1 + m the two
-// quantities of product m (Pm, POm: that product's constants of channel n), so the reductions of
-// all products run side by side.  Values and reduction order are those of publish_ln_input.
+// row: channel n, value x): row 0 publishes x, row 1 + m reduces and publishes the two quantities of
+// product m (Pm, POm: that product's constants of channel n) and row 1 also sum x and sum x^2, so the
+// reductions of all products run side by side and everything leaves in ONE store instruction (a
+// store has to queue behind the weight loads the back waves have just issued).  Values and
+// reduction order are those of publish_ln_input.
 template <int NM>
 __device__ __forceinline__ void publish_ln_input_rows(u64 *X, u64 *XR, int G, int g, int n, int row, unsigned epoch, double x,
                                                       float Pm, double POm) {
-    static_assert(NM <= 3, "one row per product");
-    if (row == 0) put_word(X + 16 * g + n, epoch, (float)x);
-    const double sa = row16_sum(row == 0 ? x : x * POm);
-    const double sb = row16_sum(x * x);
+    static_assert(NM >= 1 && NM <= 3, "one row per product");
+    const double sx = row16_sum(x);
+    const double sxx = row16_sum(x * x);
+    const double so = row16_sum(x * POm);
     const float mc = row16_max(fabsf((float)(x * (double)Pm)));
-    const float hi = (float)sa, lo = (float)(sa - (double)hi);
-    if (row == 0) {
-        if (n < 2) put_word(XR + (size_t)n * G + g, epoch, n == 0 ? (float)sa : (float)sb);
-    } else if (row <= NM) {
-        if (n < 3) put_word(XR + (size_t)(2 + 3 * (row - 1) + n) * G + g, epoch, n == 0 ? mc : (n == 1 ? hi : lo));
+    const float hi = (float)so, lo = (float)(so - (double)hi);
+    u64 *dst = X + 16 * g + n;
+    float val = (float)x;
+    bool on = row == 0;
+    if (row >= 1 && row <= NM && n < 3) {
+        dst = XR + (size_t)(2 + 3 * (row - 1) + n) * G + g;
+        val = n == 0 ? mc : (n == 1 ? hi : lo);
+        on = true;
     }
+    if (row == 1 && (n == 3 || n == 4)) {
+        dst = XR + (size_t)(n - 3) * G + g;
+        val = n == 3 ? (float)sx : (float)sxx;
+        on = true;
+    }
+    if (on) put_word(dst, epoch, val);
 }
 
 // ---- owner records --------------------------------------------------------------
@@ -643,29 +654,37 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
             const int j = row < 3 ? row : 0;             // rows 0..2: columns of k, v, r
             const int cs1 = (int)(j == 0 ? or_lo(rec, OR_CSK_CSV * 16 + n) : (j == 1 ? or_hi(rec, OR_CSK_CSV * 16 + n) : or_lo(rec, OR_CSR_CSFR * 16 + n)));
             const double y = finish_col(red, j, n, stat[8 + 2 * j], cs1, stat[9 + 2 * j]);
-            const double yv = lane_read_f64(y, n + 16), yr = lane_read_f64(y, n + 32);
+            const double yk = lane_read_f64(y, n), yv = lane_read_f64(y, n + 16), yr = lane_read_f64(y, n + 32);
             if (tr && fx.tid == 0) tr[20] = wall_clock64();
-            if (row == 0) {
+            {                                              // all four rows: the same 16 channels; one store instruction
                 const double td = or_d(rec, OR_DECAY * 16 + n), tf = or_d(rec, OR_FIRST * 16 + n);
                 const float r = sigmoid_f32((float)yr);                          // block.py:72
                 float aa = (float)or_d(rec, kOrState + n), bb = (float)or_d(rec, kOrState + 16 + n);
                 double pp = or_d(rec, kOrState + 32 + n);
-                const float wkv = wkv_step_f32(td, tf, (float)y, (float)yv, aa, bb, pp);
+                const float wkv = wkv_step_f32(td, tf, (float)yk, (float)yv, aa, bb, pp);
                 const double av = (double)(wkv * r);                             // block.py:78
                 const float xs = (float)(av * (double)__uint_as_float(or_lo(rec, OR_RNGO_CSO * 16 + n)));   // matmul.py:131
-                put_word(a.b.A + c_own, e + 1u, xs);
                 const float mx = row16_max(fabsf(xs));
                 const double so = row16_sum(av * or_d(rec, OR_OFFO * 16 + n) + 128.0 * (double)xs);
                 const float hi = (float)so, lo = (float)(so - (double)hi);
-                if (n < 3) put_word(a.b.AR + (size_t)n * G + g, e + 1u, n == 0 ? mx : (n == 1 ? hi : lo));
-                sl[2 * 16 + n] = (double)aa;
-                sl[3 * 16 + n] = (double)bb;
-                sl[4 * 16 + n] = pp;
+                u64 *dst = a.b.A + c_own;
+                float val = xs;
+                if (row == 1) { dst = a.b.AR + (size_t)n * G + g; val = n == 0 ? mx : (n == 1 ? hi : lo); }
+                if (row == 0 || (row == 1 && n < 3)) put_word(dst, e + 1u, val);
+                if (row == 0) {
+                    sl[2 * 16 + n] = (double)aa;
+                    sl[3 * 16 + n] = (double)bb;
+                    sl[4 * 16 + n] = pp;
+                }
             }
         }
         if (tr && fx.tid == 0) tr[4] = wall_clock64();
 
         // ===================== phase 2: att output =============================
+        // The next layer's owner record (l + 1 == L: the head's scalars) is fetched here, where every wave
+        // is about to wait for the other workgroups anyway: the copy to LDS has to wait for the loads.
+        RWKV_IDS();
+        stage_owner_record<FT, KW>(a, l + 1, g, G, C, own_lds, fx.tid);
         vec_front<KW, FW, NQTC>(fx, seq, a.b.A, a.b.AR, NQC, e + 1u, dig, PS, stat, tr ? tr + 5 : nullptr, tr ? tr + 17 : nullptr);
         if (!fx.ok) break;
         __syncthreads();
@@ -689,7 +708,6 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
         RWKV_IDS();
         // the LayerNorm output of the own channel is the new ffn shift state (block.py:82,87-88)
         if (fin && row == 0) sl[16 + n] = or_d(rec, OR_LN2W * 16 + n) * ((x_lds[n] - stat[0]) * stat[1]) + or_d(rec, OR_LN2B * 16 + n);
-        stage_owner_record<FT, KW>(a, l + 1, g, G, C, own_lds, fx.tid);   // while the matrix cores run (l + 1 == L: the head's scalars)
         __syncthreads();
         if (tr && fx.tid == 0) tr[11] = wall_clock64();
         if (fin) {
