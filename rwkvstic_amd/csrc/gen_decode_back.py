@@ -37,6 +37,8 @@ PF = NA - 1       # A-operand reads run this many positions ahead
 import os
 WINDOW = int(os.environ.get("RWKV_BACK_WINDOW", "5"))
 DEFER = int(os.environ.get("RWKV_BACK_DEFER", "1"))
+# per-phase windows for the reloads that follow the barrier of the att k/v/r, att output, ffn key and ffn value phases
+WINDOWS = [int(x) for x in os.environ.get("RWKV_BACK_WINDOWS", ",".join([str(WINDOW)] * 4)).split(",")]
 BURST = int(os.environ.get("RWKV_BACK_BURST", "0"))      # the first BURST reloads after a phase's barrier go out back to back
 SLEEP = int(os.environ.get("RWKV_BACK_SLEEP", "0"))      # s_sleep units (64 cycles) between a phase's barrier and its reloads   # weight loads a wave keeps in flight while it reloads slots
 
@@ -186,7 +188,7 @@ def gen(KW, R, NV, NSH):
             e(f"global_load_dwordx4 {ring(slot)}, v{V_OFF + bq}, s[{sset + 2 * jq}:{sset + 2 * jq + 1}]")
 
     e("1:")
-    for ps, pe, nbar in phases:
+    for ph, (ps, pe, nbar) in enumerate(phases):
         for _ in range(nbar):
             bar_check()
         for q in range(ps, min(ps + PF, pe)):
@@ -224,7 +226,7 @@ def gen(KW, R, NV, NSH):
             e(f"s_sleep {SLEEP}")
         for i, p in enumerate(deferred):
             assert issued_loads == p + R
-            layer_reload(p, max(BURST, WINDOW) if i < BURST else WINDOW)
+            layer_reload(p, max(BURST, WINDOWS[ph]) if i < BURST else WINDOWS[ph])
             issued_loads += 1
     # end of layer: next layer's addresses become current; fetch the layer after
     e(f"s_add_u32 s{S_JT}, s{S_JT}, 128")
