@@ -65,9 +65,8 @@ struct DModel {
     double *PO;                  // [L+1][5][C]
     DScal *sc;                   // [L+1]
     DScal *scp;                  // [L][C/512] per-token scalars (sumQO, maxQ) of each 512-channel part of a layer
-    double *amax_val;            // scratch of the device-side argmax: per block maximum, its index, arrival counter
+    double *amax_val;            // [G] device-side argmax: first maximum of the logits each workgroup wrote, and its index
     int *amax_idx;
-    unsigned *amax_count;
     double *X0;                  // [C] ln0(emb[token]) of the launch in flight
 };
 

@@ -60,6 +60,7 @@ constexpr int kBW = 8;                 // back (streaming) waves per workgroup
 constexpr int kRealJobs = 13;          // tile jobs per layer: k v r | o | ffn_r, 4 x ffn_k | 4 quarters of ffn_v
 constexpr unsigned kSpinLimit = 1u << 20;
 constexpr int kLnRows = 2 + 3 * 3;     // rows of the XR record table
+constexpr int kHeadCsPerThread = 4;    // head column sums a front thread fetches: 16 per head tile of the workgroup
 
 // LDS flag words
 enum { FLAG_ARRIVED = 0, FLAG_SCALE = 1, FLAG_ABORT = 2, FLAG_COUNT = 4 };
@@ -752,10 +753,23 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
     // ========================= head (opt.py:71-73) ==============================
     const int v_tiles = (V + 15) / 16, head_rounds = (v_tiles + G - 1) / G;
     const u64 *rec_h = own_lds + (L & 1) * kOrSlots;
+    // column sums of the workgroup's head tiles: requested now, parked in the LDS half that held the
+    // last layer's record once the wait for x is over (a load inside the loop below would cost a
+    // round trip through the busy memory pipeline in every round)
+    int *csh = reinterpret_cast<int *>(own_lds + ((L + 1) & 1) * kOrSlots);
+    int csv[kHeadCsPerThread];
+#pragma unroll
+    for (int k = 0; k < kHeadCsPerThread; ++k) {
+        const int i = fx.tid + FT * k, v = 16 * (g + G * (i >> 4)) + (i & 15);
+        csv[k] = (i < head_rounds * 16 && v < V) ? a.m.cs_head[v] : 0;
+    }
     if (fx.ok)
         ln_front<KW, FW, 1>(fx, seq, a, a.m.P32 + (size_t)L * kLnMats * C, a.m.Q32 + (size_t)L * kLnMats * C, rec_h, 0,
                             a.epoch0 + 4u * (unsigned)L, dig, stat, nullptr, nullptr);
     if (!fx.ok) return;     // every wave leaves after the same barrier: the flag is tested after each one that follows a wait
+#pragma unroll
+    for (int k = 0; k < kHeadCsPerThread; ++k)
+        if (fx.tid + FT * k < head_rounds * 16) csh[fx.tid + FT * k] = csv[k];
     RWKV_IDS();
 #undef RWKV_IDS
     unsigned par = 0;
@@ -764,13 +778,29 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
     float invSh;
     ln_scale(stat, rec_h, 0, 0, Sh, invSh);
     const double zph = ln_zp(stat, rec_h, 0, 0);
+    double best = -INFINITY;                               // first maximum of the logits this thread writes
+    int best_i = 0x7fffffff;
     for (int h0 = 0; h0 < head_rounds; h0 += NS, par ^= 1u) {
-        __syncthreads();
+        __syncthreads();                                   // (the first one also orders the csh writes above)
         const int s = fx.tid >> 4;                         // parked tile of this round
         if (s < NS && h0 + s < head_rounds) {
             const int v = 16 * (g + G * (h0 + s)) + n;
-            if (v < V) a.logits[v] = finish_col(red + par * (NS * kBW * 16), s, n, Sh, a.m.cs_head[v], zph);
+            if (v < V) {
+                const double y = finish_col(red + par * (NS * kBW * 16), s, n, Sh, csh[16 * (h0 + s) + n], zph);
+                a.logits[v] = y;
+                if (y > best) { best = y; best_i = v; }    // v grows with the round: an equal later value does not replace
+            }
         }
+    }
+    // the workgroup's candidate for the greedy token: threads 0 .. 16 NS - 1 of wave 0 hold the values
+    if (fx.wave == 0) {
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            const double ob = __shfl_xor(best, off, 64);
+            const int oi = __shfl_xor(best_i, off, 64);
+            if (ob > best || (ob == best && oi < best_i)) { best = ob; best_i = oi; }
+        }
+        if (fx.lane == 0) { a.m.amax_val[g] = best; a.m.amax_idx[g] = best_i; }
     }
     // the state rows of the own channels: st_lds[l][row][n] -> state[l][row][16 g + n]
     for (int i = fx.tid; i < L * 5 * 16; i += FT) a.state[(size_t)(i >> 4) * C + 16 * g + (i & 15)] = st_lds[i];
@@ -932,65 +962,35 @@ __global__ void __launch_bounds__(kPrepThreads) prep_kernel(const DArgs a) {
     else prep_token(a, a.token[0], a.epoch0, scr);
 }
 
-// Between two greedy tokens: argmax of the logits just produced -> out_token[0], and the
-// preparation of the next step (which reads the state the step before has just updated) in the same
-// launch.  grid: L * (C / 512) layer parts, then kArgmaxBlocks blocks that scan the logits; the one
-// that finishes last reduces their results, writes the token and prepares it.  a.epoch0: the epoch
-// of the NEXT token step.
-constexpr int kArgmaxBlocks = 32;
-
+// Between two greedy tokens: the greedy token (the single-token kernel left one candidate per
+// workgroup: the first maximum of the logits it wrote) -> out_token[0], and the preparation of the
+// next step (which reads the state the step before has just updated) in the same launch.
+// grid: L * (C / 512) layer parts, then one block for the token.  a.epoch0: the epoch of the NEXT
+// token step.
 __global__ void __launch_bounds__(kPrepThreads) next_token_kernel(const DArgs a, int64_t *__restrict__ out_token) {
     __shared__ double scr[8 * (kPrepThreads / 64)];
     __shared__ int sidx[kPrepThreads / 64];
-    __shared__ int last_flag;
     const int parts = a.m.C / kPrepThreads;
     const int b = blockIdx.x;
     if (b < a.m.L * parts) { prep_layer_part(a, b / parts, b % parts, scr); return; }
-    const int ab = b - a.m.L * parts, V = a.m.V;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     auto better = [](double v, int i, double bv, int bi) { return v > bv || (v == bv && i < bi); };
-    auto block_argmax = [&](double &best, int &bi) {        // result in thread 0
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) {
-            const double ob = __shfl_xor(best, off, 64);
-            const int oi = __shfl_xor(bi, off, 64);
-            if (better(ob, oi, best, bi)) { best = ob; bi = oi; }
-        }
-        __syncthreads();
-        if (lane == 0) { scr[wave] = best; sidx[wave] = bi; }
-        __syncthreads();
-        if (threadIdx.x == 0)
-            for (int wv = 1; wv < kPrepThreads / 64; ++wv)
-                if (better(scr[wv], sidx[wv], best, bi)) { best = scr[wv]; bi = sidx[wv]; }
-    };
     double best = -INFINITY;
     int bi = 0x7fffffff;
-    const int chunk = (V + kArgmaxBlocks - 1) / kArgmaxBlocks;
-    const int i1 = (ab + 1) * chunk < V ? (ab + 1) * chunk : V;
-    for (int i = ab * chunk + threadIdx.x; i < i1; i += kPrepThreads) {
-        const double x = a.logits[i];
-        if (better(x, i, best, bi)) { best = x; bi = i; }
+    if ((int)threadIdx.x < a.m.G) { best = a.m.amax_val[threadIdx.x]; bi = a.m.amax_idx[threadIdx.x]; }   // G <= 256
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const double ob = __shfl_xor(best, off, 64);
+        const int oi = __shfl_xor(bi, off, 64);
+        if (better(ob, oi, best, bi)) { best = ob; bi = oi; }
     }
-    block_argmax(best, bi);
-    if (threadIdx.x == 0) {
-        a.m.amax_val[ab] = best;
-        a.m.amax_idx[ab] = bi;
-        __threadfence();
-        last_flag = atomicAdd(a.m.amax_count, 1u) == kArgmaxBlocks - 1;
-    }
+    if (lane == 0) { scr[wave] = best; sidx[wave] = bi; }
     __syncthreads();
-    if (!last_flag) return;
-    __threadfence();
-    best = -INFINITY; bi = 0x7fffffff;
-    if (threadIdx.x < kArgmaxBlocks) {
-        best = __hip_atomic_load(a.m.amax_val + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        bi = __hip_atomic_load(a.m.amax_idx + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    block_argmax(best, bi);
     if (threadIdx.x == 0) {
+        for (int wv = 1; wv < kPrepThreads / 64; ++wv)
+            if (better(scr[wv], sidx[wv], best, bi)) { best = scr[wv]; bi = sidx[wv]; }
         sidx[0] = bi == 0x7fffffff ? 0 : bi;
         out_token[0] = sidx[0];
-        *a.m.amax_count = 0u;                                // ready for the next launch
     }
     __syncthreads();
     prep_token(a, (int64_t)sidx[0], a.epoch0, scr);
@@ -1152,7 +1152,10 @@ __global__ void __launch_bounds__(kPrepThreads) build_consts_kernel(const ConstA
 bool decode_supported(int64_t L, int64_t C, int64_t F, int64_t V) {
     if (L <= 0 || V <= 0 || F != 4 * C) return false;
     // one 16-column tile per workgroup, all workgroups resident: C/16 <= 256 CUs
-    return C == 1024 || C == 2048 || C == 2560 || C == 4096;
+    if (!(C == 1024 || C == 2048 || C == 2560 || C == 4096)) return false;
+    // the column sums of a workgroup's head tiles are staged by its front threads into half an owner record
+    const int64_t G = C / 16, head_rounds = ((V + 15) / 16 + G - 1) / G, front_threads = C == 2560 ? 512 : 256;
+    return head_rounds * 16 <= kHeadCsPerThread * front_threads && head_rounds * 16 * (int64_t)sizeof(int) <= kOrSlots * 8;
 }
 
 unsigned decode_epochs_per_token(int64_t L) { return (unsigned)(4 * L + 1); }
@@ -1179,7 +1182,7 @@ BlockPlan plan_block(int64_t L, int64_t C, int64_t F, int64_t V) {
     p.ownrec = take((size_t)L * G * kOrSlots * sizeof(u64));
     p.jt = take(G * (size_t)(L + 1) * 16 * sizeof(u64));
     p.scp = take((size_t)L * (C / 512) * sizeof(DScal));
-    p.amax = take(kArgmaxBlocks * (sizeof(double) + sizeof(int)) + 64);
+    p.amax = take((size_t)G * (sizeof(double) + sizeof(int)));
     p.xchg = take(((size_t)2 * C + F + (size_t)(kLnRows + 6) * G) * sizeof(u64));
     p.abort = take(256);
     p.total = off;
@@ -1237,8 +1240,7 @@ int decode_setup(void *block, const DSetup &s, DModel *dm, DecodeBuffers *db) {
     dm->ownrec = reinterpret_cast<const u64 *>(base + p.ownrec);
     dm->scp = reinterpret_cast<DScal *>(base + p.scp);
     dm->amax_val = reinterpret_cast<double *>(base + p.amax);
-    dm->amax_idx = reinterpret_cast<int *>(base + p.amax + kArgmaxBlocks * sizeof(double));
-    dm->amax_count = reinterpret_cast<unsigned *>(base + p.amax + kArgmaxBlocks * (sizeof(double) + sizeof(int)));
+    dm->amax_idx = reinterpret_cast<int *>(base + p.amax + (size_t)G * sizeof(double));
     dm->layers = reinterpret_cast<const DLayer *>(base + p.layers);
     dm->prep = reinterpret_cast<const DPrep *>(base + p.prep);
     dm->P32 = reinterpret_cast<float *>(base + p.P32);
@@ -1327,7 +1329,7 @@ int decode_launch_greedy(hipStream_t st, const DModel &m, const DecodeBuffers &b
         // argmax -> tokens[i + 1], and the preparation of step i + 1 (harmless after the last step:
         // the next forward call prepares again under the same epoch)
         args.epoch0 += ept;
-        hipLaunchKernelGGL(next_token_kernel, dim3((unsigned)(m.L * (m.C / kPrepThreads) + kArgmaxBlocks)),
+        hipLaunchKernelGGL(next_token_kernel, dim3((unsigned)(m.L * (m.C / kPrepThreads) + 1)),
                            dim3(kPrepThreads), 0, st, args, tokens + i + 1);
         RWKV_CHECK_LAUNCH("next_token_kernel");
     }
