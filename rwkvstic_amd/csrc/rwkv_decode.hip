@@ -60,6 +60,7 @@ constexpr int kBW = 8;                 // back (streaming) waves per workgroup
 constexpr int kRealJobs = 13;          // tile jobs per layer: k v r | o | ffn_r, 4 x ffn_k | 4 quarters of ffn_v
 constexpr unsigned kSpinLimit = 1u << 20;
 constexpr int kLnRows = 2 + 3 * 3;     // rows of the XR record table
+constexpr int kEarlyDiv = 4;           // gathers start when all but G / kEarlyDiv workgroups have published (measured flat from G/20 to G)
 constexpr int kHeadCsPerThread = 4;    // head column sums a front thread fetches: 16 per head tile of the workgroup
 
 // LDS flag words
@@ -218,19 +219,32 @@ struct RowPoll {
     static constexpr int PAIRS = NR * G / 2, K = (PAIRS + 63) / 64;
     static_assert(G % 2 == 0, "two words per lane");
     float v[K][2];
-    __device__ __forceinline__ void poll(Front &fx, const u64 *rows, unsigned epoch) {
+    // early_seq != 0: FLAG_ARRIVED is raised to early_seq as soon as at most `early_missing` words are
+    // still outstanding (at the latest when none is) and on_early() runs, so that the gathers overlap
+    // the wait for the last few workgroups; the words that had not arrived are re-read later.
+    struct Nothing { __device__ __forceinline__ void operator()() const {} };
+    template <typename F = Nothing>
+    __device__ __forceinline__ void poll(Front &fx, const u64 *rows, unsigned epoch, int early_seq = 0, int early_missing = 0, F on_early = F()) {
         const xtab_t t = make_xtab(rows, NR * G);
         v4u w[K];
         unsigned spins = 0;
+        bool raised = early_seq == 0;
         while (fx.ok) {
-            bool all = true;
+            int missing = 0;
 #pragma unroll
             for (int k = 0; k < K; ++k)
                 if (fx.lane + 64 * k < PAIRS) w[k] = __builtin_amdgcn_raw_buffer_load_b128(t, (fx.lane + 64 * k) * 16, 0, kAuxAgent);
 #pragma unroll
-            for (int k = 0; k < K; ++k)
-                if (fx.lane + 64 * k < PAIRS) all = all && w[k].y == epoch && w[k].w == epoch;
-            if (__ballot(!all) == 0ull) break;
+            for (int k = 0; k < K; ++k) {
+                const bool in = fx.lane + 64 * k < PAIRS;
+                missing += __popcll(__ballot(in && w[k].y != epoch)) + __popcll(__ballot(in && w[k].w != epoch));
+            }
+            if (!raised && missing <= early_missing) {
+                if (fx.lane == 0) fx.flags[FLAG_ARRIVED] = early_seq;
+                raised = true;
+                on_early();                    // this wave's own gather
+            }
+            if (missing == 0) break;
             __builtin_amdgcn_s_sleep(2);
             if ((++spins & 63u) == 0u && (spins > kSpinLimit || ALOAD32(fx.abort_flag) != 0u || fx.flags[FLAG_ABORT])) fx.fail();
         }
@@ -285,22 +299,30 @@ __device__ __forceinline__ void issue_quads(xtab_t src, int ft, int first, int n
         }
     }
 }
-// Re-reads until every word of the thread's quads carries the epoch (normally the first read does).
+// Re-reads the quads that hold a word without the epoch until none is left (normally the first
+// read is complete; with an early start of the gathers the last workgroups' words come later).
 template <int FT, int N>
 __device__ __forceinline__ void settle_quads(Front &fx, xtab_t src, int first, int nq, unsigned epoch, u64 (&w)[N][4]) {
     unsigned spins = 0;
     while (fx.ok) {
         bool all = true;
 #pragma unroll
-        for (int i = 0; i < N; ++i)
-            if (fx.tid + FT * (first + i) < nq) {
+        for (int i = 0; i < N; ++i) {
+            const int qi = fx.tid + FT * (first + i);
+            bool good = true;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) all = all && ((unsigned)(w[i][e] >> 32) == epoch);
+            for (int e = 0; e < 4; ++e) good = good && ((unsigned)(w[i][e] >> 32) == epoch);
+            if (qi < nq && !good) {
+                all = false;
+                const v4u lo = __builtin_amdgcn_raw_buffer_load_b128(src, qi * 32, 0, kAuxAgent);
+                const v4u hi = __builtin_amdgcn_raw_buffer_load_b128(src, qi * 32 + 16, 0, kAuxAgent);
+                w[i][0] = ((u64)lo.y << 32) | lo.x; w[i][1] = ((u64)lo.w << 32) | lo.z;
+                w[i][2] = ((u64)hi.y << 32) | hi.x; w[i][3] = ((u64)hi.w << 32) | hi.z;
             }
+        }
         if (all) break;
-        __builtin_amdgcn_s_sleep(1);
+        __builtin_amdgcn_s_sleep(4);
         if ((++spins & 63u) == 0u && (spins > kSpinLimit || ALOAD32(fx.abort_flag) != 0u)) { fx.fail(); break; }
-        issue_quads<FT, N>(src, fx.tid, first, nq, w);
     }
 }
 
@@ -499,10 +521,8 @@ __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, co
     const xtab_t xt = make_xtab(a.b.X, C);
     if (fx.wave == 0) {
         RowPoll<2, G> r;
-        r.poll(fx, a.b.XR, epoch);
-        if (fx.lane == 0) fx.flags[FLAG_ARRIVED] = seq;
+        r.poll(fx, a.b.XR, epoch, seq, 2 * (G / kEarlyDiv), [&] { issue_quads<FT, NQT>(xt, fx.tid, 0, NQ, w); });
         if (tp && fx.tid == 0) tp[0] = wall_clock64();
-        issue_quads<FT, NQT>(xt, fx.tid, 0, NQ, w);
         const double s0 = wave_sum_dpp(r.lane_sum(fx, 0)), s1 = wave_sum_dpp(r.lane_sum(fx, 1));
         const double mean = s0 * (1.0 / (double)C);
         double var = s1 * (1.0 / (double)C) - mean * mean;
@@ -572,10 +592,8 @@ __device__ __forceinline__ void vec_front(Front &fx, int &seq, const u64 *src, c
     float invS;
     if (fx.wave == 0) {
         RowPoll<3, G> r;
-        r.poll(fx, rec, epoch);
-        if (fx.lane == 0) fx.flags[FLAG_ARRIVED] = seq;
+        r.poll(fx, rec, epoch, seq, 3 * (G / kEarlyDiv), [&] { issue_quads<FT, CH>(st, fx.tid, 0, nq, w[0]); });
         if (tp && fx.tid == 0) tp[0] = wall_clock64();
-        issue_quads<FT, CH>(st, fx.tid, 0, nq, w[0]);
         const float mx = wave_max_dpp(r.lane_max(fx, 0));
         const double so = wave_sum_dpp(r.lane_sum(fx, 1) + r.lane_sum(fx, 2));
         double S;
