@@ -211,41 +211,66 @@ __global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
 // ---------------------------------------------------------------------------
 // GEMM: tot[t, j] = sum_k q[t, k] * (code[k, j] - 128), exact in int64.
 // Workgroup = 4 wavefronts = 64 tokens x 64 columns; wavefront (wm, wn) holds
-// 8 M-tiles x 2 N-tiles of accumulators and streams fragments of both operands
-// straight from memory (software-pipelined one block ahead).  gridDim.z splits
-// the contraction; partial totals are then added with integer atomics, which
+// 8 M-tiles x 2 N-tiles of accumulators.  The contraction may be split over
+// several workgroups; partial totals are then added with integer atomics, which
 // commute exactly.
+//
+// Launch order.  Workgroups are handed to the 8 XCDs round robin, and each XCD has its own L2.  The
+// grid is 1-D and workgroup i works for XCD i % 8 on that XCD's own row blocks (row block r belongs
+// to XCD r % 8), walking through the column blocks with the row blocks innermost: the digit
+// fragments of an XCD's rows (a few hundred KB) stay in its L2 for the whole product, and a weight
+// block fetched for one row block is reused by the next.  Without this every XCD pulls every digit
+// fragment through the fabric once per column block.
 // ---------------------------------------------------------------------------
+constexpr int kXcds = 8;
 struct GemmArgs {
     const signed char *dig;     // fragments [MT][KB][1024]
     const uint8_t *w16;         // blocks [NT][KB][1024]
     long long *tot;             // [4*MT][ldd]
     int MT, NT, KB, ldd, kb_per_split, atomic;
+    int gx, gy, gz, rows_per_xcd;   // logical grid (column blocks, row blocks, splits) behind the 1-D launch
 };
 
 constexpr int kGM = 8, kGN = 2;
 
-__global__ void __launch_bounds__(256) gemm8_kernel(const GemmArgs a) {
+constexpr int kGemmFrags = 16 + 4;      // fragments of one contraction block: 16 M-tiles of digits, 4 N-tiles of weights
+constexpr int kGemmLoads = kGemmFrags / 4;   // per thread and contraction block (wave w fetches fragments w, w + 4, ...)
+constexpr int kGemmAhead = 3;           // contraction blocks on their way from memory
+
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) gemm8_kernel(const GemmArgs a) {
+    // Both operands of a contraction block are fetched once per workgroup (registers, kGemmAhead
+    // blocks ahead), parked in LDS (two buffers, one barrier per block) and read from there by the
+    // two wavefronts that need each fragment.
+    __shared__ v4i frag[2][kGemmFrags][64];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave & 1, wn = wave >> 1;
-    const int mt0 = blockIdx.y * 16 + wm * kGM, nt0 = blockIdx.x * 4 + wn * kGN;
-    const int kb0 = blockIdx.z * a.kb_per_split;
+    const int xcd = blockIdx.x % kXcds;
+    int item = blockIdx.x / kXcds;                      // (split, column block, row slot) of this XCD, row slot fastest
+    const int rslot = item % a.rows_per_xcd; item /= a.rows_per_xcd;
+    const int bx = item % a.gx, bz = item / a.gx;
+    const int by = xcd + kXcds * rslot;
+    if (by >= a.gy || bz >= a.gz) return;
+    const int mt0 = by * 16 + wm * kGM, nt0 = bx * 4 + wn * kGN;
+    const int kb0 = bz * a.kb_per_split;
     int kb1 = kb0 + a.kb_per_split;
     if (kb1 > a.KB) kb1 = a.KB;
-    if (mt0 >= a.MT || nt0 >= a.NT || kb0 >= kb1) return;
+    if (kb0 >= kb1) return;                             // (uniform for the workgroup)
+    const int nk = kb1 - kb0;
 
-    const uint4 *ap[kGM];
-    const uint4 *bp[kGN];
+    const v4i *src[kGemmLoads];
 #pragma unroll
-    for (int i = 0; i < kGM; ++i) {
-        const int mt = mt0 + i < a.MT ? mt0 + i : a.MT - 1;       // clamped: loads stay unconditional
-        ap[i] = reinterpret_cast<const uint4 *>(a.dig + ((size_t)mt * a.KB + kb0) * 1024) + lane;
-    }
-#pragma unroll
-    for (int j = 0; j < kGN; ++j) {
-        const int nt = nt0 + j < a.NT ? nt0 + j : a.NT - 1;
-        bp[j] = reinterpret_cast<const uint4 *>(a.w16 + ((size_t)nt * a.KB + kb0) * 1024) + lane;
+    for (int i = 0; i < kGemmLoads; ++i) {
+        const int f = wave + 4 * i;                     // fragment this thread helps to fetch
+        if (f < 16) {
+            int mt = by * 16 + f;
+            if (mt >= a.MT) mt = a.MT - 1;              // clamped: loads stay unconditional, results are dropped
+            src[i] = reinterpret_cast<const v4i *>(a.dig + ((size_t)mt * a.KB + kb0) * 1024) + lane;
+        } else {
+            int nt = bx * 4 + (f - 16);
+            if (nt >= a.NT) nt = a.NT - 1;
+            src[i] = reinterpret_cast<const v4i *>(a.w16 + ((size_t)nt * a.KB + kb0) * 1024) + lane;
+        }
     }
     v4i acc[kGM][kGN];
 #pragma unroll
@@ -253,33 +278,42 @@ __global__ void __launch_bounds__(256) gemm8_kernel(const GemmArgs a) {
 #pragma unroll
         for (int j = 0; j < kGN; ++j) acc[i][j] = v4i{0, 0, 0, 0};
 
-    uint4 A[kGM], B[kGN];
-#pragma unroll
-    for (int i = 0; i < kGM; ++i) A[i] = ap[i][0];
-#pragma unroll
-    for (int j = 0; j < kGN; ++j) B[j] = bp[j][0];
-    const int nk = kb1 - kb0;
-    for (int k = 0; k < nk; ++k) {
-        uint4 An[kGM], Bn[kGN];
-        const int kn = k + 1 < nk ? k + 1 : k;                    // last step reloads itself (unused)
-#pragma unroll
-        for (int i = 0; i < kGM; ++i) An[i] = ap[i][(size_t)kn * 64];
-#pragma unroll
-        for (int j = 0; j < kGN; ++j) Bn[j] = bp[j][(size_t)kn * 64];
-#pragma unroll
-        for (int i = 0; i < kGM; ++i) {
-            const v4i Av = {(int)A[i].x, (int)A[i].y, (int)A[i].z, (int)A[i].w};
-#pragma unroll
-            for (int j = 0; j < kGN; ++j) {
-                const v4i Bv = {(int)B[j].x, (int)B[j].y, (int)B[j].z, (int)B[j].w};
-                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Av, Bv, acc[i][j], 0, 0, 0);
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < kGM; ++i) A[i] = An[i];
-#pragma unroll
-        for (int j = 0; j < kGN; ++j) B[j] = Bn[j];
+    // the blocks in flight live in three separately named register sets: an array indexed by the
+    // stage would be indexed dynamically once the loop is rotated, and end up in scratch memory
+    static_assert(kGemmAhead == 3, "three named stages below");
+    static_assert(kGemmLoads == 5, "five named members below");
+    struct Fly { v4i v0, v1, v2, v3, v4; };           // named members, not an array: they must stay registers
+    Fly fly0, fly1, fly2;
+#define RWKV_GEMM_FETCH(F, K)                                                                        \
+    do {                                                                                             \
+        const size_t o_ = (size_t)((K) < nk ? (K) : nk - 1) * 64; /* past the end: the last block again (unused) */ \
+        F.v0 = src[0][o_]; F.v1 = src[1][o_]; F.v2 = src[2][o_]; F.v3 = src[3][o_]; F.v4 = src[4][o_]; \
+    } while (0)
+#define RWKV_GEMM_STEP(F, K)                                                                         \
+    if ((K) < nk) { /* uniform */                                                                    \
+        const int buf_ = (K) & 1;                                                                    \
+        frag[buf_][wave][lane] = F.v0; frag[buf_][wave + 4][lane] = F.v1; frag[buf_][wave + 8][lane] = F.v2;     \
+        frag[buf_][wave + 12][lane] = F.v3; frag[buf_][wave + 16][lane] = F.v4;                      \
+        RWKV_GEMM_FETCH(F, (K) + kGemmAhead);                                                        \
+        __syncthreads();                                                                             \
+        v4i Bv_[kGN];                                                                                \
+        _Pragma("unroll") for (int j = 0; j < kGN; ++j) {                                            \
+            Bv_[j] = frag[buf_][16 + wn * kGN + j][lane];                                            \
+        }                                                                                            \
+        _Pragma("unroll") for (int i = 0; i < kGM; ++i) {                                            \
+            const v4i Av_ = frag[buf_][wm * kGM + i][lane];                                          \
+            _Pragma("unroll") for (int j = 0; j < kGN; ++j)                                          \
+                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Av_, Bv_[j], acc[i][j], 0, 0, 0);  \
+        }                                                                                            \
     }
+    RWKV_GEMM_FETCH(fly0, 0); RWKV_GEMM_FETCH(fly1, 1); RWKV_GEMM_FETCH(fly2, 2);
+    for (int k0 = 0; k0 < nk; k0 += kGemmAhead) {
+        RWKV_GEMM_STEP(fly0, k0)
+        RWKV_GEMM_STEP(fly1, k0 + 1)
+        RWKV_GEMM_STEP(fly2, k0 + 2)
+    }
+#undef RWKV_GEMM_STEP
+#undef RWKV_GEMM_FETCH
     // lane 16g + n, register i  <->  digit i of token 4*mt + g, column 16*nt + n
     const int g = lane >> 4, n = lane & 15;
 #pragma unroll
@@ -473,7 +507,8 @@ int rows_matmul(hipStream_t st, const RowsScratch &s, int64_t R, int64_t K, int6
         const size_t n = (size_t)g.MT * 4 * g.ldd;
         hipLaunchKernelGGL(rows_fill_kernel, dim3((unsigned)ceil_div((int64_t)n, 1024)), dim3(256), 0, st, s.tot, n);
     }
-    hipLaunchKernelGGL(gemm8_kernel, dim3(gx, gy, split), dim3(256), 0, st, g);
+    g.gx = gx; g.gy = gy; g.gz = split; g.rows_per_xcd = (gy + kXcds - 1) / kXcds;
+    hipLaunchKernelGGL(gemm8_kernel, dim3((unsigned)(kXcds * g.rows_per_xcd * gx * split)), dim3(256), 0, st, g);
     RWKV_CHECK_LAUNCH("gemm8_kernel");
 
     FinishArgs f;
