@@ -210,8 +210,8 @@ __global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
 
 // ---------------------------------------------------------------------------
 // GEMM: tot[t, j] = sum_k q[t, k] * (code[k, j] - 128), exact in int64.
-// Workgroup = 4 wavefronts = 64 tokens x 64 columns; wavefront (wm, wn) holds
-// 8 M-tiles x 2 N-tiles of accumulators.  The contraction may be split over
+// Workgroup = 4 wavefronts = 64 tokens x 128 columns; wavefront (wm, wn) holds
+// 8 M-tiles x 4 N-tiles of accumulators.  The contraction may be split over
 // several workgroups; partial totals are then added with integer atomics, which
 // commute exactly.
 //
@@ -231,11 +231,19 @@ struct GemmArgs {
     int gx, gy, gz, rows_per_xcd;   // logical grid (column blocks, row blocks, splits) behind the 1-D launch
 };
 
-constexpr int kGM = 8, kGN = 2;
+#ifndef RWKV_GEMM_GN
+#define RWKV_GEMM_GN 4
+#endif
+constexpr int kGM = 8, kGN = RWKV_GEMM_GN;   // M-tiles x N-tiles of accumulators per wavefront
+constexpr int kGemmNT = 2 * kGN;         // N-tiles per workgroup (two wavefronts side by side)
 
-constexpr int kGemmFrags = 16 + 4;      // fragments of one contraction block: 16 M-tiles of digits, 4 N-tiles of weights
+constexpr int kGemmFrags = 16 + kGemmNT; // fragments of one contraction block: 16 M-tiles of digits, kGemmNT N-tiles of weights
 constexpr int kGemmLoads = kGemmFrags / 4;   // per thread and contraction block (wave w fetches fragments w, w + 4, ...)
 constexpr int kGemmAhead = 3;           // contraction blocks on their way from memory
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global load
+// the wavefront has in flight, which would drain the prefetched contraction blocks at every step.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) gemm8_kernel(const GemmArgs a) {
     // Both operands of a contraction block are fetched once per workgroup (registers, kGemmAhead
@@ -251,7 +259,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int bx = item % a.gx, bz = item / a.gx;
     const int by = xcd + kXcds * rslot;
     if (by >= a.gy || bz >= a.gz) return;
-    const int mt0 = by * 16 + wm * kGM, nt0 = bx * 4 + wn * kGN;
+    const int mt0 = by * 16 + wm * kGM, nt0 = bx * kGemmNT + wn * kGN;
     const int kb0 = bz * a.kb_per_split;
     int kb1 = kb0 + a.kb_per_split;
     if (kb1 > a.KB) kb1 = a.KB;
@@ -267,7 +275,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
             if (mt >= a.MT) mt = a.MT - 1;              // clamped: loads stay unconditional, results are dropped
             src[i] = reinterpret_cast<const v4i *>(a.dig + ((size_t)mt * a.KB + kb0) * 1024) + lane;
         } else {
-            int nt = bx * 4 + (f - 16);
+            int nt = bx * kGemmNT + (f - 16);
             if (nt >= a.NT) nt = a.NT - 1;
             src[i] = reinterpret_cast<const v4i *>(a.w16 + ((size_t)nt * a.KB + kb0) * 1024) + lane;
         }
@@ -281,21 +289,21 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     // the blocks in flight live in three separately named register sets: an array indexed by the
     // stage would be indexed dynamically once the loop is rotated, and end up in scratch memory
     static_assert(kGemmAhead == 3, "three named stages below");
-    static_assert(kGemmLoads == 5, "five named members below");
-    struct Fly { v4i v0, v1, v2, v3, v4; };           // named members, not an array: they must stay registers
+    static_assert(kGemmLoads == 6 || kGemmLoads == 5, "named members below");
+    struct Fly { v4i v0, v1, v2, v3, v4, v5; };           // named members, not an array: they must stay registers
     Fly fly0, fly1, fly2;
 #define RWKV_GEMM_FETCH(F, K)                                                                        \
     do {                                                                                             \
         const size_t o_ = (size_t)((K) < nk ? (K) : nk - 1) * 64; /* past the end: the last block again (unused) */ \
-        F.v0 = src[0][o_]; F.v1 = src[1][o_]; F.v2 = src[2][o_]; F.v3 = src[3][o_]; F.v4 = src[4][o_]; \
+        F.v0 = src[0][o_]; F.v1 = src[1][o_]; F.v2 = src[2][o_]; F.v3 = src[3][o_]; F.v4 = src[4][o_]; if (kGemmLoads > 5) F.v5 = src[kGemmLoads - 1][o_]; \
     } while (0)
 #define RWKV_GEMM_STEP(F, K)                                                                         \
     if ((K) < nk) { /* uniform */                                                                    \
         const int buf_ = (K) & 1;                                                                    \
         frag[buf_][wave][lane] = F.v0; frag[buf_][wave + 4][lane] = F.v1; frag[buf_][wave + 8][lane] = F.v2;     \
-        frag[buf_][wave + 12][lane] = F.v3; frag[buf_][wave + 16][lane] = F.v4;                      \
+        frag[buf_][wave + 12][lane] = F.v3; frag[buf_][wave + 16][lane] = F.v4; if (kGemmLoads > 5) frag[buf_][wave + 4 * (kGemmLoads - 1)][lane] = F.v5; \
         RWKV_GEMM_FETCH(F, (K) + kGemmAhead);                                                        \
-        __syncthreads();                                                                             \
+        lds_barrier();                                                                               \
         v4i Bv_[kGN];                                                                                \
         _Pragma("unroll") for (int j = 0; j < kGN; ++j) {                                            \
             Bv_[j] = frag[buf_][16 + wn * kGN + j][lane];                                            \
@@ -496,10 +504,10 @@ int rows_matmul(hipStream_t st, const RowsScratch &s, int64_t R, int64_t K, int6
     GemmArgs g;
     g.dig = s.dig; g.w16 = w16; g.tot = s.tot;
     g.MT = (int)ceil_div(R, 4); g.NT = (int)ceil_div(N, 16); g.KB = (int)(K / 64); g.ldd = g.NT * 16;
-    const int gx = (int)ceil_div(g.NT, 4), gy = (int)ceil_div(g.MT, 16);
+    const int gx = (int)ceil_div(g.NT, kGemmNT), gy = (int)ceil_div(g.MT, 16);
     // Split the contraction until the grid has a few workgroups per compute unit.
     int split = 1;
-    while (gx * gy * split < 512 && g.KB / (split * 2) >= 8) split *= 2;
+    while (gx * gy * split < 256 && g.KB / (split * 2) >= 8) split *= 2;
     g.kb_per_split = (int)ceil_div(g.KB, split);
     g.atomic = split > 1;
     if (g.atomic) {
