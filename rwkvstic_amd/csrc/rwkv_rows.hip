@@ -150,17 +150,44 @@ struct QuantArgs {
     double *S, *qs, *zp;        // [R]
 };
 
+constexpr int kQuantSeg = 3;        // 16-element segments a thread keeps in registers (rows up to 48 * kRT = 12288 long in one read)
+
 __global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
     __shared__ double red[2 * kRW];
     __shared__ float redf[kRW];
     const int t = blockIdx.x, K = a.K;
     const double *row = a.in + (size_t)t * K;
+    // The thread that will write a 16-element group of digits reads it once: xs stays in registers
+    // between the pass that finds the row's scale and the pass that forms the digits (longer rows
+    // fall back to a second read).
+    float xs[kQuantSeg][16];
+    const bool fits = K <= kQuantSeg * 16 * kRT;
     float amax = 0.f;
     double z[1] = {0.0};
-    for (int c = threadIdx.x; c < K; c += kRT) {
-        const double v = row[c];
-        amax = fmaxf(amax, fabsf((float)(v * (double)a.range[c])));
-        z[0] += v * a.offset[c];
+    if (fits) {
+#pragma unroll
+        for (int s = 0; s < kQuantSeg; ++s) {
+            const int c0 = (threadIdx.x + s * kRT) * 16;
+            if (c0 < K) {
+#pragma unroll
+                for (int i = 0; i < 16; i += 2) {
+                    const double2 v = *reinterpret_cast<const double2 *>(row + c0 + i);
+                    const float2 r = *reinterpret_cast<const float2 *>(a.range + c0 + i);
+                    const double2 o = *reinterpret_cast<const double2 *>(a.offset + c0 + i);
+                    xs[s][i] = (float)(v.x * (double)r.x);
+                    xs[s][i + 1] = (float)(v.y * (double)r.y);
+                    amax = fmaxf(amax, fmaxf(fabsf(xs[s][i]), fabsf(xs[s][i + 1])));
+                    z[0] += v.x * o.x;
+                    z[0] += v.y * o.y;
+                }
+            }
+        }
+    } else {
+        for (int c = threadIdx.x; c < K; c += kRT) {
+            const double v = row[c];
+            amax = fmaxf(amax, fabsf((float)(v * (double)a.range[c])));
+            z[0] += v * a.offset[c];
+        }
     }
     amax = wmaxf(amax);
     if ((threadIdx.x & 63) == 0) redf[threadIdx.x >> 6] = amax;
@@ -178,7 +205,7 @@ __global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
     const int KB = K >> 6;
     const int mt = t >> 2, m0 = (t & 3) * 4;
     double qsum[1] = {0.0};
-    for (int c0 = threadIdx.x * 16; c0 < K; c0 += kRT * 16) {
+    auto emit = [&](int c0, const float (&x16)[16]) {
         unsigned pl[4][4];
 #pragma unroll
         for (int d = 0; d < 4; ++d)
@@ -186,8 +213,7 @@ __global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
             for (int j = 0; j < 4; ++j) pl[d][j] = 0u;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const float xs = (float)(row[c0 + i] * (double)a.range[c0 + i]);
-            int q = __double2int_rn((double)xs * invS);
+            int q = __double2int_rn((double)x16[i] * invS);
             qsum[0] += (double)q;
             const int d3 = (int)(signed char)(q & 0xff); q = (q - d3) >> 8;
             const int d2 = (int)(signed char)(q & 0xff); q = (q - d2) >> 8;
@@ -203,6 +229,20 @@ __global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
 #pragma unroll
         for (int d = 0; d < 4; ++d)
             *reinterpret_cast<uint4 *>(frag + (16 * g + m0 + d) * 16) = make_uint4(pl[d][0], pl[d][1], pl[d][2], pl[d][3]);
+    };
+    if (fits) {
+#pragma unroll
+        for (int s = 0; s < kQuantSeg; ++s) {
+            const int c0 = (threadIdx.x + s * kRT) * 16;
+            if (c0 < K) emit(c0, xs[s]);
+        }
+    } else {
+        for (int c0 = threadIdx.x * 16; c0 < K; c0 += kRT * 16) {
+            float x16[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) x16[i] = (float)(row[c0 + i] * (double)a.range[c0 + i]);
+            emit(c0, x16);
+        }
     }
     rsum<1>(qsum, red);
     if (threadIdx.x == 0) { a.S[t] = S; a.qs[t] = qsum[0]; a.zp[t] = z[0]; }
