@@ -269,6 +269,10 @@ struct GemmArgs {
     long long *tot;             // [4*MT][ldd]
     int MT, NT, KB, ldd, kb_per_split, atomic;
     int gx, gy, gz, rows_per_xcd;   // logical grid (column blocks, row blocks, splits) behind the 1-D launch
+    // when the contraction is not split the tail of the product is applied here (see rows_finish_kernel)
+    int tail, R, N;                 // tail < 0: totals only
+    const double *S, *qs, *zp, *gate;
+    double *out;
 };
 
 #ifndef RWKV_GEMM_GN
@@ -372,7 +376,20 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
             if (nt0 + j >= a.NT) continue;
             const v4i d = acc[i][j];
             const long long tot = ((((long long)d.x * 256 + d.y) * 256 + d.z) * 256) + d.w;
-            long long *p = a.tot + (size_t)(4 * (mt0 + i) + g) * a.ldd + 16 * (nt0 + j) + n;
+            const int t = 4 * (mt0 + i) + g, col = 16 * (nt0 + j) + n;
+            if (a.tail >= 0) {
+                if (t < a.R && col < a.N) {
+                    const double S = a.S[t];
+                    const double y = S * (double)tot + 128.0 * (S * a.qs[t]) + a.zp[t];
+                    double *o = a.out + (size_t)t * a.N + col;
+                    if (a.tail == ROW_STORE) *o = y;
+                    else if (a.tail == ROW_RELU2) { const double r = y > 0.0 ? y : 0.0; *o = r * r; }              // block.py:97
+                    else if (a.tail == ROW_ADD) *o += y;                                                            // block.py:80
+                    else *o += y * (1.0 / (1.0 + exp(-a.gate[(size_t)t * a.N + col])));                             // block.py:95-100
+                }
+                continue;
+            }
+            long long *p = a.tot + (size_t)t * a.ldd + col;
             if (a.atomic) atomicAdd(reinterpret_cast<unsigned long long *>(p), (unsigned long long)tot);
             else *p = tot;
         }
@@ -556,8 +573,11 @@ int rows_matmul(hipStream_t st, const RowsScratch &s, int64_t R, int64_t K, int6
         hipLaunchKernelGGL(rows_fill_kernel, dim3((unsigned)ceil_div((int64_t)n, 1024)), dim3(256), 0, st, s.tot, n);
     }
     g.gx = gx; g.gy = gy; g.gz = split; g.rows_per_xcd = (gy + kXcds - 1) / kXcds;
+    g.tail = g.atomic ? -1 : op; g.R = (int)R; g.N = (int)N; g.S = s.S; g.qs = s.qs; g.zp = s.zp; g.gate = gate; g.out = out;
+    if (op < ROW_STORE || op > ROW_GATE_ADD) return set_error(RWKV_ERR_ARG, "rows_matmul: unknown tail %d", op);
     hipLaunchKernelGGL(gemm8_kernel, dim3((unsigned)(kXcds * g.rows_per_xcd * gx * split)), dim3(256), 0, st, g);
     RWKV_CHECK_LAUNCH("gemm8_kernel");
+    if (!g.atomic) return RWKV_OK;      // the tail was applied in the product's epilogue
 
     FinishArgs f;
     f.R = (int)R; f.N = (int)N; f.ldd = g.ldd; f.tot = s.tot; f.S = s.S; f.qs = s.qs; f.zp = s.zp; f.out = out;
