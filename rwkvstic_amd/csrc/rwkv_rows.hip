@@ -260,7 +260,8 @@ __global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
 // to XCD r % 8), walking through the column blocks with the row blocks innermost: the digit
 // fragments of an XCD's rows (a few hundred KB) stay in its L2 for the whole product, and a weight
 // block fetched for one row block is reused by the next.  Without this every XCD pulls every digit
-// fragment through the fabric once per column block.
+// fragment through the fabric once per column block.  With fewer row blocks than XCDs (a batch of
+// single tokens) the column blocks are dealt out to the XCDs instead.
 // ---------------------------------------------------------------------------
 constexpr int kXcds = 8;
 struct GemmArgs {
@@ -268,7 +269,7 @@ struct GemmArgs {
     const uint8_t *w16;         // blocks [NT][KB][1024]
     long long *tot;             // [4*MT][ldd]
     int MT, NT, KB, ldd, kb_per_split, atomic;
-    int gx, gy, gz, rows_per_xcd;   // logical grid (column blocks, row blocks, splits) behind the 1-D launch
+    int gx, gy, gz, per_xcd, by_rows;   // logical grid (column blocks, row blocks, splits) behind the 1-D launch
     // when the contraction is not split the tail of the product is applied here (see rows_finish_kernel)
     int tail, R, N;                 // tail < 0: totals only
     const double *S, *qs, *zp, *gate;
@@ -298,11 +299,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave & 1, wn = wave >> 1;
     const int xcd = blockIdx.x % kXcds;
-    int item = blockIdx.x / kXcds;                      // (split, column block, row slot) of this XCD, row slot fastest
-    const int rslot = item % a.rows_per_xcd; item /= a.rows_per_xcd;
-    const int bx = item % a.gx, bz = item / a.gx;
-    const int by = xcd + kXcds * rslot;
-    if (by >= a.gy || bz >= a.gz) return;
+    int item = blockIdx.x / kXcds, bx, by, bz;
+    if (a.by_rows) {                                    // (split, column block, row slot) of this XCD, row slot fastest
+        const int rslot = item % a.per_xcd; item /= a.per_xcd;
+        bx = item % a.gx; bz = item / a.gx;
+        by = xcd + kXcds * rslot;
+    } else {                                            // few row blocks: the XCDs share out the column blocks instead
+        const int cslot = item % a.per_xcd; item /= a.per_xcd;
+        by = item % a.gy; bz = item / a.gy;
+        bx = xcd + kXcds * cslot;
+    }
+    if (by >= a.gy || bx >= a.gx || bz >= a.gz) return;
     const int mt0 = by * 16 + wm * kGM, nt0 = bx * kGemmNT + wn * kGN;
     const int kb0 = bz * a.kb_per_split;
     int kb1 = kb0 + a.kb_per_split;
@@ -572,10 +579,11 @@ int rows_matmul(hipStream_t st, const RowsScratch &s, int64_t R, int64_t K, int6
         const size_t n = (size_t)g.MT * 4 * g.ldd;
         hipLaunchKernelGGL(rows_fill_kernel, dim3((unsigned)ceil_div((int64_t)n, 1024)), dim3(256), 0, st, s.tot, n);
     }
-    g.gx = gx; g.gy = gy; g.gz = split; g.rows_per_xcd = (gy + kXcds - 1) / kXcds;
+    g.gx = gx; g.gy = gy; g.gz = split; g.by_rows = gy >= kXcds;
+    g.per_xcd = ((g.by_rows ? gy : gx) + kXcds - 1) / kXcds;
     g.tail = g.atomic ? -1 : op; g.R = (int)R; g.N = (int)N; g.S = s.S; g.qs = s.qs; g.zp = s.zp; g.gate = gate; g.out = out;
     if (op < ROW_STORE || op > ROW_GATE_ADD) return set_error(RWKV_ERR_ARG, "rows_matmul: unknown tail %d", op);
-    hipLaunchKernelGGL(gemm8_kernel, dim3((unsigned)(kXcds * g.rows_per_xcd * gx * split)), dim3(256), 0, st, g);
+    hipLaunchKernelGGL(gemm8_kernel, dim3((unsigned)(kXcds * g.per_xcd * (g.by_rows ? gx : gy) * split)), dim3(256), 0, st, g);
     RWKV_CHECK_LAUNCH("gemm8_kernel");
     if (!g.atomic) return RWKV_OK;      // the tail was applied in the product's epilogue
 
