@@ -25,7 +25,7 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E vendor peak
 # HBM bytes per launch of the single-token kernel from rocprofv3 counters (FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB,
 # both scaled by a 1 GiB device copy in the same run): a measured constant per shape, not something this script
 # can read live.  Shapes without a counter run report null.
-PMC_TRAFFIC_BYTES = {"3B": 2_963_700_000}
+PMC_TRAFFIC_BYTES = {"3B": 2_964_600_000}
 
 
 def cpu_baseline(shape, threads: int):
