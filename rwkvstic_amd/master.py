@@ -147,18 +147,21 @@ class RWKVMaster:
 
 def RWKV(path: Union[str, Dict[str, torch.Tensor]], mode: str = MODE, *, tokenizer=None, device: str = "cuda",
          sampler: Optional[Callable] = typical, **kwargs) -> RWKVMaster:
-    """``path``: a BlinkDL ``.pth`` checkpoint (loaded with ``weights_only=True``) or an already loaded state
-    dict.  Only the FASTQUANT mode exists in this backend (load.py:42-47); other modes raise."""
+    """``path``: a BlinkDL ``.pth`` checkpoint, a file written by ``HipRWKV.save_quantized`` (the quantised
+    attribute tree of the reference's .rwkv export, opt.py:89-92, as plain tensors; by convention ``.rwkvq``), both
+    loaded with ``weights_only=True``, or an already loaded dict of either kind.  TorchScript ``.rwkv`` archives
+    themselves are not read: loading one runs the code stored in it.  Only the FASTQUANT mode exists in this
+    backend (load.py:42-47); other modes raise."""
     if mode != MODE:
         raise ValueError(f"mode {mode!r} is not provided by this backend (only {MODE!r})")
     if kwargs:
         raise TypeError(f"unsupported options for mode {MODE!r}: {sorted(kwargs)}")
     from .model import HipRWKV
     if isinstance(path, str):
-        if not path.endswith(".pth"):
-            raise ValueError("only .pth checkpoints are supported")
+        if not (path.endswith(".pth") or path.endswith(".rwkvq")):
+            raise ValueError("only .pth checkpoints and .rwkvq quantised trees are supported")
         weights = torch.load(path, map_location="cpu", weights_only=True)
     else:
         weights = path
-    model = HipRWKV(weights, device=device)
+    model = HipRWKV.from_quantized(weights, device=device) if "emb.w" in weights else HipRWKV(weights, device=device)
     return RWKVMaster(model, model.emptyState.clone(), sampler, tokenizer)

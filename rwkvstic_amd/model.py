@@ -77,23 +77,15 @@ class HipRWKV:
         if self.emb is None:
             raise KeyError("emb.weight")
         # opt.py:96-98
-        self.dims = mats["blocks.0.att.key.weight"].n_out
-        self.layers = len([k for k in vec if "blocks" in k and "ln1.bias" in k])
-        self.ffn = mats["blocks.0.ffn.key.weight"].n_out
-        self.vocab = self.emb.shape[0]
-        Cn = self.dims
+        layers = len([k for k in vec if "blocks" in k and "ln1.bias" in k])
 
         def v64(key):
             return vec[key].reshape(-1).to(**f64).contiguous()
 
-        self._keep: List[torch.Tensor] = []
-        self.ln0 = (v64("blocks.0.ln0.weight"), v64("blocks.0.ln0.bias"))
-        self.ln_out = (v64("ln_out.weight"), v64("ln_out.bias"))
-        self.head = mats["head.weight"]
-        self.blocks: List[dict] = []
-        for i in range(self.layers):
+        blocks: List[dict] = []
+        for i in range(layers):
             p = f"blocks.{i}."
-            blk = dict(
+            blocks.append(dict(
                 ln1_w=v64(p + "ln1.weight"), ln1_b=v64(p + "ln1.bias"),
                 ln2_w=v64(p + "ln2.weight"), ln2_b=v64(p + "ln2.bias"),
                 # block.py:35-47
@@ -106,13 +98,100 @@ class HipRWKV:
                 att_r=mats[p + "att.receptance.weight"], att_o=mats[p + "att.output.weight"],
                 ffn_k=mats[p + "ffn.key.weight"], ffn_r=mats[p + "ffn.receptance.weight"],
                 ffn_v=mats[p + "ffn.value.weight"],
-            )
-            self.blocks.append(blk)
+            ))
+        self._finish_init((v64("blocks.0.ln0.weight"), v64("blocks.0.ln0.bias")),
+                          (v64("ln_out.weight"), v64("ln_out.bias")), mats["head.weight"], blocks)
+
+    def _finish_init(self, ln0, ln_out, head: QuantMatrix, blocks: List[dict]) -> None:
+        self.ln0, self.ln_out, self.head, self.blocks = ln0, ln_out, head, blocks
+        self.layers = len(blocks)
+        self.dims = blocks[0]["att_k"].n_out
+        self.ffn = blocks[0]["ffn_k"].n_out
+        self.vocab = self.emb.shape[0]
+        self._keep: List[torch.Tensor] = []
         # opt.py:31-32,80
-        es = torch.zeros((self.layers, 5, Cn), **f64)
+        es = torch.zeros((self.layers, 5, self.dims), device=self.device, dtype=torch.float64)
         es[:, 4] = -1e30
         self.emptyState = es
         self._build_handle()
+
+    # ------------------------------------------------------------------
+    # The quantised model as the reference keeps it (and exports it in a .rwkv archive, opt.py:89-92,112-117):
+    # a tree of module attributes.  Names: matmul.py:12,67-68,175,254 (weights.0.{weight,range,offset}[1,2]),
+    # block.py:13-47 (ln1, ln2, att, ffnkey, ffnvalue, attout, ffnreceptance, attmix, ffnmix, time_first,
+    # time_decay), opt.py:31-48 (emptyState, emb.w, ln_in, ln_out, head).  Codes are uint8 [in, out], range
+    # float32 [in], offset float64 [in]; time_decay is stored as -exp(raw) (block.py:41).
+    _MAT_ATTRS = (("att_k", "att.weights.0.", ""), ("att_v", "att.weights.0.", "1"), ("att_r", "att.weights.0.", "2"),
+                  ("att_o", "attout.weights.0.", ""), ("ffn_k", "ffnkey.weights.0.", ""),
+                  ("ffn_r", "ffnreceptance.weights.0.", ""), ("ffn_v", "ffnvalue.weights.0.", ""))
+
+    def quantized_tree(self) -> Dict[str, torch.Tensor]:
+        """Flat ``{attribute path: tensor}`` (on the CPU) of the quantised model under the reference's names."""
+        out: Dict[str, torch.Tensor] = {}
+
+        def put_mat(prefix: str, suffix: str, m: QuantMatrix) -> None:
+            out[f"{prefix}weight{suffix}"] = m.codes().cpu()
+            out[f"{prefix}range{suffix}"] = m.range.cpu()
+            out[f"{prefix}offset{suffix}"] = m.offset.cpu()
+
+        out["emptyState"] = self.emptyState.cpu()
+        out["emb.w"] = self.emb.cpu()
+        out["ln_in.weight"], out["ln_in.bias"] = self.ln0[0].cpu(), self.ln0[1].cpu()
+        out["ln_out.weight"], out["ln_out.bias"] = self.ln_out[0].cpu(), self.ln_out[1].cpu()
+        put_mat("head.weights.0.", "", self.head)
+        for i, b in enumerate(self.blocks):
+            p = f"blocks.{i}."
+            for name in ("ln1", "ln2"):
+                out[p + name + ".weight"], out[p + name + ".bias"] = b[name + "_w"].cpu(), b[name + "_b"].cpu()
+            for key, prefix, suffix in self._MAT_ATTRS:
+                put_mat(p + prefix, suffix, b[key])
+            out[p + "attmix"] = b["att_mix"].cpu().unsqueeze(1)        # [3, 1, C] (block.py:35-36)
+            out[p + "ffnmix"] = b["ffn_mix"].cpu().unsqueeze(1)        # [2, 1, C]
+            out[p + "time_first"] = b["time_first"].cpu()
+            out[p + "time_decay"] = b["time_decay"].cpu()
+        return out
+
+    @classmethod
+    def from_quantized(cls, tree: Dict[str, torch.Tensor], device: str = "cuda") -> "HipRWKV":
+        """From ``quantized_tree()`` (or the same attributes taken from a reference model): nothing is
+        quantised again, the codes are only repacked into the streaming layouts."""
+        if not torch.cuda.is_available():
+            raise RuntimeError("HipRWKV needs a ROCm GPU (gfx950); there is no CPU path in this backend")
+        N.lib()
+        self = cls.__new__(cls)
+        self.device = torch.device(device)
+        f64 = dict(device=self.device, dtype=torch.float64)
+
+        def v64(key):
+            return tree[key].reshape(-1).to(**f64).contiguous()
+
+        def mat(prefix: str, suffix: str = "") -> QuantMatrix:
+            codes = tree[f"{prefix}weight{suffix}"]
+            if codes.dtype != torch.uint8 or codes.dim() != 2:
+                raise ValueError(f"{prefix}weight{suffix}: expected uint8 codes [in, out]")
+            return QuantMatrix.from_codes(codes.contiguous(), tree[f"{prefix}range{suffix}"].reshape(-1),
+                                          tree[f"{prefix}offset{suffix}"].reshape(-1), self.device)
+
+        self.emb = tree["emb.w"].to(device=self.device, dtype=torch.float32).contiguous()
+        layers = len([k for k in tree if k.startswith("blocks.") and k.endswith(".ln1.bias")])
+        blocks: List[dict] = []
+        for i in range(layers):
+            p = f"blocks.{i}."
+            blk = dict(ln1_w=v64(p + "ln1.weight"), ln1_b=v64(p + "ln1.bias"),
+                       ln2_w=v64(p + "ln2.weight"), ln2_b=v64(p + "ln2.bias"),
+                       att_mix=tree[p + "attmix"].reshape(3, -1).to(**f64).contiguous(),
+                       ffn_mix=tree[p + "ffnmix"].reshape(2, -1).to(**f64).contiguous(),
+                       time_first=v64(p + "time_first"), time_decay=v64(p + "time_decay"))
+            for key, prefix, suffix in cls._MAT_ATTRS:
+                blk[key] = mat(p + prefix, suffix)
+            blocks.append(blk)
+        self._finish_init((v64("ln_in.weight"), v64("ln_in.bias")), (v64("ln_out.weight"), v64("ln_out.bias")),
+                          mat("head.weights.0."), blocks)
+        return self
+
+    def save_quantized(self, path: str) -> None:
+        """``torch.save`` of ``quantized_tree()``: plain tensors, loadable with ``weights_only=True``."""
+        torch.save(self.quantized_tree(), path)
 
     # ------------------------------------------------------------------
     def _build_handle(self) -> None:

@@ -274,3 +274,44 @@ def test_rwkv_shell_loads_checkpoint_file_and_generates(tmp_path, tiny):
     toks, _, s2 = hip.decode_greedy(prompt[-1], 6, s2)
     assert out["output"] == " ".join(str(int(t)) for t in toks)
     assert torch.equal(out["state"], s2)
+
+
+def test_quantized_tree_round_trip_and_oracle_layout(tmp_path, tiny):
+    """The quantised model under the reference's attribute names (what its .rwkv export holds, opt.py:89-92;
+    names from matmul.py:12,67-68, block.py:13-47, opt.py:31-48): the codes and ranges equal the CPU oracle's
+    quantiser output bit for bit (offsets to the last bits), and a model rebuilt from the tree (no second quantisation) gives identical results."""
+    from rwkvstic_amd.master import RWKV, greedy
+    from rwkvstic_amd.model import HipRWKV
+    ref, hip = tiny
+    sd = synth.make_state_dict(layers=3, C=64, V=512, seed=5)
+    tree = hip.quantized_tree()
+    assert tree["emptyState"].shape == (3, 5, 64) and tree["emb.w"].shape == (512, 64)
+    assert tree["blocks.0.attmix"].shape == (3, 1, 64) and tree["blocks.2.ffnmix"].shape == (2, 1, 64)
+    names = {"blocks.1.att.weights.0.": ("blocks.1.att.key.weight", "blocks.1.att.value.weight", "blocks.1.att.receptance.weight"),
+             "blocks.1.attout.weights.0.": ("blocks.1.att.output.weight",), "blocks.1.ffnkey.weights.0.": ("blocks.1.ffn.key.weight",),
+             "blocks.1.ffnvalue.weights.0.": ("blocks.1.ffn.value.weight",),
+             "blocks.1.ffnreceptance.weights.0.": ("blocks.1.ffn.receptance.weight",), "head.weights.0.": ("head.weight",)}
+    for prefix, keys in names.items():
+        for suffix, key in zip(("", "1", "2"), keys):
+            codes, rng, off = O.quantize_matrix(sd[key].float())
+            assert tree[prefix + "weight" + suffix].dtype == torch.uint8
+            assert torch.equal(tree[prefix + "weight" + suffix], codes), (prefix, suffix)       # [in, out]
+            assert torch.equal(tree[prefix + "range" + suffix], rng) and rng.dtype == torch.float32
+            # (the offset holds a mean of fractions: equal up to the order of that one sum)
+            assert torch.allclose(tree[prefix + "offset" + suffix], off, rtol=1e-13, atol=1e-300) and off.dtype == torch.float64
+    assert torch.equal(tree["blocks.1.time_decay"], sd["blocks.1.att.time_decay"].reshape(-1).double().exp().neg())
+    again = HipRWKV.from_quantized(tree)
+    toks = synth.random_tokens(7, V=512, seed=31).tolist()
+    l1, s1 = hip.forward(toks, hip.emptyState.clone())
+    l2, s2 = again.forward(toks, again.emptyState.clone())
+    assert torch.equal(l1, l2) and torch.equal(s1, s2)
+    # through a file and the loader shell
+    path = str(tmp_path / "tiny.rwkvq")
+    hip.save_quantized(path)
+    r = RWKV(path, sampler=greedy)
+    l3, s3 = r.model.forward(toks, r.emptyState.clone())
+    assert torch.equal(l1, l3) and torch.equal(s1, s3)
+    with pytest.raises(ValueError):
+        bad = dict(tree)
+        bad["head.weights.0.weight"] = bad["head.weights.0.weight"].float()
+        HipRWKV.from_quantized(bad)
