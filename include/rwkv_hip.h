@@ -197,10 +197,11 @@ typedef struct rwkv_model_desc {
 typedef struct rwkv_model rwkv_model;
 
 /* Copies the descriptor; the device buffers it names must outlive the handle.
- * This is the one entry point that allocates device memory (a table of the
- * layer pointers and three small exchange vectors for the single-token
- * kernel); rwkv_model_destroy frees it.  One forward call may be in flight
- * per handle at a time. */
+ * This is the one entry point that allocates device memory: one block with the
+ * tables of the single-token kernel (packed per-layer constants, column sums,
+ * 4 KiB of owner record and 128 bytes of job pointers per layer and
+ * 16-channel tile, the exchange vectors); rwkv_model_destroy frees it.  One
+ * forward call may be in flight per handle at a time. */
 int rwkv_model_create(const rwkv_model_desc *desc, rwkv_model **out);
 void rwkv_model_destroy(rwkv_model *m);
 
