@@ -251,9 +251,9 @@ __global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
 // ---------------------------------------------------------------------------
 // GEMM: tot[t, j] = sum_k q[t, k] * (code[k, j] - 128), exact in int64.
 // Workgroup = 4 wavefronts = 64 tokens x 128 columns; wavefront (wm, wn) holds
-// 8 M-tiles x 4 N-tiles of accumulators.  The contraction may be split over
-// several workgroups; partial totals are then added with integer atomics, which
-// commute exactly.
+// 8 M-tiles x 4 N-tiles of accumulators.  With few rows the contraction is split over
+// several workgroups; each split writes its own slice of integer totals and the tail
+// kernel adds the slices (integer sums: exact in any order).
 //
 // Launch order.  Workgroups are handed to the 8 XCDs round robin, and each XCD has its own L2.  The
 // grid is 1-D and workgroup i works for XCD i % 8 on that XCD's own row blocks (row block r belongs
@@ -268,7 +268,8 @@ struct GemmArgs {
     const signed char *dig;     // fragments [MT][KB][1024]
     const uint8_t *w16;         // blocks [NT][KB][1024]
     long long *tot;             // [4*MT][ldd]
-    int MT, NT, KB, ldd, kb_per_split, atomic;
+    int MT, NT, KB, ldd, kb_per_split, atomic;    // atomic: (historic name) the contraction is split: slice bz of tot
+    size_t slice;                   // elements between the slices of tot
     int gx, gy, gz, per_xcd, by_rows;   // logical grid (column blocks, row blocks, splits) behind the 1-D launch
     // when the contraction is not split the tail of the product is applied here (see rows_finish_kernel)
     int tail, R, N;                 // tail < 0: totals only
@@ -396,25 +397,18 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
                 }
                 continue;
             }
-            long long *p = a.tot + (size_t)t * a.ldd + col;
-            if (a.atomic) atomicAdd(reinterpret_cast<unsigned long long *>(p), (unsigned long long)tot);
-            else *p = tot;
+            a.tot[(size_t)bz * a.slice + (size_t)t * a.ldd + col] = tot;     // this split's slice
         }
     }
 }
 
-__global__ void __launch_bounds__(256) rows_fill_kernel(long long *p, size_t n) {
-    const size_t i0 = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-        if (i0 + i < n) p[i0 + i] = 0;
-}
 
 // ---------------------------------------------------------------------------
 // y[t, j] = S_t * tot + 128 * S_t * sum q_t + zp_t, then the phase's element-wise tail.
 // ---------------------------------------------------------------------------
 struct FinishArgs {
-    int R, N, ldd;
+    int R, N, ldd, slices;
+    size_t slice;
     const long long *tot;
     const double *S, *qs, *zp;
     double *out;                // [R, N]
@@ -427,7 +421,9 @@ __global__ void __launch_bounds__(256) rows_finish_kernel(const FinishArgs a) {
     const int j = blockIdx.x * 256 + threadIdx.x;
     if (j >= a.N) return;
     const double S = a.S[t];
-    const double y = S * (double)a.tot[(size_t)t * a.ldd + j] + 128.0 * (S * a.qs[t]) + a.zp[t];
+    long long tot = 0;                                   // integer partial sums of the contraction splits: exact in any order
+    for (int z = 0; z < a.slices; ++z) tot += a.tot[(size_t)z * a.slice + (size_t)t * a.ldd + j];
+    const double y = S * (double)tot + 128.0 * (S * a.qs[t]) + a.zp[t];
     double *o = a.out + (size_t)t * a.N + j;
     if (OP == ROW_STORE) *o = y;
     else if (OP == ROW_RELU2) { const double r = y > 0.0 ? y : 0.0; *o = r * r; }            // block.py:97
@@ -529,7 +525,18 @@ __global__ void __launch_bounds__(64) wkv_chunk_replay_kernel(const WkvRowsArgs 
 // ---------------------------------------------------------------------------
 size_t rows_dig_bytes(int64_t R, int64_t K) { return (size_t)(ceil_div(R, 4) * (K / 64) * 1024); }
 size_t rows_wkv_scratch_bytes(int64_t R, int64_t C) { return (size_t)(ceil_div(R, kWkvChunk) * 3 * C * 8); }
-size_t rows_tot_bytes(int64_t R, int64_t N) { return (size_t)(ceil_div(R, 4) * 4 * round_up(N, 16) * 8); }
+constexpr int kMaxSplit = 8;
+// Upper bound of the number of contraction splits rows_matmul will choose for R rows and N columns:
+// each split writes its own slice of totals (summed by the tail kernel), so the buffer has that many.
+static int gemm_split_bound(int64_t R, int64_t N) {
+    const int64_t gx = ceil_div(ceil_div(N, 16), kGemmNT), gy = ceil_div(ceil_div(R, 4), 16);
+    int s = 1;
+    while (gx * gy * s < 256 && s < kMaxSplit) s *= 2;
+    return s;
+}
+size_t rows_tot_bytes(int64_t R, int64_t N) {
+    return (size_t)(ceil_div(R, 4) * 4 * round_up(N, 16) * 8) * (size_t)gemm_split_bound(R, N);
+}
 
 int rows_embed(hipStream_t st, const int64_t *tokens, int64_t R, int V, int C, const float *emb, const double *w,
                const double *b, double *x) {
@@ -571,14 +578,10 @@ int rows_matmul(hipStream_t st, const RowsScratch &s, int64_t R, int64_t K, int6
     const int gx = (int)ceil_div(g.NT, kGemmNT), gy = (int)ceil_div(g.MT, 16);
     // Split the contraction until the grid has a few workgroups per compute unit.
     int split = 1;
-    while (gx * gy * split < 256 && g.KB / (split * 2) >= 8) split *= 2;
+    while (gx * gy * split < 256 && g.KB / (split * 2) >= 8 && split < kMaxSplit) split *= 2;
     g.kb_per_split = (int)ceil_div(g.KB, split);
     g.atomic = split > 1;
-    if (g.atomic) {
-        // (a fill kernel rather than a memset node, so the sequence can be captured in a graph)
-        const size_t n = (size_t)g.MT * 4 * g.ldd;
-        hipLaunchKernelGGL(rows_fill_kernel, dim3((unsigned)ceil_div((int64_t)n, 1024)), dim3(256), 0, st, s.tot, n);
-    }
+    g.slice = (size_t)g.MT * 4 * g.ldd;
     g.gx = gx; g.gy = gy; g.gz = split; g.by_rows = gy >= kXcds;
     g.per_xcd = ((g.by_rows ? gy : gx) + kXcds - 1) / kXcds;
     g.tail = g.atomic ? -1 : op; g.R = (int)R; g.N = (int)N; g.S = s.S; g.qs = s.qs; g.zp = s.zp; g.gate = gate; g.out = out;
@@ -588,7 +591,7 @@ int rows_matmul(hipStream_t st, const RowsScratch &s, int64_t R, int64_t K, int6
     if (!g.atomic) return RWKV_OK;      // the tail was applied in the product's epilogue
 
     FinishArgs f;
-    f.R = (int)R; f.N = (int)N; f.ldd = g.ldd; f.tot = s.tot; f.S = s.S; f.qs = s.qs; f.zp = s.zp; f.out = out;
+    f.R = (int)R; f.N = (int)N; f.ldd = g.ldd; f.slices = split; f.slice = g.slice; f.tot = s.tot; f.S = s.S; f.qs = s.qs; f.zp = s.zp; f.out = out;
     f.gate = gate;
     const dim3 fg((unsigned)ceil_div(N, 256), (unsigned)R), fb(256);
     switch (op) {
