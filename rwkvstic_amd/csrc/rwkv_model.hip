@@ -489,20 +489,26 @@ constexpr int64_t kRowsChunk = 1024;   // rows per pass: bounds the workspace of
 constexpr int64_t kRowsMin = 4;        // shorter prompts go token by token
 
 struct RowsWs {
-    double *x, *mix, *kvr, *att, *h, *prev0, *wkv_scr;
-    RowsScratch s;
+    double *x, *kvr, *att, *h, *prev0, *wkv_scr;
+    RowsOperand q[3];       // quantised left operands: q[0] up to n_ffn wide, q[1], q[2] n_embd wide
+    long long *tot;
 };
+
+size_t rows_tot_ws_bytes(int64_t R, int64_t C, int64_t n_wide) {
+    const size_t a = rows_tot_bytes(R, n_wide), b = 3 * rows_tot_bytes(R, C);     // k, v, r share a launch
+    return a > b ? a : b;
+}
 
 // n_wide = widest product output (n_ffn, or the vocabulary when every row needs logits)
 size_t rows_ws_bytes(int64_t R, int64_t C, int64_t F, int64_t n_wide) {
     size_t n = 0;
-    n += round_up((size_t)R * C * 8, 256) * 8;          // x, mix[3], kvr[3], att
+    n += round_up((size_t)R * C * 8, 256) * 5;          // x, kvr[3], att
     n += round_up((size_t)R * F * 8, 256);              // h
     n += round_up((size_t)C * 8, 256);                  // prev0
     n += round_up(rows_wkv_scratch_bytes(R, C), 256);
-    n += round_up((size_t)R * 8, 256) * 3;              // S, qs, zp
-    n += round_up(rows_dig_bytes(R, F), 256);
-    n += round_up(rows_tot_bytes(R, n_wide), 256);
+    n += round_up((size_t)R * 8, 256) * 9;              // S, qs, zp of three operands
+    n += round_up(rows_dig_bytes(R, F), 256) + 2 * round_up(rows_dig_bytes(R, C), 256);
+    n += round_up(rows_tot_ws_bytes(R, C, n_wide), 256);
     return n;
 }
 
@@ -511,24 +517,24 @@ RowsWs rows_carve(void *ws, int64_t R, int64_t C, int64_t F, int64_t n_wide) {
     auto take = [&](size_t bytes) { void *q = p; p += round_up(bytes, 256); return q; };
     RowsWs w;
     w.x = (double *)take((size_t)R * C * 8);
-    w.mix = (double *)take((size_t)R * C * 8 * 3);
     w.kvr = (double *)take((size_t)R * C * 8 * 3);
     w.att = (double *)take((size_t)R * C * 8);
     w.h = (double *)take((size_t)R * F * 8);
     w.prev0 = (double *)take((size_t)C * 8);
     w.wkv_scr = (double *)take(rows_wkv_scratch_bytes(R, C));
-    w.s.S = (double *)take((size_t)R * 8);
-    w.s.qs = (double *)take((size_t)R * 8);
-    w.s.zp = (double *)take((size_t)R * 8);
-    w.s.dig = (signed char *)take(rows_dig_bytes(R, F));
-    w.s.tot = (long long *)take(rows_tot_bytes(R, n_wide));
-    (void)n_wide;
+    for (int i = 0; i < 3; ++i) {
+        w.q[i].S = (double *)take((size_t)R * 8);
+        w.q[i].qs = (double *)take((size_t)R * 8);
+        w.q[i].zp = (double *)take((size_t)R * 8);
+        w.q[i].dig = (signed char *)take(rows_dig_bytes(R, i == 0 ? F : C));
+    }
+    w.tot = (long long *)take(rows_tot_ws_bytes(R, C, n_wide));
     return w;
 }
 
 bool rows_supported(const rwkv_model *m) {
     const rwkv_model_desc &d = m->d;
-    if (d.n_embd % 64 || d.n_ffn % 64 || !d.head.packed16) return false;
+    if (d.n_embd % 64 || d.n_ffn % 64 || !d.head.packed16 || !rows_ln_width_supported(d.n_embd)) return false;
     for (const rwkv_layer_desc &ld : m->layers)
         if (!(ld.att_k.packed16 && ld.att_v.packed16 && ld.att_r.packed16 && ld.att_o.packed16 &&
               ld.ffn_k.packed16 && ld.ffn_r.packed16 && ld.ffn_v.packed16))
@@ -551,26 +557,31 @@ int rows_layers(rwkv_model *m, hipStream_t st, const int64_t *tokens, int64_t R,
         double *sl = state + (size_t)l * 5 * C;
         // TimeMix (block.py:58-80)
         if (sequence) RWKV_CHECK_HIP(hipMemcpyAsync(w.prev0, sl, (size_t)C * 8, hipMemcpyDeviceToDevice, st));
-        RWKV_TRY(rows_ln_mix(st, 3, R, C, sequence, w.x, L.ln1_w, L.ln1_b, L.att_mix, sequence ? w.prev0 : sl, sl,
-                             state_stride, w.mix));
         const rwkv_qmat *kvr[3] = {&L.att_k, &L.att_v, &L.att_r};
-        for (int i = 0; i < 3; ++i)
-            RWKV_TRY(rows_matmul(st, w.s, R, C, C, w.mix + i * RC, kvr[i]->packed16, kvr[i]->range, kvr[i]->offset,
-                                 ROW_STORE, w.kvr + i * RC, nullptr));
+        const float *rg[3] = {kvr[0]->range, kvr[1]->range, kvr[2]->range};
+        const double *of[3] = {kvr[0]->offset, kvr[1]->offset, kvr[2]->offset};
+        RWKV_TRY(rows_ln_mix_quant(st, 3, R, C, sequence, w.x, L.ln1_w, L.ln1_b, L.att_mix, sequence ? w.prev0 : sl, sl,
+                                   state_stride, rg, of, w.q));
+        RowsProduct pk[3];
+        for (int i = 0; i < 3; ++i) { pk[i].a = w.q[i]; pk[i].w16 = kvr[i]->packed16; pk[i].out = w.kvr + i * RC; }
+        RWKV_TRY(rows_products(st, 3, pk, w.tot, R, C, C, ROW_STORE, nullptr));
         RWKV_TRY(rows_wkv(st, R, C, sequence, w.kvr, w.kvr + RC, w.kvr + 2 * RC, L.time_decay, L.time_first,
                           sl + 2 * (size_t)C, state_stride, w.att, w.wkv_scr));
-        RWKV_TRY(rows_matmul(st, w.s, R, C, C, w.att, L.att_o.packed16, L.att_o.range, L.att_o.offset, ROW_ADD, w.x,
-                             nullptr));
+        RWKV_TRY(rows_quant(st, R, C, w.att, L.att_o.range, L.att_o.offset, w.q[0]));
+        const RowsProduct po = {w.q[0], L.att_o.packed16, w.x};
+        RWKV_TRY(rows_products(st, 1, &po, w.tot, R, C, C, ROW_ADD, nullptr));
         // ChannelMix (block.py:82-100)
         if (sequence) RWKV_CHECK_HIP(hipMemcpyAsync(w.prev0, sl + C, (size_t)C * 8, hipMemcpyDeviceToDevice, st));
-        RWKV_TRY(rows_ln_mix(st, 2, R, C, sequence, w.x, L.ln2_w, L.ln2_b, L.ffn_mix, sequence ? w.prev0 : sl + C,
-                             sl + C, state_stride, w.mix));
-        RWKV_TRY(rows_matmul(st, w.s, R, C, F, w.mix, L.ffn_k.packed16, L.ffn_k.range, L.ffn_k.offset, ROW_RELU2, w.h,
-                             nullptr));
-        RWKV_TRY(rows_matmul(st, w.s, R, C, C, w.mix + RC, L.ffn_r.packed16, L.ffn_r.range, L.ffn_r.offset, ROW_STORE,
-                             w.kvr, nullptr));
-        RWKV_TRY(rows_matmul(st, w.s, R, F, C, w.h, L.ffn_v.packed16, L.ffn_v.range, L.ffn_v.offset, ROW_GATE_ADD, w.x,
-                             w.kvr));
+        const float *rg2[2] = {L.ffn_k.range, L.ffn_r.range};
+        const double *of2[2] = {L.ffn_k.offset, L.ffn_r.offset};
+        RWKV_TRY(rows_ln_mix_quant(st, 2, R, C, sequence, w.x, L.ln2_w, L.ln2_b, L.ffn_mix, sequence ? w.prev0 : sl + C,
+                                   sl + C, state_stride, rg2, of2, w.q + 1));
+        const RowsProduct pfk = {w.q[1], L.ffn_k.packed16, w.h}, pfr = {w.q[2], L.ffn_r.packed16, w.kvr};
+        RWKV_TRY(rows_products(st, 1, &pfk, w.tot, R, C, F, ROW_RELU2, nullptr));
+        RWKV_TRY(rows_products(st, 1, &pfr, w.tot, R, C, C, ROW_STORE, nullptr));
+        RWKV_TRY(rows_quant(st, R, F, w.h, L.ffn_v.range, L.ffn_v.offset, w.q[0]));
+        const RowsProduct pfv = {w.q[0], L.ffn_v.packed16, w.x};
+        RWKV_TRY(rows_products(st, 1, &pfv, w.tot, R, F, C, ROW_GATE_ADD, w.kvr));
     }
     return RWKV_OK;
 }
@@ -737,10 +748,13 @@ int rwkv_model_forward_batch(rwkv_model *m, rwkv_stream_t stream, const int64_t 
     const RowsWs rw = rows_carve(workspace, batch, C, F, F > V ? F : V);
     int rc = rows_layers(m, st, tokens, batch, false, states, d.n_layer * 5 * C, rw);
     if (rc) return rc;
-    rc = rows_ln_mix(st, 0, batch, (int)C, false, rw.x, d.ln_out_w, d.ln_out_b, nullptr, nullptr, nullptr, 0, rw.mix);
+    const float *rg[1] = {d.head.range};
+    const double *of[1] = {d.head.offset};
+    rc = rows_ln_mix_quant(st, 0, batch, (int)C, false, rw.x, d.ln_out_w, d.ln_out_b, nullptr, nullptr, nullptr, 0, rg, of,
+                           rw.q);
     if (rc) return rc;
-    return rows_matmul(st, rw.s, batch, C, V, rw.mix, d.head.packed16, d.head.range, d.head.offset, ROW_STORE, logits,
-                       nullptr);
+    const RowsProduct ph = {rw.q[0], d.head.packed16, logits};
+    return rows_products(st, 1, &ph, rw.tot, batch, C, V, ROW_STORE, nullptr);
 }
 
 int rwkv_gemm8(rwkv_stream_t stream, int64_t T, int64_t n_in, int64_t n_out, const double *x,
@@ -758,13 +772,16 @@ int rwkv_gemm8(rwkv_stream_t stream, int64_t T, int64_t n_in, int64_t n_out, con
         return set_error(RWKV_ERR_WORKSPACE, "rwkv_gemm8: workspace of %zu bytes needed, %zu given", need,
                          workspace_bytes);
     unsigned char *p = static_cast<unsigned char *>(workspace);
-    RowsScratch s;
-    s.S = (double *)p; p += round_up((size_t)T * 8, 256);
-    s.qs = (double *)p; p += round_up((size_t)T * 8, 256);
-    s.zp = (double *)p; p += round_up((size_t)T * 8, 256);
-    s.dig = (signed char *)p; p += round_up(rows_dig_bytes(T, n_in), 256);
-    s.tot = (long long *)p;
-    return rows_matmul((hipStream_t)stream, s, T, n_in, n_out, x, packed16, range, offset, ROW_STORE, y, nullptr);
+    RowsOperand q;
+    q.S = (double *)p; p += round_up((size_t)T * 8, 256);
+    q.qs = (double *)p; p += round_up((size_t)T * 8, 256);
+    q.zp = (double *)p; p += round_up((size_t)T * 8, 256);
+    q.dig = (signed char *)p; p += round_up(rows_dig_bytes(T, n_in), 256);
+    const hipStream_t st = (hipStream_t)stream;
+    const int rc = rows_quant(st, T, n_in, x, range, offset, q);
+    if (rc) return rc;
+    const RowsProduct pr = {q, packed16, y};
+    return rows_products(st, 1, &pr, (long long *)p, T, n_in, n_out, ROW_STORE, nullptr);
 }
 
 size_t rwkv_gemm8_workspace_bytes(int64_t T, int64_t n_in, int64_t n_out) {

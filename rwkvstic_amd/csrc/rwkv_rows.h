@@ -7,27 +7,39 @@ namespace rwkv {
 
 enum RowTail { ROW_STORE = 0, ROW_RELU2 = 1, ROW_ADD = 2, ROW_GATE_ADD = 3 };
 
-// Device scratch one rows_matmul call needs for R rows (sizes from the helpers below,
-// taken at the largest contraction length K and output width N that will be used).
-struct RowsScratch {
+// One quantised left operand of a product: R rows rewritten as fixed-point digit fragments plus the
+// per-row constants of the tail (scale, sum of the fixed-point values, zero-point sum).
+struct RowsOperand {
     signed char *dig;       // rows_dig_bytes(R, K)
-    long long *tot;         // rows_tot_bytes(R, N)
     double *S, *qs, *zp;    // [R] each
 };
+struct RowsProduct {        // out[R, N] (tail op) a x quantised matrix in M16 blocks
+    RowsOperand a;
+    const uint8_t *w16;
+    double *out;
+};
+constexpr int kRowsMaxProducts = 3;     // products of equal shape and tail that share one launch
 size_t rows_dig_bytes(int64_t R, int64_t K);
-size_t rows_tot_bytes(int64_t R, int64_t N);
+size_t rows_tot_bytes(int64_t R, int64_t N);        // integer totals of ONE product (times the products in a launch)
 size_t rows_wkv_scratch_bytes(int64_t R, int64_t C);
+bool rows_ln_width_supported(int64_t C);            // widths the fused LayerNorm + mix + quantise kernel holds in registers
 
 int rows_embed(hipStream_t st, const int64_t *tokens, int64_t R, int V, int C, const float *emb, const double *w,
                const double *b, double *x);
-// n_mix in {0, 2, 3}; see LnMixArgs in rwkv_rows.hip for the meaning of prev0 / shift_dst / prev_stride.
-int rows_ln_mix(hipStream_t st, int n_mix, int64_t R, int C, bool sequence, const double *x, const double *ln_w,
-                const double *ln_b, const double *mu, const double *prev0, double *shift_dst, int64_t prev_stride,
-                double *mix);
-// out[R, N] (tail op) in[R, K] x quantised matrix (M16 blocks, per-input-channel range / offset).
-int rows_matmul(hipStream_t st, const RowsScratch &s, int64_t R, int64_t K, int64_t N, const double *in,
-                const uint8_t *w16, const float *range, const double *offset, int op, double *out,
-                const double *gate);
+// LayerNorm + token shift + time mix of R rows, each mixed row quantised for its matrix (range / offset per
+// input channel): n_mix in {0, 2, 3}; 0 = LayerNorm only, one output.  See LnQuantArgs in rwkv_rows.hip for
+// the meaning of prev0 / shift_dst / prev_stride.
+int rows_ln_mix_quant(hipStream_t st, int n_mix, int64_t R, int C, bool sequence, const double *x, const double *ln_w,
+                      const double *ln_b, const double *mu, const double *prev0, double *shift_dst,
+                      int64_t prev_stride, const float *const *range, const double *const *offset,
+                      const RowsOperand *out);
+// Rows of float64 values quantised for a matrix with the given per-input-channel range / offset.
+int rows_quant(hipStream_t st, int64_t R, int64_t K, const double *in, const float *range, const double *offset,
+               const RowsOperand &out);
+// n (<= kRowsMaxProducts) products of the same shape [R, K] x [K, N] and tail in one launch;
+// tot: n * rows_tot_bytes(R, N) bytes of scratch.
+int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, int64_t R, int64_t K, int64_t N, int op,
+                  const double *gate);
 int rows_wkv(hipStream_t st, int64_t R, int C, bool sequence, const double *k, const double *v, const double *r,
              const double *w, const double *u, double *state, int64_t state_stride, double *out,
              double *scratch /* rows_wkv_scratch_bytes(R, C), or null: serial over the rows */);

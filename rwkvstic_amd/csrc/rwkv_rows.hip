@@ -85,12 +85,55 @@ rows_embed_kernel(const int64_t *__restrict__ tokens, int V, int C, const float 
 }
 
 // ---------------------------------------------------------------------------
-// LayerNorm + token shift + time mix      (layernorm.py:15-20, block.py:58-67,82-91)
-//   xy = ln(x[t]);  prev = sequence ? (t == 0 ? prev0 : ln(x[t-1])) : prev0[t];
-//   mix_m[t] = xy * mu_m + prev * (1 - mu_m);  the newest xy becomes the shift state.
-// NM == 0: LayerNorm only, written to mix_0 (the head's ln_out).
+// Fixed-point digits of four consecutive values of a row (columns c0..c0+3 of token t), written into
+// the row's fragments; returns the sum of the four fixed-point values.
 // ---------------------------------------------------------------------------
-struct LnMixArgs {
+__device__ __forceinline__ double emit_quad(const float (&x4)[4], double invS, int c0, int t, int KB,
+                                            signed char *dig) {
+    unsigned pl[4] = {0u, 0u, 0u, 0u};
+    double qsum = 0.0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int q = __double2int_rn((double)x4[i] * invS);
+        qsum += (double)q;
+        const int d3 = (int)(signed char)(q & 0xff); q = (q - d3) >> 8;
+        const int d2 = (int)(signed char)(q & 0xff); q = (q - d2) >> 8;
+        const int d1 = (int)(signed char)(q & 0xff); q = (q - d1) >> 8;
+        const int sh = 8 * i;
+        pl[0] |= (unsigned)(q & 0xff) << sh;
+        pl[1] |= (unsigned)(d1 & 0xff) << sh;
+        pl[2] |= (unsigned)(d2 & 0xff) << sh;
+        pl[3] |= (unsigned)(d3 & 0xff) << sh;
+    }
+    const int mt = t >> 2, m0 = (t & 3) * 4;
+    const int kb = c0 >> 6, g = (c0 & 63) >> 4, j = (c0 & 15) >> 2;
+    signed char *frag = dig + ((size_t)mt * KB + kb) * 1024 + (16 * g + m0) * 16 + 4 * j;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) *reinterpret_cast<unsigned *>(frag + d * 16) = pl[d];
+    return qsum;
+}
+
+// Power-of-two scale of a row whose largest |xs| is amax: |xs / S| <= 2^30.
+__device__ __forceinline__ void row_scale(float amax, double &S, double &invS) {
+    S = 0.0; invS = 0.0;
+    if (amax > 0.f && amax < INFINITY) {
+        int e;
+        frexpf(amax, &e);                  // amax = f * 2^e, f in [0.5, 1)  =>  |xs| < 2^e
+        S = ldexp(1.0, e - 30);
+        invS = ldexp(1.0, 30 - e);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// LayerNorm + token shift + time mix + row quantiser      (layernorm.py:15-20, block.py:58-67,82-91,
+// matmul.py:59-62,131-133)
+//   xy = ln(x[t]);  prev = sequence ? (t == 0 ? prev0 : ln(x[t-1])) : prev0[t];
+//   mix_m[t] = xy * mu_m + prev * (1 - mu_m), quantised for matrix m; the newest xy becomes the shift state.
+// NM == 0: LayerNorm only, one output (the head's ln_out).
+// One workgroup per row; a thread keeps its NSEG groups of four channels in registers from the one
+// read of x to the digits, so the mixed rows never travel through memory.
+// ---------------------------------------------------------------------------
+struct LnQuantArgs {
     int C, R, sequence;
     const double *x;            // [R, C]
     const double *ln_w, *ln_b;  // [C]
@@ -98,42 +141,128 @@ struct LnMixArgs {
     const double *prev0;        // sequence: [C]; batch: row t at prev0 + t * prev_stride
     double *shift_dst;          // sequence: [C] (written by row R-1); batch: row t at shift_dst + t * prev_stride
     int64_t prev_stride;
-    double *mix;                // [max(NM,1), R, C]
+    const float *range[3];      // per output: the matrix's per-input-channel range / offset
+    const double *offset[3];
+    signed char *dig[3];        // per output: fragments [ceil(R/4)][C/64][1024] and the row constants
+    double *S[3], *qs[3], *zp[3];
 };
 
-template <int NM>
-__global__ void __launch_bounds__(kRT) rows_ln_mix_kernel(const LnMixArgs a) {
+template <int NM, int NSEG>
+__global__ void __launch_bounds__(kRT) rows_ln_mix_quant_kernel(const LnQuantArgs a) {
+    constexpr int NO = NM > 0 ? NM : 1;
     __shared__ double red[4 * kRW];
-    const int t = blockIdx.x, C = a.C;
+    __shared__ float redf[NO * kRW];
+    const int t = blockIdx.x, C = a.C, nq = C >> 2, tid = threadIdx.x;
     const bool need_prev = NM > 0 && a.sequence && t > 0;
     const double *xr = a.x + (size_t)t * C;
-    const double *xp = need_prev ? xr - C : xr;
+    const double *pr = NM == 0 ? xr : need_prev ? xr - C : a.sequence ? a.prev0 : a.prev0 + (size_t)t * a.prev_stride;
+    double xv[NSEG][4], pv[NSEG][4];
     double s[2] = {0.0, 0.0};
-    for (int c = threadIdx.x; c < C; c += kRT) { s[0] += xr[c]; s[1] += xp[c]; }
+#pragma unroll
+    for (int g = 0; g < NSEG; ++g) {
+        const int c0 = 4 * (tid + g * kRT);
+        if (c0 < C) {
+            const double2 x0 = *reinterpret_cast<const double2 *>(xr + c0), x1 = *reinterpret_cast<const double2 *>(xr + c0 + 2);
+            xv[g][0] = x0.x; xv[g][1] = x0.y; xv[g][2] = x1.x; xv[g][3] = x1.y;
+            if (NM > 0) {
+                const double2 p0 = *reinterpret_cast<const double2 *>(pr + c0), p1 = *reinterpret_cast<const double2 *>(pr + c0 + 2);
+                pv[g][0] = p0.x; pv[g][1] = p0.y; pv[g][2] = p1.x; pv[g][3] = p1.y;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { s[0] += xv[g][i]; if (NM > 0) s[1] += pv[g][i]; }
+        }
+    }
     rsum<2>(s, red);
     const double mean = s[0] / (double)C, meanp = s[1] / (double)C;
     double q[2] = {0.0, 0.0};
-    for (int c = threadIdx.x; c < C; c += kRT) {
-        const double d = xr[c] - mean, dp = xp[c] - meanp;
-        q[0] += d * d; q[1] += dp * dp;
+#pragma unroll
+    for (int g = 0; g < NSEG; ++g) {
+        if (4 * (tid + g * kRT) < C) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const double d = xv[g][i] - mean;
+                q[0] += d * d;
+                if (NM > 0) { const double dp = pv[g][i] - meanp; q[1] += dp * dp; }
+            }
+        }
     }
     rsum<2>(q, red);
     const double sd = sqrt(q[0] / (double)C + 1e-5), sdp = sqrt(q[1] / (double)C + 1e-5);
-    const size_t RC = (size_t)a.R * C;
-    for (int c = threadIdx.x; c < C; c += kRT) {
-        const double w = a.ln_w[c], b = a.ln_b[c];
-        const double xy = w * ((xr[c] - mean) / sd) + b;
-        if (NM == 0) { a.mix[(size_t)t * C + c] = xy; continue; }
-        double prev;
-        if (need_prev) prev = w * ((xp[c] - meanp) / sdp) + b;
-        else prev = a.sequence ? a.prev0[c] : a.prev0[(size_t)t * a.prev_stride + c];
+    float xs[NO][NSEG][4];
+    float amax[NO];
+    double z[NO];
 #pragma unroll
-        for (int m = 0; m < NM; ++m) {
-            const double mu = a.mu[(size_t)m * C + c];
-            a.mix[m * RC + (size_t)t * C + c] = xy * mu + prev * (1.0 - mu);
+    for (int m = 0; m < NO; ++m) { amax[m] = 0.f; z[m] = 0.0; }
+#pragma unroll
+    for (int g = 0; g < NSEG; ++g) {
+        const int c0 = 4 * (tid + g * kRT);
+        if (c0 < C) {
+            double xy[4], prev[4];
+#pragma unroll
+            for (int i = 0; i < 4; i += 2) {
+                const double2 w = *reinterpret_cast<const double2 *>(a.ln_w + c0 + i);
+                const double2 b = *reinterpret_cast<const double2 *>(a.ln_b + c0 + i);
+                xy[i] = w.x * ((xv[g][i] - mean) / sd) + b.x;
+                xy[i + 1] = w.y * ((xv[g][i + 1] - mean) / sd) + b.y;
+                if (NM > 0) {
+                    prev[i] = need_prev ? w.x * ((pv[g][i] - meanp) / sdp) + b.x : pv[g][i];
+                    prev[i + 1] = need_prev ? w.y * ((pv[g][i + 1] - meanp) / sdp) + b.y : pv[g][i + 1];
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < NO; ++m) {
+                const float4 r = *reinterpret_cast<const float4 *>(a.range[m] + c0);
+                const float rr[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+                for (int i = 0; i < 4; i += 2) {
+                    const double2 o = *reinterpret_cast<const double2 *>(a.offset[m] + c0 + i);
+                    double v0 = xy[i], v1 = xy[i + 1];
+                    if (NM > 0) {
+                        const double2 mu = *reinterpret_cast<const double2 *>(a.mu + (size_t)m * C + c0 + i);
+                        v0 = xy[i] * mu.x + prev[i] * (1.0 - mu.x);
+                        v1 = xy[i + 1] * mu.y + prev[i + 1] * (1.0 - mu.y);
+                    }
+                    xs[m][g][i] = (float)(v0 * (double)rr[i]);
+                    xs[m][g][i + 1] = (float)(v1 * (double)rr[i + 1]);
+                    amax[m] = fmaxf(amax[m], fmaxf(fabsf(xs[m][g][i]), fabsf(xs[m][g][i + 1])));
+                    z[m] += v0 * o.x;
+                    z[m] += v1 * o.y;
+                }
+            }
+            if (NM > 0) {
+                double *sh = !a.sequence ? a.shift_dst + (size_t)t * a.prev_stride : t == a.R - 1 ? a.shift_dst : nullptr;
+                if (sh) {
+                    *reinterpret_cast<double2 *>(sh + c0) = make_double2(xy[0], xy[1]);
+                    *reinterpret_cast<double2 *>(sh + c0 + 2) = make_double2(xy[2], xy[3]);
+                }
+            }
         }
-        if (!a.sequence) a.shift_dst[(size_t)t * a.prev_stride + c] = xy;
-        else if (t == a.R - 1) a.shift_dst[c] = xy;
+    }
+#pragma unroll
+    for (int m = 0; m < NO; ++m) {
+        amax[m] = wmaxf(amax[m]);
+        if ((tid & 63) == 0) redf[m * kRW + (tid >> 6)] = amax[m];
+    }
+    rsum<NO>(z, red);                      // (its barriers also publish redf)
+    double S[NO], invS[NO], qsum[NO];
+    const int KB = C >> 6;
+#pragma unroll
+    for (int m = 0; m < NO; ++m) {
+        float am = redf[m * kRW];
+#pragma unroll
+        for (int w = 1; w < kRW; ++w) am = fmaxf(am, redf[m * kRW + w]);
+        row_scale(am, S[m], invS[m]);
+        qsum[m] = 0.0;
+#pragma unroll
+        for (int g = 0; g < NSEG; ++g) {
+            const int c0 = 4 * (tid + g * kRT);
+            if (c0 < C) qsum[m] += emit_quad(xs[m][g], invS[m], c0, t, KB, a.dig[m]);
+        }
+    }
+    rsum<NO>(qsum, red);
+    if (tid == 0) {
+#pragma unroll
+        for (int m = 0; m < NO; ++m) { a.S[m][t] = S[m]; a.qs[m][t] = qsum[m]; a.zp[m][t] = z[m]; }
     }
 }
 
@@ -150,7 +279,7 @@ struct QuantArgs {
     double *S, *qs, *zp;        // [R]
 };
 
-constexpr int kQuantSeg = 3;        // 16-element segments a thread keeps in registers (rows up to 48 * kRT = 12288 long in one read)
+constexpr int kQuantSeg = 5;        // 16-element segments a thread keeps in registers (rows up to 80 * kRT = 20480 long in one read)
 
 __global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
     __shared__ double red[2 * kRW];
@@ -195,13 +324,8 @@ __global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
     amax = redf[0];
 #pragma unroll
     for (int w = 1; w < kRW; ++w) amax = fmaxf(amax, redf[w]);
-    double S = 0.0, invS = 0.0;
-    if (amax > 0.f && amax < INFINITY) {
-        int e;
-        frexpf(amax, &e);                  // amax = f * 2^e, f in [0.5, 1)  =>  |xs| < 2^e
-        S = ldexp(1.0, e - 30);
-        invS = ldexp(1.0, 30 - e);
-    }
+    double S, invS;
+    row_scale(amax, S, invS);
     const int KB = K >> 6;
     const int mt = t >> 2, m0 = (t & 3) * 4;
     double qsum[1] = {0.0};
@@ -265,16 +389,18 @@ __global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
 // ---------------------------------------------------------------------------
 constexpr int kXcds = 8;
 struct GemmArgs {
-    const signed char *dig;     // fragments [MT][KB][1024]
-    const uint8_t *w16;         // blocks [NT][KB][1024]
-    long long *tot;             // [4*MT][ldd]
-    int MT, NT, KB, ldd, kb_per_split, atomic;    // atomic: (historic name) the contraction is split: slice bz of tot
+    // up to kRowsMaxProducts products of one shape share a launch (the grid's split index also counts products)
+    const signed char *dig[kRowsMaxProducts];   // fragments [MT][KB][1024]
+    const uint8_t *w16[kRowsMaxProducts];       // blocks [NT][KB][1024]
+    const double *S[kRowsMaxProducts], *qs[kRowsMaxProducts], *zp[kRowsMaxProducts];
+    double *out[kRowsMaxProducts];
+    long long *tot;             // [products][splits][4*MT][ldd]
+    int MT, NT, KB, ldd, kb_per_split, split;     // split > 1: the contraction is split, each part writes its slice of tot
     size_t slice;                   // elements between the slices of tot
-    int gx, gy, gz, per_xcd, by_rows;   // logical grid (column blocks, row blocks, splits) behind the 1-D launch
+    int gx, gy, gz, per_xcd, by_rows;   // logical grid (column blocks, row blocks, splits x products) behind the 1-D launch
     // when the contraction is not split the tail of the product is applied here (see rows_finish_kernel)
     int tail, R, N;                 // tail < 0: totals only
-    const double *S, *qs, *zp, *gate;
-    double *out;
+    const double *gate;
 };
 
 #ifndef RWKV_GEMM_GN
@@ -311,6 +437,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         bx = xcd + kXcds * cslot;
     }
     if (by >= a.gy || bx >= a.gx || bz >= a.gz) return;
+    const int mat = bz / a.split;                       // which product; then which part of its contraction
+    bz -= mat * a.split;
+    const signed char *dig = mat == 0 ? a.dig[0] : mat == 1 ? a.dig[1] : a.dig[2];
+    const uint8_t *w16 = mat == 0 ? a.w16[0] : mat == 1 ? a.w16[1] : a.w16[2];
     const int mt0 = by * 16 + wm * kGM, nt0 = bx * kGemmNT + wn * kGN;
     const int kb0 = bz * a.kb_per_split;
     int kb1 = kb0 + a.kb_per_split;
@@ -325,11 +455,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         if (f < 16) {
             int mt = by * 16 + f;
             if (mt >= a.MT) mt = a.MT - 1;              // clamped: loads stay unconditional, results are dropped
-            src[i] = reinterpret_cast<const v4i *>(a.dig + ((size_t)mt * a.KB + kb0) * 1024) + lane;
+            src[i] = reinterpret_cast<const v4i *>(dig + ((size_t)mt * a.KB + kb0) * 1024) + lane;
         } else {
             int nt = bx * kGemmNT + (f - 16);
             if (nt >= a.NT) nt = a.NT - 1;
-            src[i] = reinterpret_cast<const v4i *>(a.w16 + ((size_t)nt * a.KB + kb0) * 1024) + lane;
+            src[i] = reinterpret_cast<const v4i *>(w16 + ((size_t)nt * a.KB + kb0) * 1024) + lane;
         }
     }
     v4i acc[kGM][kGN];
@@ -376,20 +506,27 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 #undef RWKV_GEMM_FETCH
     // lane 16g + n, register i  <->  digit i of token 4*mt + g, column 16*nt + n
     const int g = lane >> 4, n = lane & 15;
+    const double *Sv = mat == 0 ? a.S[0] : mat == 1 ? a.S[1] : a.S[2];
+    const double *qsv = mat == 0 ? a.qs[0] : mat == 1 ? a.qs[1] : a.qs[2];
+    const double *zpv = mat == 0 ? a.zp[0] : mat == 1 ? a.zp[1] : a.zp[2];
+    double *outv = mat == 0 ? a.out[0] : mat == 1 ? a.out[1] : a.out[2];
+    long long *totv = a.tot + (size_t)(mat * a.split + bz) * a.slice;      // this part's slice
 #pragma unroll
     for (int i = 0; i < kGM; ++i) {
         if (mt0 + i >= a.MT) continue;
+        const int t = 4 * (mt0 + i) + g;
+        double S = 0.0, add = 0.0;
+        if (a.tail >= 0 && t < a.R) { S = Sv[t]; add = 128.0 * (S * qsv[t]) + zpv[t]; }
 #pragma unroll
         for (int j = 0; j < kGN; ++j) {
             if (nt0 + j >= a.NT) continue;
             const v4i d = acc[i][j];
             const long long tot = ((((long long)d.x * 256 + d.y) * 256 + d.z) * 256) + d.w;
-            const int t = 4 * (mt0 + i) + g, col = 16 * (nt0 + j) + n;
+            const int col = 16 * (nt0 + j) + n;
             if (a.tail >= 0) {
                 if (t < a.R && col < a.N) {
-                    const double S = a.S[t];
-                    const double y = S * (double)tot + 128.0 * (S * a.qs[t]) + a.zp[t];
-                    double *o = a.out + (size_t)t * a.N + col;
+                    const double y = S * (double)tot + add;
+                    double *o = outv + (size_t)t * a.N + col;
                     if (a.tail == ROW_STORE) *o = y;
                     else if (a.tail == ROW_RELU2) { const double r = y > 0.0 ? y : 0.0; *o = r * r; }              // block.py:97
                     else if (a.tail == ROW_ADD) *o += y;                                                            // block.py:80
@@ -397,7 +534,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
                 }
                 continue;
             }
-            a.tot[(size_t)bz * a.slice + (size_t)t * a.ldd + col] = tot;     // this split's slice
+            totv[(size_t)t * a.ldd + col] = tot;
         }
     }
 }
@@ -409,22 +546,27 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 struct FinishArgs {
     int R, N, ldd, slices;
     size_t slice;
-    const long long *tot;
-    const double *S, *qs, *zp;
-    double *out;                // [R, N]
+    const long long *tot;       // [products][slices][...]
+    const double *S[kRowsMaxProducts], *qs[kRowsMaxProducts], *zp[kRowsMaxProducts];
+    double *out[kRowsMaxProducts];      // [R, N] each
     const double *gate;         // ROW_GATE_ADD: raw receptance [R, N]
 };
 
 template <int OP>
 __global__ void __launch_bounds__(256) rows_finish_kernel(const FinishArgs a) {
-    const int t = blockIdx.y;
+    const int t = blockIdx.y, mat = blockIdx.z;
     const int j = blockIdx.x * 256 + threadIdx.x;
     if (j >= a.N) return;
-    const double S = a.S[t];
+    const double *Sv = mat == 0 ? a.S[0] : mat == 1 ? a.S[1] : a.S[2];
+    const double *qsv = mat == 0 ? a.qs[0] : mat == 1 ? a.qs[1] : a.qs[2];
+    const double *zpv = mat == 0 ? a.zp[0] : mat == 1 ? a.zp[1] : a.zp[2];
+    double *outv = mat == 0 ? a.out[0] : mat == 1 ? a.out[1] : a.out[2];
+    const double S = Sv[t];
     long long tot = 0;                                   // integer partial sums of the contraction splits: exact in any order
-    for (int z = 0; z < a.slices; ++z) tot += a.tot[(size_t)z * a.slice + (size_t)t * a.ldd + j];
-    const double y = S * (double)tot + 128.0 * (S * a.qs[t]) + a.zp[t];
-    double *o = a.out + (size_t)t * a.N + j;
+    const long long *tp = a.tot + (size_t)mat * a.slices * a.slice + (size_t)t * a.ldd + j;
+    for (int z = 0; z < a.slices; ++z) tot += tp[(size_t)z * a.slice];
+    const double y = S * (double)tot + 128.0 * (S * qsv[t]) + zpv[t];
+    double *o = outv + (size_t)t * a.N + j;
     if (OP == ROW_STORE) *o = y;
     else if (OP == ROW_RELU2) { const double r = y > 0.0 ? y : 0.0; *o = r * r; }            // block.py:97
     else if (OP == ROW_ADD) *o += y;                                                          // block.py:80
@@ -545,61 +687,88 @@ int rows_embed(hipStream_t st, const int64_t *tokens, int64_t R, int V, int C, c
     return RWKV_OK;
 }
 
-int rows_ln_mix(hipStream_t st, int n_mix, int64_t R, int C, bool sequence, const double *x, const double *ln_w,
-                const double *ln_b, const double *mu, const double *prev0, double *shift_dst, int64_t prev_stride,
-                double *mix) {
-    LnMixArgs a;
+bool rows_ln_width_supported(int64_t C) { return C % 4 == 0 && C <= 6 * 4 * kRT; }
+
+int rows_ln_mix_quant(hipStream_t st, int n_mix, int64_t R, int C, bool sequence, const double *x, const double *ln_w,
+                      const double *ln_b, const double *mu, const double *prev0, double *shift_dst,
+                      int64_t prev_stride, const float *const *range, const double *const *offset,
+                      const RowsOperand *out) {
+    if (C % 64 != 0 || !rows_ln_width_supported(C))
+        return set_error(RWKV_ERR_SIZE, "rows_ln_mix_quant: width %d is not a multiple of 64 up to %d", C, 6 * 4 * kRT);
+    LnQuantArgs a;
     a.C = C; a.R = (int)R; a.sequence = sequence ? 1 : 0; a.x = x; a.ln_w = ln_w; a.ln_b = ln_b; a.mu = mu;
-    a.prev0 = prev0; a.shift_dst = shift_dst; a.prev_stride = prev_stride; a.mix = mix;
-    const dim3 grid((unsigned)R), block(kRT);
-    switch (n_mix) {
-        case 0: hipLaunchKernelGGL(rows_ln_mix_kernel<0>, grid, block, 0, st, a); break;
-        case 2: hipLaunchKernelGGL(rows_ln_mix_kernel<2>, grid, block, 0, st, a); break;
-        case 3: hipLaunchKernelGGL(rows_ln_mix_kernel<3>, grid, block, 0, st, a); break;
-        default: return set_error(RWKV_ERR_ARG, "rows_ln_mix: unsupported mix count %d", n_mix);
+    a.prev0 = prev0; a.shift_dst = shift_dst; a.prev_stride = prev_stride;
+    const int n_out = n_mix > 0 ? n_mix : 1;
+    for (int m = 0; m < 3; ++m) {
+        const int k = m < n_out ? m : 0;
+        a.range[m] = range[k]; a.offset[m] = offset[k];
+        a.dig[m] = out[k].dig; a.S[m] = out[k].S; a.qs[m] = out[k].qs; a.zp[m] = out[k].zp;
     }
-    RWKV_CHECK_LAUNCH("rows_ln_mix_kernel");
+    const dim3 grid((unsigned)R), block(kRT);
+    const bool small = C <= 3 * 4 * kRT;
+#define RWKV_LNQ(NM)                                                                                  \
+    do {                                                                                              \
+        if (small) hipLaunchKernelGGL((rows_ln_mix_quant_kernel<NM, 3>), grid, block, 0, st, a);      \
+        else hipLaunchKernelGGL((rows_ln_mix_quant_kernel<NM, 6>), grid, block, 0, st, a);            \
+    } while (0)
+    switch (n_mix) {
+        case 0: RWKV_LNQ(0); break;
+        case 2: RWKV_LNQ(2); break;
+        case 3: RWKV_LNQ(3); break;
+        default: return set_error(RWKV_ERR_ARG, "rows_ln_mix_quant: unsupported mix count %d", n_mix);
+    }
+#undef RWKV_LNQ
+    RWKV_CHECK_LAUNCH("rows_ln_mix_quant_kernel");
     return RWKV_OK;
 }
 
-int rows_matmul(hipStream_t st, const RowsScratch &s, int64_t R, int64_t K, int64_t N, const double *in,
-                const uint8_t *w16, const float *range, const double *offset, int op, double *out,
-                const double *gate) {
-    if (K % 64 != 0) return set_error(RWKV_ERR_SIZE, "rows_matmul: contraction length %lld is not a multiple of 64",
+int rows_quant(hipStream_t st, int64_t R, int64_t K, const double *in, const float *range, const double *offset,
+               const RowsOperand &out) {
+    if (K % 64 != 0) return set_error(RWKV_ERR_SIZE, "rows_quant: contraction length %lld is not a multiple of 64",
                                       (long long)K);
     QuantArgs q;
-    q.K = (int)K; q.in = in; q.range = range; q.offset = offset; q.dig = s.dig; q.S = s.S; q.qs = s.qs; q.zp = s.zp;
+    q.K = (int)K; q.in = in; q.range = range; q.offset = offset; q.dig = out.dig; q.S = out.S; q.qs = out.qs; q.zp = out.zp;
     hipLaunchKernelGGL(rows_quant_kernel, dim3((unsigned)R), dim3(kRT), 0, st, q);
     RWKV_CHECK_LAUNCH("rows_quant_kernel");
+    return RWKV_OK;
+}
 
+int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, int64_t R, int64_t K, int64_t N, int op,
+                  const double *gate) {
+    if (K % 64 != 0) return set_error(RWKV_ERR_SIZE, "rows_products: contraction length %lld is not a multiple of 64",
+                                      (long long)K);
+    if (n < 1 || n > kRowsMaxProducts) return set_error(RWKV_ERR_ARG, "rows_products: %d products in one launch", n);
+    if (op < ROW_STORE || op > ROW_GATE_ADD) return set_error(RWKV_ERR_ARG, "rows_products: unknown tail %d", op);
     GemmArgs g;
-    g.dig = s.dig; g.w16 = w16; g.tot = s.tot;
+    FinishArgs f;
+    for (int m = 0; m < kRowsMaxProducts; ++m) {
+        const RowsProduct &q = p[m < n ? m : 0];
+        g.dig[m] = q.a.dig; g.w16[m] = q.w16; g.S[m] = q.a.S; g.qs[m] = q.a.qs; g.zp[m] = q.a.zp; g.out[m] = q.out;
+        f.S[m] = q.a.S; f.qs[m] = q.a.qs; f.zp[m] = q.a.zp; f.out[m] = q.out;
+    }
+    g.tot = tot;
     g.MT = (int)ceil_div(R, 4); g.NT = (int)ceil_div(N, 16); g.KB = (int)(K / 64); g.ldd = g.NT * 16;
     const int gx = (int)ceil_div(g.NT, kGemmNT), gy = (int)ceil_div(g.MT, 16);
     // Split the contraction until the grid has a few workgroups per compute unit.
     int split = 1;
-    while (gx * gy * split < 256 && g.KB / (split * 2) >= 8 && split < kMaxSplit) split *= 2;
+    while (gx * gy * n * split < 256 && g.KB / (split * 2) >= 8 && split < kMaxSplit) split *= 2;
     g.kb_per_split = (int)ceil_div(g.KB, split);
-    g.atomic = split > 1;
+    g.split = split;
     g.slice = (size_t)g.MT * 4 * g.ldd;
-    g.gx = gx; g.gy = gy; g.gz = split; g.by_rows = gy >= kXcds;
+    g.gx = gx; g.gy = gy; g.gz = split * n; g.by_rows = gy >= kXcds;
     g.per_xcd = ((g.by_rows ? gy : gx) + kXcds - 1) / kXcds;
-    g.tail = g.atomic ? -1 : op; g.R = (int)R; g.N = (int)N; g.S = s.S; g.qs = s.qs; g.zp = s.zp; g.gate = gate; g.out = out;
-    if (op < ROW_STORE || op > ROW_GATE_ADD) return set_error(RWKV_ERR_ARG, "rows_matmul: unknown tail %d", op);
-    hipLaunchKernelGGL(gemm8_kernel, dim3((unsigned)(kXcds * g.per_xcd * (g.by_rows ? gx : gy) * split)), dim3(256), 0, st, g);
+    g.tail = split > 1 ? -1 : op; g.R = (int)R; g.N = (int)N; g.gate = gate;
+    hipLaunchKernelGGL(gemm8_kernel, dim3((unsigned)(kXcds * g.per_xcd * (g.by_rows ? gx : gy) * g.gz)), dim3(256), 0, st, g);
     RWKV_CHECK_LAUNCH("gemm8_kernel");
-    if (!g.atomic) return RWKV_OK;      // the tail was applied in the product's epilogue
+    if (split == 1) return RWKV_OK;     // the tail was applied in the product's epilogue
 
-    FinishArgs f;
-    f.R = (int)R; f.N = (int)N; f.ldd = g.ldd; f.slices = split; f.slice = g.slice; f.tot = s.tot; f.S = s.S; f.qs = s.qs; f.zp = s.zp; f.out = out;
-    f.gate = gate;
-    const dim3 fg((unsigned)ceil_div(N, 256), (unsigned)R), fb(256);
+    f.R = (int)R; f.N = (int)N; f.ldd = g.ldd; f.slices = split; f.slice = g.slice; f.tot = tot; f.gate = gate;
+    const dim3 fg((unsigned)ceil_div(N, 256), (unsigned)R, (unsigned)n), fb(256);
     switch (op) {
         case ROW_STORE: hipLaunchKernelGGL(rows_finish_kernel<ROW_STORE>, fg, fb, 0, st, f); break;
         case ROW_RELU2: hipLaunchKernelGGL(rows_finish_kernel<ROW_RELU2>, fg, fb, 0, st, f); break;
         case ROW_ADD: hipLaunchKernelGGL(rows_finish_kernel<ROW_ADD>, fg, fb, 0, st, f); break;
-        case ROW_GATE_ADD: hipLaunchKernelGGL(rows_finish_kernel<ROW_GATE_ADD>, fg, fb, 0, st, f); break;
-        default: return set_error(RWKV_ERR_ARG, "rows_matmul: unknown tail %d", op);
+        default: hipLaunchKernelGGL(rows_finish_kernel<ROW_GATE_ADD>, fg, fb, 0, st, f); break;
     }
     RWKV_CHECK_LAUNCH("rows_finish_kernel");
     return RWKV_OK;
