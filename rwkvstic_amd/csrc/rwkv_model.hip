@@ -602,6 +602,29 @@ int head_logits(rwkv_model *m, hipStream_t st, const double *xrow, double *logit
     return RWKV_OK;
 }
 
+// Which path a sequence of T tokens takes: the many-row kernels for prompts, and for single tokens too when
+// the persistent single-token kernel does not serve the shape (their integer products beat one launch per
+// phase with float32 sums both in time and in accuracy).
+bool use_rows(const rwkv_model *m, int64_t T) { return rows_supported(m) && (T >= kRowsMin || !m->fused); }
+
+// T consecutive tokens of one sequence through the many-row kernels, in chunks of kRowsChunk rows; logits
+// from the last row only.  workspace: as rwkv_model_workspace_bytes(m, T) sizes it.
+int rows_sequence(rwkv_model *m, hipStream_t st, const int64_t *tokens, int64_t T, double *state, double *logits,
+                  void *workspace) {
+    const int64_t C = m->d.n_embd, F = m->d.n_ffn;
+    unsigned char *rows_base = static_cast<unsigned char *>(workspace) + round_up(ws_doubles(C, F) * sizeof(double), 256);
+    const int64_t Rmax = T < kRowsChunk ? T : kRowsChunk;
+    const RowsWs rw = rows_carve(rows_base, Rmax, C, F, F);
+    for (int64_t t0 = 0; t0 < T; t0 += kRowsChunk) {
+        const int64_t R = T - t0 < kRowsChunk ? T - t0 : kRowsChunk;
+        int rc = rows_layers(m, st, tokens + t0, R, true, state, 0, rw);
+        if (rc) return rc;
+        if (t0 + R == T) rc = head_logits(m, st, rw.x + (size_t)(R - 1) * C, logits);
+        if (rc) return rc;
+    }
+    return RWKV_OK;
+}
+
 // One token through the persistent kernel (argument checks done by the caller).
 int fused_token(rwkv_model *m, hipStream_t st, const int64_t *token, double *state, double *logits) {
     const int rc = decode_launch(st, m->dm, m->db, m->epoch, token, state, logits);
@@ -683,7 +706,7 @@ int rwkv_model_check(rwkv_model *m) {
 size_t rwkv_model_workspace_bytes(const rwkv_model *m, int64_t max_tokens) {
     if (!m || max_tokens <= 0) return 0;
     size_t n = round_up(ws_doubles(m->d.n_embd, m->d.n_ffn) * sizeof(double), 256);
-    if (max_tokens >= kRowsMin && rows_supported(m)) {
+    if (use_rows(m, max_tokens)) {
         const int64_t R = max_tokens < kRowsChunk ? max_tokens : kRowsChunk;
         n += rows_ws_bytes(R, m->d.n_embd, m->d.n_ffn, m->d.n_ffn);
     }
@@ -701,23 +724,7 @@ int rwkv_model_forward(rwkv_model *m, rwkv_stream_t stream, const int64_t *token
     int rc = check_forward_args(m, tokens, state, logits, workspace, workspace_bytes, T, "rwkv_model_forward");
     if (rc) return rc;
     const Workspace w = carve(workspace, m->d.n_embd, m->d.n_ffn);
-    if (T >= kRowsMin && rows_supported(m)) {
-        // prompt: GEMM path in chunks of kRowsChunk rows, logits from the last row only
-        const hipStream_t st = (hipStream_t)stream;
-        const int64_t C = m->d.n_embd, F = m->d.n_ffn;
-        unsigned char *rows_base = static_cast<unsigned char *>(workspace) +
-                                   round_up(ws_doubles(C, F) * sizeof(double), 256);
-        const int64_t Rmax = T < kRowsChunk ? T : kRowsChunk;
-        const RowsWs rw = rows_carve(rows_base, Rmax, C, F, F);
-        for (int64_t t0 = 0; t0 < T; t0 += kRowsChunk) {
-            const int64_t R = T - t0 < kRowsChunk ? T - t0 : kRowsChunk;
-            rc = rows_layers(m, st, tokens + t0, R, true, state, 0, rw);
-            if (rc) return rc;
-            if (t0 + R == T) rc = head_logits(m, st, rw.x + (size_t)(R - 1) * C, logits);
-            if (rc) return rc;
-        }
-        return RWKV_OK;
-    }
+    if (use_rows(m, T)) return rows_sequence(m, (hipStream_t)stream, tokens, T, state, logits, workspace);
     for (int64_t t = 0; t < T; ++t) {
         if (m->fused) rc = fused_token(m, (hipStream_t)stream, tokens + t, state, logits);
         else rc = step_token(m, (hipStream_t)stream, tokens + t, state, logits, w, t == T - 1);
@@ -802,7 +809,8 @@ int rwkv_model_decode_greedy(rwkv_model *m, rwkv_stream_t stream, int64_t *token
         return rc;
     }
     for (int64_t i = 0; i < n; ++i) {
-        rc = step_token(m, (hipStream_t)stream, tokens + i, state, logits, w, true);
+        if (use_rows(m, 1)) rc = rows_sequence(m, (hipStream_t)stream, tokens + i, 1, state, logits, workspace);
+        else rc = step_token(m, (hipStream_t)stream, tokens + i, state, logits, w, true);
         if (rc) return rc;
         rc = rwkv_argmax_f64(stream, logits, m->d.n_vocab, tokens + i + 1);
         if (rc) return rc;

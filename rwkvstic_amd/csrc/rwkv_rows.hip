@@ -147,20 +147,42 @@ struct LnQuantArgs {
     double *S[3], *qs[3], *zp[3];
 };
 
+constexpr int kLT = 512, kLW = kLT / 64;    // threads / wavefronts of the LayerNorm kernel
+
+// Sum of N values per thread over the kLT threads (fixed order), broadcast.
+template <int N>
+__device__ __forceinline__ void lsum(double (&v)[N], double *red /*[N*kLW]*/) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        const double s = wsum(v[i]);
+        if (lane == 0) red[i * kLW + wave] = s;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        double s = 0.0;
+#pragma unroll
+        for (int w = 0; w < kLW; ++w) s += red[i * kLW + w];
+        v[i] = s;
+    }
+    __syncthreads();
+}
+
 template <int NM, int NSEG>
-__global__ void __launch_bounds__(kRT) rows_ln_mix_quant_kernel(const LnQuantArgs a) {
+__global__ void __launch_bounds__(kLT) rows_ln_mix_quant_kernel(const LnQuantArgs a) {
     constexpr int NO = NM > 0 ? NM : 1;
-    __shared__ double red[4 * kRW];
-    __shared__ float redf[NO * kRW];
-    const int t = blockIdx.x, C = a.C, nq = C >> 2, tid = threadIdx.x;
+    __shared__ double red[3 * kLW];
+    __shared__ float redf[NO * kLW];
+    const int t = blockIdx.x, C = a.C, tid = threadIdx.x;
     const bool need_prev = NM > 0 && a.sequence && t > 0;
     const double *xr = a.x + (size_t)t * C;
     const double *pr = NM == 0 ? xr : need_prev ? xr - C : a.sequence ? a.prev0 : a.prev0 + (size_t)t * a.prev_stride;
-    double xv[NSEG][4], pv[NSEG][4];
+    double xv[NSEG][4], pv[NSEG][4], lw[NSEG][4], lb[NSEG][4];
     double s[2] = {0.0, 0.0};
 #pragma unroll
     for (int g = 0; g < NSEG; ++g) {
-        const int c0 = 4 * (tid + g * kRT);
+        const int c0 = 4 * (tid + g * kLT);
         if (c0 < C) {
             const double2 x0 = *reinterpret_cast<const double2 *>(xr + c0), x1 = *reinterpret_cast<const double2 *>(xr + c0 + 2);
             xv[g][0] = x0.x; xv[g][1] = x0.y; xv[g][2] = x1.x; xv[g][3] = x1.y;
@@ -168,16 +190,21 @@ __global__ void __launch_bounds__(kRT) rows_ln_mix_quant_kernel(const LnQuantArg
                 const double2 p0 = *reinterpret_cast<const double2 *>(pr + c0), p1 = *reinterpret_cast<const double2 *>(pr + c0 + 2);
                 pv[g][0] = p0.x; pv[g][1] = p0.y; pv[g][2] = p1.x; pv[g][3] = p1.y;
             }
+            // the LayerNorm weights travel with the row: nothing is left to fetch between the reductions
+            const double2 w0 = *reinterpret_cast<const double2 *>(a.ln_w + c0), w1 = *reinterpret_cast<const double2 *>(a.ln_w + c0 + 2);
+            const double2 b0 = *reinterpret_cast<const double2 *>(a.ln_b + c0), b1 = *reinterpret_cast<const double2 *>(a.ln_b + c0 + 2);
+            lw[g][0] = w0.x; lw[g][1] = w0.y; lw[g][2] = w1.x; lw[g][3] = w1.y;
+            lb[g][0] = b0.x; lb[g][1] = b0.y; lb[g][2] = b1.x; lb[g][3] = b1.y;
 #pragma unroll
             for (int i = 0; i < 4; ++i) { s[0] += xv[g][i]; if (NM > 0) s[1] += pv[g][i]; }
         }
     }
-    rsum<2>(s, red);
+    lsum<2>(s, red);
     const double mean = s[0] / (double)C, meanp = s[1] / (double)C;
     double q[2] = {0.0, 0.0};
 #pragma unroll
     for (int g = 0; g < NSEG; ++g) {
-        if (4 * (tid + g * kRT) < C) {
+        if (4 * (tid + g * kLT) < C) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const double d = xv[g][i] - mean;
@@ -186,7 +213,7 @@ __global__ void __launch_bounds__(kRT) rows_ln_mix_quant_kernel(const LnQuantArg
             }
         }
     }
-    rsum<2>(q, red);
+    lsum<2>(q, red);
     const double sd = sqrt(q[0] / (double)C + 1e-5), sdp = sqrt(q[1] / (double)C + 1e-5);
     float xs[NO][NSEG][4];
     float amax[NO];
@@ -195,19 +222,13 @@ __global__ void __launch_bounds__(kRT) rows_ln_mix_quant_kernel(const LnQuantArg
     for (int m = 0; m < NO; ++m) { amax[m] = 0.f; z[m] = 0.0; }
 #pragma unroll
     for (int g = 0; g < NSEG; ++g) {
-        const int c0 = 4 * (tid + g * kRT);
+        const int c0 = 4 * (tid + g * kLT);
         if (c0 < C) {
             double xy[4], prev[4];
 #pragma unroll
-            for (int i = 0; i < 4; i += 2) {
-                const double2 w = *reinterpret_cast<const double2 *>(a.ln_w + c0 + i);
-                const double2 b = *reinterpret_cast<const double2 *>(a.ln_b + c0 + i);
-                xy[i] = w.x * ((xv[g][i] - mean) / sd) + b.x;
-                xy[i + 1] = w.y * ((xv[g][i + 1] - mean) / sd) + b.y;
-                if (NM > 0) {
-                    prev[i] = need_prev ? w.x * ((pv[g][i] - meanp) / sdp) + b.x : pv[g][i];
-                    prev[i + 1] = need_prev ? w.y * ((pv[g][i + 1] - meanp) / sdp) + b.y : pv[g][i + 1];
-                }
+            for (int i = 0; i < 4; ++i) {
+                xy[i] = lw[g][i] * ((xv[g][i] - mean) / sd) + lb[g][i];
+                if (NM > 0) prev[i] = need_prev ? lw[g][i] * ((pv[g][i] - meanp) / sdp) + lb[g][i] : pv[g][i];
             }
 #pragma unroll
             for (int m = 0; m < NO; ++m) {
@@ -241,25 +262,25 @@ __global__ void __launch_bounds__(kRT) rows_ln_mix_quant_kernel(const LnQuantArg
 #pragma unroll
     for (int m = 0; m < NO; ++m) {
         amax[m] = wmaxf(amax[m]);
-        if ((tid & 63) == 0) redf[m * kRW + (tid >> 6)] = amax[m];
+        if ((tid & 63) == 0) redf[m * kLW + (tid >> 6)] = amax[m];
     }
-    rsum<NO>(z, red);                      // (its barriers also publish redf)
+    lsum<NO>(z, red);                      // (its barriers also publish redf)
     double S[NO], invS[NO], qsum[NO];
     const int KB = C >> 6;
 #pragma unroll
     for (int m = 0; m < NO; ++m) {
-        float am = redf[m * kRW];
+        float am = redf[m * kLW];
 #pragma unroll
-        for (int w = 1; w < kRW; ++w) am = fmaxf(am, redf[m * kRW + w]);
+        for (int w = 1; w < kLW; ++w) am = fmaxf(am, redf[m * kLW + w]);
         row_scale(am, S[m], invS[m]);
         qsum[m] = 0.0;
 #pragma unroll
         for (int g = 0; g < NSEG; ++g) {
-            const int c0 = 4 * (tid + g * kRT);
+            const int c0 = 4 * (tid + g * kLT);
             if (c0 < C) qsum[m] += emit_quad(xs[m][g], invS[m], c0, t, KB, a.dig[m]);
         }
     }
-    rsum<NO>(qsum, red);
+    lsum<NO>(qsum, red);
     if (tid == 0) {
 #pragma unroll
         for (int m = 0; m < NO; ++m) { a.S[m][t] = S[m]; a.qs[m][t] = qsum[m]; a.zp[m][t] = z[m]; }
@@ -417,6 +438,46 @@ constexpr int kGemmAhead = 3;           // contraction blocks on their way from 
 // the wavefront has in flight, which would drain the prefetched contraction blocks at every step.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// Accumulators of one wavefront (GM M-tiles x GN N-tiles from (mt0, nt0)) to totals or, when the
+// contraction is not split, straight through the product's tail.
+template <int GM, int GN>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs &a, const v4i (&acc)[GM][GN], int mt0, int nt0, int mat,
+                                              int bz, int lane) {
+    // lane 16g + n, register i  <->  digit i of token 4*mt + g, column 16*nt + n
+    const int g = lane >> 4, n = lane & 15;
+    const double *Sv = mat == 0 ? a.S[0] : mat == 1 ? a.S[1] : a.S[2];
+    const double *qsv = mat == 0 ? a.qs[0] : mat == 1 ? a.qs[1] : a.qs[2];
+    const double *zpv = mat == 0 ? a.zp[0] : mat == 1 ? a.zp[1] : a.zp[2];
+    double *outv = mat == 0 ? a.out[0] : mat == 1 ? a.out[1] : a.out[2];
+    long long *totv = a.tot + (size_t)(mat * a.split + bz) * a.slice;      // this part's slice
+#pragma unroll
+    for (int i = 0; i < GM; ++i) {
+        if (mt0 + i >= a.MT) continue;
+        const int t = 4 * (mt0 + i) + g;
+        double S = 0.0, add = 0.0;
+        if (a.tail >= 0 && t < a.R) { S = Sv[t]; add = 128.0 * (S * qsv[t]) + zpv[t]; }
+#pragma unroll
+        for (int j = 0; j < GN; ++j) {
+            if (nt0 + j >= a.NT) continue;
+            const v4i d = acc[i][j];
+            const long long tot = ((((long long)d.x * 256 + d.y) * 256 + d.z) * 256) + d.w;
+            const int col = 16 * (nt0 + j) + n;
+            if (a.tail >= 0) {
+                if (t < a.R && col < a.N) {
+                    const double y = S * (double)tot + add;
+                    double *o = outv + (size_t)t * a.N + col;
+                    if (a.tail == ROW_STORE) *o = y;
+                    else if (a.tail == ROW_RELU2) { const double r = y > 0.0 ? y : 0.0; *o = r * r; }              // block.py:97
+                    else if (a.tail == ROW_ADD) *o += y;                                                            // block.py:80
+                    else *o += y * (1.0 / (1.0 + exp(-a.gate[(size_t)t * a.N + col])));                             // block.py:95-100
+                }
+                continue;
+            }
+            totv[(size_t)t * a.ldd + col] = tot;
+        }
+    }
+}
+
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) gemm8_kernel(const GemmArgs a) {
     // Both operands of a contraction block are fetched once per workgroup (registers, kGemmAhead
     // blocks ahead), parked in LDS (two buffers, one barrier per block) and read from there by the
@@ -480,7 +541,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         F.v0 = src[0][o_]; F.v1 = src[1][o_]; F.v2 = src[2][o_]; F.v3 = src[3][o_]; F.v4 = src[4][o_]; if (kGemmLoads > 5) F.v5 = src[kGemmLoads - 1][o_]; \
     } while (0)
 #define RWKV_GEMM_STEP(F, K)                                                                         \
-    if ((K) < nk) { /* uniform */                                                                    \
+    {                                                                                                \
         const int buf_ = (K) & 1;                                                                    \
         frag[buf_][wave][lane] = F.v0; frag[buf_][wave + 4][lane] = F.v1; frag[buf_][wave + 8][lane] = F.v2;     \
         frag[buf_][wave + 12][lane] = F.v3; frag[buf_][wave + 16][lane] = F.v4; if (kGemmLoads > 5) frag[buf_][wave + 4 * (kGemmLoads - 1)][lane] = F.v5; \
@@ -497,48 +558,115 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         }                                                                                            \
     }
     RWKV_GEMM_FETCH(fly0, 0); RWKV_GEMM_FETCH(fly1, 1); RWKV_GEMM_FETCH(fly2, 2);
-    for (int k0 = 0; k0 < nk; k0 += kGemmAhead) {
+    // whole rounds run without a branch between the steps: the compiler then counts exactly which loads
+    // a step has to wait for (with a test per step it drains every load in flight once per round)
+    int k0 = 0;
+    for (; k0 + kGemmAhead <= nk; k0 += kGemmAhead) {
         RWKV_GEMM_STEP(fly0, k0)
         RWKV_GEMM_STEP(fly1, k0 + 1)
         RWKV_GEMM_STEP(fly2, k0 + 2)
     }
+    if (k0 < nk) RWKV_GEMM_STEP(fly0, k0)
+    if (k0 + 1 < nk) RWKV_GEMM_STEP(fly1, k0 + 1)
 #undef RWKV_GEMM_STEP
 #undef RWKV_GEMM_FETCH
-    // lane 16g + n, register i  <->  digit i of token 4*mt + g, column 16*nt + n
-    const int g = lane >> 4, n = lane & 15;
-    const double *Sv = mat == 0 ? a.S[0] : mat == 1 ? a.S[1] : a.S[2];
-    const double *qsv = mat == 0 ? a.qs[0] : mat == 1 ? a.qs[1] : a.qs[2];
-    const double *zpv = mat == 0 ? a.zp[0] : mat == 1 ? a.zp[1] : a.zp[2];
-    double *outv = mat == 0 ? a.out[0] : mat == 1 ? a.out[1] : a.out[2];
-    long long *totv = a.tot + (size_t)(mat * a.split + bz) * a.slice;      // this part's slice
-#pragma unroll
-    for (int i = 0; i < kGM; ++i) {
-        if (mt0 + i >= a.MT) continue;
-        const int t = 4 * (mt0 + i) + g;
-        double S = 0.0, add = 0.0;
-        if (a.tail >= 0 && t < a.R) { S = Sv[t]; add = 128.0 * (S * qsv[t]) + zpv[t]; }
-#pragma unroll
-        for (int j = 0; j < kGN; ++j) {
-            if (nt0 + j >= a.NT) continue;
-            const v4i d = acc[i][j];
-            const long long tot = ((((long long)d.x * 256 + d.y) * 256 + d.z) * 256) + d.w;
-            const int col = 16 * (nt0 + j) + n;
-            if (a.tail >= 0) {
-                if (t < a.R && col < a.N) {
-                    const double y = S * (double)tot + add;
-                    double *o = outv + (size_t)t * a.N + col;
-                    if (a.tail == ROW_STORE) *o = y;
-                    else if (a.tail == ROW_RELU2) { const double r = y > 0.0 ? y : 0.0; *o = r * r; }              // block.py:97
-                    else if (a.tail == ROW_ADD) *o += y;                                                            // block.py:80
-                    else *o += y * (1.0 / (1.0 + exp(-a.gate[(size_t)t * a.N + col])));                             // block.py:95-100
-                }
-                continue;
-            }
-            totv[(size_t)t * a.ldd + col] = tot;
-        }
-    }
+    gemm_epilogue<kGM, kGN>(a, acc, mt0, nt0, mat, bz, lane);
 }
 
+// ---------------------------------------------------------------------------
+// The same product for at most 32 rows (a batch of single tokens): the weights are read once and
+// hardly reused, so what counts is how many weight bytes a compute unit has in flight.  Workgroup =
+// 4 wavefronts side by side = 8 M-tiles x 8 N-tiles (wavefront: 8 x 2); a contraction block is 8 digit
+// fragments + 8 weight fragments, fetched kSkinnyAhead blocks ahead (48 KiB of weights per workgroup).
+// ---------------------------------------------------------------------------
+constexpr int kSkinnyMT = 8, kSkinnyGN = 2, kSkinnyNT = 4 * kSkinnyGN;
+constexpr int kSkinnyFrags = kSkinnyMT + kSkinnyNT;     // 16: wave w fetches fragments w, w + 4, w + 8, w + 12
+constexpr int kSkinnyAhead = 6;
+
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) gemm8_skinny_kernel(const GemmArgs a) {
+    __shared__ v4i frag[2][kSkinnyFrags][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int xcd = blockIdx.x % kXcds;
+    int item = blockIdx.x / kXcds;
+    const int cslot = item % a.per_xcd; item /= a.per_xcd;      // the XCDs share out the column blocks
+    const int bx = xcd + kXcds * cslot;
+    int bz = item;
+    if (bx >= a.gx || bz >= a.gz) return;
+    const int mat = bz / a.split;
+    bz -= mat * a.split;
+    const signed char *dig = mat == 0 ? a.dig[0] : mat == 1 ? a.dig[1] : a.dig[2];
+    const uint8_t *w16 = mat == 0 ? a.w16[0] : mat == 1 ? a.w16[1] : a.w16[2];
+    const int nt0 = bx * kSkinnyNT + wave * kSkinnyGN;
+    const int kb0 = bz * a.kb_per_split;
+    int kb1 = kb0 + a.kb_per_split;
+    if (kb1 > a.KB) kb1 = a.KB;
+    if (kb0 >= kb1) return;                             // (uniform for the workgroup)
+    const int nk = kb1 - kb0;
+
+    const v4i *src[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int f = wave + 4 * i;
+        if (f < kSkinnyMT) {
+            const int mt = f < a.MT ? f : a.MT - 1;     // clamped: loads stay unconditional, results are dropped
+            src[i] = reinterpret_cast<const v4i *>(dig + ((size_t)mt * a.KB + kb0) * 1024) + lane;
+        } else {
+            int nt = bx * kSkinnyNT + (f - kSkinnyMT);
+            if (nt >= a.NT) nt = a.NT - 1;
+            src[i] = reinterpret_cast<const v4i *>(w16 + ((size_t)nt * a.KB + kb0) * 1024) + lane;
+        }
+    }
+    v4i acc[kSkinnyMT][kSkinnyGN];
+#pragma unroll
+    for (int i = 0; i < kSkinnyMT; ++i)
+#pragma unroll
+        for (int j = 0; j < kSkinnyGN; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+
+    static_assert(kSkinnyAhead == 6, "six named stages below");
+    struct Fly { v4i v0, v1, v2, v3; };                 // named members, not an array: they must stay registers
+    Fly fly0, fly1, fly2, fly3, fly4, fly5;
+#define RWKV_SKINNY_FETCH(F, K)                                                                      \
+    do {                                                                                             \
+        const size_t o_ = (size_t)((K) < nk ? (K) : nk - 1) * 64; /* past the end: the last block again (unused) */ \
+        F.v0 = src[0][o_]; F.v1 = src[1][o_]; F.v2 = src[2][o_]; F.v3 = src[3][o_];                  \
+    } while (0)
+#define RWKV_SKINNY_STEP(F, K)                                                                       \
+    {                                                                                                \
+        const int buf_ = (K) & 1;                                                                    \
+        frag[buf_][wave][lane] = F.v0; frag[buf_][wave + 4][lane] = F.v1;                            \
+        frag[buf_][wave + 8][lane] = F.v2; frag[buf_][wave + 12][lane] = F.v3;                       \
+        RWKV_SKINNY_FETCH(F, (K) + kSkinnyAhead);                                                    \
+        lds_barrier();                                                                               \
+        v4i Bv_[kSkinnyGN];                                                                          \
+        _Pragma("unroll") for (int j = 0; j < kSkinnyGN; ++j)                                        \
+            Bv_[j] = frag[buf_][kSkinnyMT + wave * kSkinnyGN + j][lane];                             \
+        _Pragma("unroll") for (int i = 0; i < kSkinnyMT; ++i) {                                      \
+            const v4i Av_ = frag[buf_][i][lane];                                                     \
+            _Pragma("unroll") for (int j = 0; j < kSkinnyGN; ++j)                                    \
+                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Av_, Bv_[j], acc[i][j], 0, 0, 0);  \
+        }                                                                                            \
+    }
+    RWKV_SKINNY_FETCH(fly0, 0); RWKV_SKINNY_FETCH(fly1, 1); RWKV_SKINNY_FETCH(fly2, 2);
+    RWKV_SKINNY_FETCH(fly3, 3); RWKV_SKINNY_FETCH(fly4, 4); RWKV_SKINNY_FETCH(fly5, 5);
+    int k0 = 0;
+    for (; k0 + kSkinnyAhead <= nk; k0 += kSkinnyAhead) {      // whole rounds: no branch between the steps
+        RWKV_SKINNY_STEP(fly0, k0)
+        RWKV_SKINNY_STEP(fly1, k0 + 1)
+        RWKV_SKINNY_STEP(fly2, k0 + 2)
+        RWKV_SKINNY_STEP(fly3, k0 + 3)
+        RWKV_SKINNY_STEP(fly4, k0 + 4)
+        RWKV_SKINNY_STEP(fly5, k0 + 5)
+    }
+    if (k0 < nk) RWKV_SKINNY_STEP(fly0, k0)
+    if (k0 + 1 < nk) RWKV_SKINNY_STEP(fly1, k0 + 1)
+    if (k0 + 2 < nk) RWKV_SKINNY_STEP(fly2, k0 + 2)
+    if (k0 + 3 < nk) RWKV_SKINNY_STEP(fly3, k0 + 3)
+    if (k0 + 4 < nk) RWKV_SKINNY_STEP(fly4, k0 + 4)
+#undef RWKV_SKINNY_STEP
+#undef RWKV_SKINNY_FETCH
+    gemm_epilogue<kSkinnyMT, kSkinnyGN>(a, acc, 0, nt0, mat, bz, lane);
+}
 
 // ---------------------------------------------------------------------------
 // y[t, j] = S_t * tot + 128 * S_t * sum q_t + zp_t, then the phase's element-wise tail.
@@ -668,12 +796,17 @@ __global__ void __launch_bounds__(64) wkv_chunk_replay_kernel(const WkvRowsArgs 
 size_t rows_dig_bytes(int64_t R, int64_t K) { return (size_t)(ceil_div(R, 4) * (K / 64) * 1024); }
 size_t rows_wkv_scratch_bytes(int64_t R, int64_t C) { return (size_t)(ceil_div(R, kWkvChunk) * 3 * C * 8); }
 constexpr int kMaxSplit = 8;
+#ifndef RWKV_GEMM_FILL
+#define RWKV_GEMM_FILL 256
+#endif
+constexpr int kGemmFillWgs = RWKV_GEMM_FILL;   // the contraction is split until the grid has this many workgroups
 // Upper bound of the number of contraction splits rows_matmul will choose for R rows and N columns:
 // each split writes its own slice of totals (summed by the tail kernel), so the buffer has that many.
 static int gemm_split_bound(int64_t R, int64_t N) {
-    const int64_t gx = ceil_div(ceil_div(N, 16), kGemmNT), gy = ceil_div(ceil_div(R, 4), 16);
+    const int64_t MT = ceil_div(R, 4);
+    const int64_t gx = ceil_div(ceil_div(N, 16), MT <= kSkinnyMT ? kSkinnyNT : kGemmNT), gy = ceil_div(MT, 16);
     int s = 1;
-    while (gx * gy * s < 256 && s < kMaxSplit) s *= 2;
+    while (gx * gy * s < kGemmFillWgs && s < kMaxSplit) s *= 2;
     return s;
 }
 size_t rows_tot_bytes(int64_t R, int64_t N) {
@@ -687,14 +820,14 @@ int rows_embed(hipStream_t st, const int64_t *tokens, int64_t R, int V, int C, c
     return RWKV_OK;
 }
 
-bool rows_ln_width_supported(int64_t C) { return C % 4 == 0 && C <= 6 * 4 * kRT; }
+bool rows_ln_width_supported(int64_t C) { return C % 4 == 0 && C <= 3 * 4 * kLT; }
 
 int rows_ln_mix_quant(hipStream_t st, int n_mix, int64_t R, int C, bool sequence, const double *x, const double *ln_w,
                       const double *ln_b, const double *mu, const double *prev0, double *shift_dst,
                       int64_t prev_stride, const float *const *range, const double *const *offset,
                       const RowsOperand *out) {
     if (C % 64 != 0 || !rows_ln_width_supported(C))
-        return set_error(RWKV_ERR_SIZE, "rows_ln_mix_quant: width %d is not a multiple of 64 up to %d", C, 6 * 4 * kRT);
+        return set_error(RWKV_ERR_SIZE, "rows_ln_mix_quant: width %d is not a multiple of 64 up to %d", C, 3 * 4 * kLT);
     LnQuantArgs a;
     a.C = C; a.R = (int)R; a.sequence = sequence ? 1 : 0; a.x = x; a.ln_w = ln_w; a.ln_b = ln_b; a.mu = mu;
     a.prev0 = prev0; a.shift_dst = shift_dst; a.prev_stride = prev_stride;
@@ -704,12 +837,12 @@ int rows_ln_mix_quant(hipStream_t st, int n_mix, int64_t R, int C, bool sequence
         a.range[m] = range[k]; a.offset[m] = offset[k];
         a.dig[m] = out[k].dig; a.S[m] = out[k].S; a.qs[m] = out[k].qs; a.zp[m] = out[k].zp;
     }
-    const dim3 grid((unsigned)R), block(kRT);
-    const bool small = C <= 3 * 4 * kRT;
+    const dim3 grid((unsigned)R), block(kLT);
+    const bool small = C <= 2 * 4 * kLT;
 #define RWKV_LNQ(NM)                                                                                  \
     do {                                                                                              \
-        if (small) hipLaunchKernelGGL((rows_ln_mix_quant_kernel<NM, 3>), grid, block, 0, st, a);      \
-        else hipLaunchKernelGGL((rows_ln_mix_quant_kernel<NM, 6>), grid, block, 0, st, a);            \
+        if (small) hipLaunchKernelGGL((rows_ln_mix_quant_kernel<NM, 2>), grid, block, 0, st, a);      \
+        else hipLaunchKernelGGL((rows_ln_mix_quant_kernel<NM, 3>), grid, block, 0, st, a);            \
     } while (0)
     switch (n_mix) {
         case 0: RWKV_LNQ(0); break;
@@ -748,17 +881,20 @@ int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, i
     }
     g.tot = tot;
     g.MT = (int)ceil_div(R, 4); g.NT = (int)ceil_div(N, 16); g.KB = (int)(K / 64); g.ldd = g.NT * 16;
-    const int gx = (int)ceil_div(g.NT, kGemmNT), gy = (int)ceil_div(g.MT, 16);
+    const bool skinny = g.MT <= kSkinnyMT;              // few rows: the weight-streaming variant
+    const int gx = (int)ceil_div(g.NT, skinny ? kSkinnyNT : kGemmNT), gy = (int)ceil_div(g.MT, 16);
     // Split the contraction until the grid has a few workgroups per compute unit.
     int split = 1;
-    while (gx * gy * n * split < 256 && g.KB / (split * 2) >= 8 && split < kMaxSplit) split *= 2;
+    while (gx * gy * n * split < kGemmFillWgs && g.KB / (split * 2) >= 8 && split < kMaxSplit) split *= 2;
     g.kb_per_split = (int)ceil_div(g.KB, split);
     g.split = split;
     g.slice = (size_t)g.MT * 4 * g.ldd;
     g.gx = gx; g.gy = gy; g.gz = split * n; g.by_rows = gy >= kXcds;
     g.per_xcd = ((g.by_rows ? gy : gx) + kXcds - 1) / kXcds;
     g.tail = split > 1 ? -1 : op; g.R = (int)R; g.N = (int)N; g.gate = gate;
-    hipLaunchKernelGGL(gemm8_kernel, dim3((unsigned)(kXcds * g.per_xcd * (g.by_rows ? gx : gy) * g.gz)), dim3(256), 0, st, g);
+    const dim3 grid((unsigned)(kXcds * g.per_xcd * (g.by_rows ? gx : gy) * g.gz));
+    if (skinny) hipLaunchKernelGGL(gemm8_skinny_kernel, grid, dim3(256), 0, st, g);
+    else hipLaunchKernelGGL(gemm8_kernel, grid, dim3(256), 0, st, g);
     RWKV_CHECK_LAUNCH("gemm8_kernel");
     if (split == 1) return RWKV_OK;     // the tail was applied in the product's epilogue
 
