@@ -424,14 +424,8 @@ struct GemmArgs {
     const double *gate;
 };
 
-#ifndef RWKV_GEMM_GN
-#define RWKV_GEMM_GN 4
-#endif
-constexpr int kGM = 8, kGN = RWKV_GEMM_GN;   // M-tiles x N-tiles of accumulators per wavefront
-constexpr int kGemmNT = 2 * kGN;         // N-tiles per workgroup (two wavefronts side by side)
-
-constexpr int kGemmFrags = 16 + kGemmNT; // fragments of one contraction block: 16 M-tiles of digits, kGemmNT N-tiles of weights
-constexpr int kGemmLoads = kGemmFrags / 4;   // per thread and contraction block (wave w fetches fragments w, w + 4, ...)
+constexpr int kGM = 8;                   // M-tiles of accumulators per wavefront (GN N-tiles: 4, or 5 in the wide variant)
+constexpr int kGemmNT = 8, kGemmWideNT = 10;     // N-tiles per workgroup (two wavefronts side by side)
 constexpr int kGemmAhead = 3;           // contraction blocks on their way from memory
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global load
@@ -478,11 +472,18 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs &a, const v4i (&acc
     }
 }
 
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) gemm8_kernel(const GemmArgs a) {
+// One workgroup of the product: 64 tokens x 32*GN columns.  GN = 4 is the general shape (two workgroups per
+// compute unit); GN = 5 needs the whole register file of a SIMD for one wavefront and is used where it turns a
+// grid of 1.25 workgroups per compute unit into exactly one (2560 columns: 16 column blocks instead of 20).
+template <int GN>
+__device__ __forceinline__ void gemm8_body(const GemmArgs a) {
     // Both operands of a contraction block are fetched once per workgroup (registers, kGemmAhead
     // blocks ahead), parked in LDS (two buffers, one barrier per block) and read from there by the
     // two wavefronts that need each fragment.
-    __shared__ v4i frag[2][kGemmFrags][64];
+    constexpr int kGN = GN, kNT = 2 * GN;
+    constexpr int kGemmFrags = 16 + kNT;                // fragments of one contraction block: 16 M-tiles of digits, kNT N-tiles of weights
+    constexpr int kGemmLoads = (kGemmFrags + 3) / 4;    // per thread and contraction block (wave w fetches fragments w, w + 4, ...)
+    __shared__ v4i frag[2][4 * kGemmLoads][64];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave & 1, wn = wave >> 1;
@@ -502,7 +503,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     bz -= mat * a.split;
     const signed char *dig = mat == 0 ? a.dig[0] : mat == 1 ? a.dig[1] : a.dig[2];
     const uint8_t *w16 = mat == 0 ? a.w16[0] : mat == 1 ? a.w16[1] : a.w16[2];
-    const int mt0 = by * 16 + wm * kGM, nt0 = bx * kGemmNT + wn * kGN;
+    const int mt0 = by * 16 + wm * kGM, nt0 = bx * kNT + wn * kGN;
     const int kb0 = bz * a.kb_per_split;
     int kb1 = kb0 + a.kb_per_split;
     if (kb1 > a.KB) kb1 = a.KB;
@@ -518,7 +519,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
             if (mt >= a.MT) mt = a.MT - 1;              // clamped: loads stay unconditional, results are dropped
             src[i] = reinterpret_cast<const v4i *>(dig + ((size_t)mt * a.KB + kb0) * 1024) + lane;
         } else {
-            int nt = bx * kGemmNT + (f - 16);
+            int nt = bx * kNT + (f - 16 < kNT ? f - 16 : 0);   // (slots past the last fragment: a copy nobody reads)
             if (nt >= a.NT) nt = a.NT - 1;
             src[i] = reinterpret_cast<const v4i *>(w16 + ((size_t)nt * a.KB + kb0) * 1024) + lane;
         }
@@ -532,45 +533,67 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     // the blocks in flight live in three separately named register sets: an array indexed by the
     // stage would be indexed dynamically once the loop is rotated, and end up in scratch memory
     static_assert(kGemmAhead == 3, "three named stages below");
-    static_assert(kGemmLoads == 6 || kGemmLoads == 5, "named members below");
-    struct Fly { v4i v0, v1, v2, v3, v4, v5; };           // named members, not an array: they must stay registers
+    static_assert(kGemmLoads == 6 || kGemmLoads == 7, "named members below");
+    struct Fly { v4i v0, v1, v2, v3, v4, v5, v6; };       // named members, not an array: they must stay registers
     Fly fly0, fly1, fly2;
 #define RWKV_GEMM_FETCH(F, K)                                                                        \
     do {                                                                                             \
         const size_t o_ = (size_t)((K) < nk ? (K) : nk - 1) * 64; /* past the end: the last block again (unused) */ \
-        F.v0 = src[0][o_]; F.v1 = src[1][o_]; F.v2 = src[2][o_]; F.v3 = src[3][o_]; F.v4 = src[4][o_]; if (kGemmLoads > 5) F.v5 = src[kGemmLoads - 1][o_]; \
+        F.v0 = src[0][o_]; F.v1 = src[1][o_]; F.v2 = src[2][o_]; F.v3 = src[3][o_]; F.v4 = src[4][o_]; F.v5 = src[5][o_]; \
+        if (kGemmLoads > 6) F.v6 = src[kGemmLoads - 1][o_];                                          \
     } while (0)
-#define RWKV_GEMM_STEP(F, K)                                                                         \
+#define RWKV_GEMM_PARK(F, B)                                                                         \
+    do {                                                                                             \
+        frag[B][wave][lane] = F.v0; frag[B][wave + 4][lane] = F.v1; frag[B][wave + 8][lane] = F.v2;  \
+        frag[B][wave + 12][lane] = F.v3; frag[B][wave + 16][lane] = F.v4; frag[B][wave + 20][lane] = F.v5; \
+        if (kGemmLoads > 6) frag[B][wave + 4 * (kGemmLoads - 1)][lane] = F.v6;                       \
+    } while (0)
+    // Step K multiplies block K out of buffer K & 1.  The barrier at its top says that block K is parked and
+    // that every wavefront is done with block K - 1, whose buffer is then free: the NEXT block (registers FN,
+    // fetched kGemmAhead steps ago) is parked there right after the first operand reads, so its LDS writes
+    // run under this step's matrix instructions instead of standing between two steps.
+#define RWKV_GEMM_STEP(FN, K)                                                                        \
     {                                                                                                \
         const int buf_ = (K) & 1;                                                                    \
-        frag[buf_][wave][lane] = F.v0; frag[buf_][wave + 4][lane] = F.v1; frag[buf_][wave + 8][lane] = F.v2;     \
-        frag[buf_][wave + 12][lane] = F.v3; frag[buf_][wave + 16][lane] = F.v4; if (kGemmLoads > 5) frag[buf_][wave + 4 * (kGemmLoads - 1)][lane] = F.v5; \
-        RWKV_GEMM_FETCH(F, (K) + kGemmAhead);                                                        \
         lds_barrier();                                                                               \
         v4i Bv_[kGN];                                                                                \
         _Pragma("unroll") for (int j = 0; j < kGN; ++j) {                                            \
             Bv_[j] = frag[buf_][16 + wn * kGN + j][lane];                                            \
         }                                                                                            \
+        v4i Av_ = frag[buf_][wm * kGM][lane];                                                        \
+        RWKV_GEMM_PARK(FN, buf_ ^ 1);                                                                \
+        RWKV_GEMM_FETCH(FN, (K) + 1 + kGemmAhead);                                                   \
         _Pragma("unroll") for (int i = 0; i < kGM; ++i) {                                            \
-            const v4i Av_ = frag[buf_][wm * kGM + i][lane];                                          \
+            const v4i An_ = frag[buf_][wm * kGM + (i + 1 < kGM ? i + 1 : i)][lane];                  \
             _Pragma("unroll") for (int j = 0; j < kGN; ++j)                                          \
                 acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Av_, Bv_[j], acc[i][j], 0, 0, 0);  \
+            Av_ = An_;                                                                               \
         }                                                                                            \
     }
     RWKV_GEMM_FETCH(fly0, 0); RWKV_GEMM_FETCH(fly1, 1); RWKV_GEMM_FETCH(fly2, 2);
+    RWKV_GEMM_PARK(fly0, 0);
+    RWKV_GEMM_FETCH(fly0, kGemmAhead);
     // whole rounds run without a branch between the steps: the compiler then counts exactly which loads
     // a step has to wait for (with a test per step it drains every load in flight once per round)
     int k0 = 0;
     for (; k0 + kGemmAhead <= nk; k0 += kGemmAhead) {
-        RWKV_GEMM_STEP(fly0, k0)
-        RWKV_GEMM_STEP(fly1, k0 + 1)
-        RWKV_GEMM_STEP(fly2, k0 + 2)
+        RWKV_GEMM_STEP(fly1, k0)
+        RWKV_GEMM_STEP(fly2, k0 + 1)
+        RWKV_GEMM_STEP(fly0, k0 + 2)
     }
-    if (k0 < nk) RWKV_GEMM_STEP(fly0, k0)
-    if (k0 + 1 < nk) RWKV_GEMM_STEP(fly1, k0 + 1)
+    if (k0 < nk) RWKV_GEMM_STEP(fly1, k0)
+    if (k0 + 1 < nk) RWKV_GEMM_STEP(fly2, k0 + 1)
 #undef RWKV_GEMM_STEP
+#undef RWKV_GEMM_PARK
 #undef RWKV_GEMM_FETCH
     gemm_epilogue<kGM, kGN>(a, acc, mt0, nt0, mat, bz, lane);
+}
+
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) gemm8_kernel(const GemmArgs a) {
+    gemm8_body<4>(a);
+}
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) gemm8_wide_kernel(const GemmArgs a) {
+    gemm8_body<5>(a);
 }
 
 // ---------------------------------------------------------------------------
@@ -631,39 +654,49 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         const size_t o_ = (size_t)((K) < nk ? (K) : nk - 1) * 64; /* past the end: the last block again (unused) */ \
         F.v0 = src[0][o_]; F.v1 = src[1][o_]; F.v2 = src[2][o_]; F.v3 = src[3][o_];                  \
     } while (0)
-#define RWKV_SKINNY_STEP(F, K)                                                                       \
+#define RWKV_SKINNY_PARK(F, B)                                                                       \
+    do {                                                                                             \
+        frag[B][wave][lane] = F.v0; frag[B][wave + 4][lane] = F.v1;                                  \
+        frag[B][wave + 8][lane] = F.v2; frag[B][wave + 12][lane] = F.v3;                             \
+    } while (0)
+    // (same step as gemm8_kernel: the next block is parked under this block's matrix instructions)
+#define RWKV_SKINNY_STEP(FN, K)                                                                      \
     {                                                                                                \
         const int buf_ = (K) & 1;                                                                    \
-        frag[buf_][wave][lane] = F.v0; frag[buf_][wave + 4][lane] = F.v1;                            \
-        frag[buf_][wave + 8][lane] = F.v2; frag[buf_][wave + 12][lane] = F.v3;                       \
-        RWKV_SKINNY_FETCH(F, (K) + kSkinnyAhead);                                                    \
         lds_barrier();                                                                               \
         v4i Bv_[kSkinnyGN];                                                                          \
         _Pragma("unroll") for (int j = 0; j < kSkinnyGN; ++j)                                        \
             Bv_[j] = frag[buf_][kSkinnyMT + wave * kSkinnyGN + j][lane];                             \
+        v4i Av_ = frag[buf_][0][lane];                                                               \
+        RWKV_SKINNY_PARK(FN, buf_ ^ 1);                                                              \
+        RWKV_SKINNY_FETCH(FN, (K) + 1 + kSkinnyAhead);                                               \
         _Pragma("unroll") for (int i = 0; i < kSkinnyMT; ++i) {                                      \
-            const v4i Av_ = frag[buf_][i][lane];                                                     \
+            const v4i An_ = frag[buf_][i + 1 < kSkinnyMT ? i + 1 : i][lane];                         \
             _Pragma("unroll") for (int j = 0; j < kSkinnyGN; ++j)                                    \
                 acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Av_, Bv_[j], acc[i][j], 0, 0, 0);  \
+            Av_ = An_;                                                                               \
         }                                                                                            \
     }
     RWKV_SKINNY_FETCH(fly0, 0); RWKV_SKINNY_FETCH(fly1, 1); RWKV_SKINNY_FETCH(fly2, 2);
     RWKV_SKINNY_FETCH(fly3, 3); RWKV_SKINNY_FETCH(fly4, 4); RWKV_SKINNY_FETCH(fly5, 5);
+    RWKV_SKINNY_PARK(fly0, 0);
+    RWKV_SKINNY_FETCH(fly0, kSkinnyAhead);
     int k0 = 0;
     for (; k0 + kSkinnyAhead <= nk; k0 += kSkinnyAhead) {      // whole rounds: no branch between the steps
-        RWKV_SKINNY_STEP(fly0, k0)
-        RWKV_SKINNY_STEP(fly1, k0 + 1)
-        RWKV_SKINNY_STEP(fly2, k0 + 2)
-        RWKV_SKINNY_STEP(fly3, k0 + 3)
-        RWKV_SKINNY_STEP(fly4, k0 + 4)
-        RWKV_SKINNY_STEP(fly5, k0 + 5)
+        RWKV_SKINNY_STEP(fly1, k0)
+        RWKV_SKINNY_STEP(fly2, k0 + 1)
+        RWKV_SKINNY_STEP(fly3, k0 + 2)
+        RWKV_SKINNY_STEP(fly4, k0 + 3)
+        RWKV_SKINNY_STEP(fly5, k0 + 4)
+        RWKV_SKINNY_STEP(fly0, k0 + 5)
     }
-    if (k0 < nk) RWKV_SKINNY_STEP(fly0, k0)
-    if (k0 + 1 < nk) RWKV_SKINNY_STEP(fly1, k0 + 1)
-    if (k0 + 2 < nk) RWKV_SKINNY_STEP(fly2, k0 + 2)
-    if (k0 + 3 < nk) RWKV_SKINNY_STEP(fly3, k0 + 3)
-    if (k0 + 4 < nk) RWKV_SKINNY_STEP(fly4, k0 + 4)
+    if (k0 < nk) RWKV_SKINNY_STEP(fly1, k0)
+    if (k0 + 1 < nk) RWKV_SKINNY_STEP(fly2, k0 + 1)
+    if (k0 + 2 < nk) RWKV_SKINNY_STEP(fly3, k0 + 2)
+    if (k0 + 3 < nk) RWKV_SKINNY_STEP(fly4, k0 + 3)
+    if (k0 + 4 < nk) RWKV_SKINNY_STEP(fly5, k0 + 4)
 #undef RWKV_SKINNY_STEP
+#undef RWKV_SKINNY_PARK
 #undef RWKV_SKINNY_FETCH
     gemm_epilogue<kSkinnyMT, kSkinnyGN>(a, acc, 0, nt0, mat, bz, lane);
 }
@@ -796,6 +829,10 @@ __global__ void __launch_bounds__(64) wkv_chunk_replay_kernel(const WkvRowsArgs 
 size_t rows_dig_bytes(int64_t R, int64_t K) { return (size_t)(ceil_div(R, 4) * (K / 64) * 1024); }
 size_t rows_wkv_scratch_bytes(int64_t R, int64_t C) { return (size_t)(ceil_div(R, kWkvChunk) * 3 * C * 8); }
 constexpr int kMaxSplit = 8;
+#ifndef RWKV_GEMM_WIDE_NUM
+#define RWKV_GEMM_WIDE_NUM 10
+#define RWKV_GEMM_WIDE_DEN 9
+#endif
 #ifndef RWKV_GEMM_FILL
 #define RWKV_GEMM_FILL 256
 #endif
@@ -882,7 +919,17 @@ int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, i
     g.tot = tot;
     g.MT = (int)ceil_div(R, 4); g.NT = (int)ceil_div(N, 16); g.KB = (int)(K / 64); g.ldd = g.NT * 16;
     const bool skinny = g.MT <= kSkinnyMT;              // few rows: the weight-streaming variant
-    const int gx = (int)ceil_div(g.NT, skinny ? kSkinnyNT : kGemmNT), gy = (int)ceil_div(g.MT, 16);
+    const int gy = (int)ceil_div(g.MT, 16);
+    bool wide = false;
+    if (!skinny) {
+        // Rounds of workgroups on 256 compute units, in matrix instructions per step: two general workgroups
+        // share a compute unit (2 x 32), a wide one has it alone (40).
+        const int w4 = (int)ceil_div(g.NT, kGemmNT) * gy * n, w5 = (int)ceil_div(g.NT, kGemmWideNT) * gy * n;
+        const int rem = w4 % 512;
+        const int cost4 = (w4 / 512) * 64 + (rem == 0 ? 0 : rem <= 256 ? 32 : 64), cost5 = (int)ceil_div(w5, 256) * 40;
+        wide = w4 >= 256 && RWKV_GEMM_WIDE_NUM * cost5 < RWKV_GEMM_WIDE_DEN * cost4;
+    }
+    const int gx = (int)ceil_div(g.NT, skinny ? kSkinnyNT : wide ? kGemmWideNT : kGemmNT);
     // Split the contraction until the grid has a few workgroups per compute unit.
     int split = 1;
     while (gx * gy * n * split < kGemmFillWgs && g.KB / (split * 2) >= 8 && split < kMaxSplit) split *= 2;
@@ -894,6 +941,7 @@ int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, i
     g.tail = split > 1 ? -1 : op; g.R = (int)R; g.N = (int)N; g.gate = gate;
     const dim3 grid((unsigned)(kXcds * g.per_xcd * (g.by_rows ? gx : gy) * g.gz));
     if (skinny) hipLaunchKernelGGL(gemm8_skinny_kernel, grid, dim3(256), 0, st, g);
+    else if (wide) hipLaunchKernelGGL(gemm8_wide_kernel, grid, dim3(256), 0, st, g);
     else hipLaunchKernelGGL(gemm8_kernel, grid, dim3(256), 0, st, g);
     RWKV_CHECK_LAUNCH("gemm8_kernel");
     if (split == 1) return RWKV_OK;     // the tail was applied in the product's epilogue

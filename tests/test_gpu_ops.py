@@ -252,8 +252,10 @@ def test_pack_m16_round_trip(ops):
         assert torch.equal(p[lane].view(torch.int8), want)
 
 
+# the last two run the 160-column workgroup variant (320 general workgroups would make 1.25 per compute unit),
+# with ragged rows, ragged columns and a contraction that ends inside a round of the pipeline
 @pytest.mark.parametrize("T,K,N", [(1, 64, 16), (5, 256, 100), (64, 2560, 2560), (130, 2560, 10240),
-                                   (33, 10240, 2560), (8, 2560, 50277)])
+                                   (33, 10240, 2560), (8, 2560, 50277), (1000, 192, 2560), (1024, 320, 2500)])
 def test_gemm8_matches_fp64_dense(ops, T, K, N):
     """Prompt GEMM (matmul.py:56-57 without its bfloat16 rounding) against the float64 dense product."""
     g = torch.Generator().manual_seed(T * 7 + K + N)
@@ -278,8 +280,9 @@ def test_gemm8_rows_do_not_depend_on_batching(ops):
     K, N = 2560, 2560
     w = torch.randn(N, K, generator=g) * 0.02
     codes, rng, off = O.quantize_matrix(w)
-    x = torch.randn(300, K, generator=g, dtype=torch.float64).cuda()
+    x = torch.randn(1024, K, generator=g, dtype=torch.float64).cuda()
     p16 = ops.pack_m16(codes.cuda())
-    full = ops.gemm8(x, p16, rng.cuda(), off.cuda(), K, N)
-    few = ops.gemm8(x[37:40].contiguous(), p16, rng.cuda(), off.cuda(), K, N)
-    assert torch.equal(full[37:40], few)
+    wide = ops.gemm8(x, p16, rng.cuda(), off.cuda(), K, N)            # 160-column workgroups
+    full = ops.gemm8(x[:300].contiguous(), p16, rng.cuda(), off.cuda(), K, N)    # 128-column workgroups
+    few = ops.gemm8(x[37:40].contiguous(), p16, rng.cuda(), off.cuda(), K, N)    # few-row variant, split contraction
+    assert torch.equal(full[37:40], few) and torch.equal(wide[:300], full)
