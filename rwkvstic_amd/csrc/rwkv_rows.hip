@@ -147,10 +147,10 @@ struct LnQuantArgs {
     double *S[3], *qs[3], *zp[3];
 };
 
-constexpr int kLT = 512, kLW = kLT / 64;    // threads / wavefronts of the LayerNorm kernel
+constexpr int kLnMaxThreads = 512;      // the LayerNorm kernel runs 512 threads per row for few rows, 256 for many
 
-// Sum of N values per thread over the kLT threads (fixed order), broadcast.
-template <int N>
+// Sum of N values per thread over the kLW wavefronts of the workgroup (fixed order), broadcast.
+template <int N, int kLW>
 __device__ __forceinline__ void lsum(double (&v)[N], double *red /*[N*kLW]*/) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
@@ -169,9 +169,9 @@ __device__ __forceinline__ void lsum(double (&v)[N], double *red /*[N*kLW]*/) {
     __syncthreads();
 }
 
-template <int NM, int NSEG>
+template <int NM, int NSEG, int kLT>
 __global__ void __launch_bounds__(kLT) rows_ln_mix_quant_kernel(const LnQuantArgs a) {
-    constexpr int NO = NM > 0 ? NM : 1;
+    constexpr int NO = NM > 0 ? NM : 1, kLW = kLT / 64;
     __shared__ double red[3 * kLW];
     __shared__ float redf[NO * kLW];
     const int t = blockIdx.x, C = a.C, tid = threadIdx.x;
@@ -190,16 +190,18 @@ __global__ void __launch_bounds__(kLT) rows_ln_mix_quant_kernel(const LnQuantArg
                 const double2 p0 = *reinterpret_cast<const double2 *>(pr + c0), p1 = *reinterpret_cast<const double2 *>(pr + c0 + 2);
                 pv[g][0] = p0.x; pv[g][1] = p0.y; pv[g][2] = p1.x; pv[g][3] = p1.y;
             }
-            // the LayerNorm weights travel with the row: nothing is left to fetch between the reductions
+            // few rows: the LayerNorm weights travel with the row, nothing is left to fetch between the
+            // reductions; many rows: fetched where they are used, for fewer registers and more rows in flight
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { s[0] += xv[g][i]; if (NM > 0) s[1] += pv[g][i]; }
+            if (kLT < 512) continue;
             const double2 w0 = *reinterpret_cast<const double2 *>(a.ln_w + c0), w1 = *reinterpret_cast<const double2 *>(a.ln_w + c0 + 2);
             const double2 b0 = *reinterpret_cast<const double2 *>(a.ln_b + c0), b1 = *reinterpret_cast<const double2 *>(a.ln_b + c0 + 2);
             lw[g][0] = w0.x; lw[g][1] = w0.y; lw[g][2] = w1.x; lw[g][3] = w1.y;
             lb[g][0] = b0.x; lb[g][1] = b0.y; lb[g][2] = b1.x; lb[g][3] = b1.y;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) { s[0] += xv[g][i]; if (NM > 0) s[1] += pv[g][i]; }
         }
     }
-    lsum<2>(s, red);
+    lsum<2, kLW>(s, red);
     const double mean = s[0] / (double)C, meanp = s[1] / (double)C;
     double q[2] = {0.0, 0.0};
 #pragma unroll
@@ -213,7 +215,7 @@ __global__ void __launch_bounds__(kLT) rows_ln_mix_quant_kernel(const LnQuantArg
             }
         }
     }
-    lsum<2>(q, red);
+    lsum<2, kLW>(q, red);
     const double sd = sqrt(q[0] / (double)C + 1e-5), sdp = sqrt(q[1] / (double)C + 1e-5);
     float xs[NO][NSEG][4];
     float amax[NO];
@@ -225,6 +227,12 @@ __global__ void __launch_bounds__(kLT) rows_ln_mix_quant_kernel(const LnQuantArg
         const int c0 = 4 * (tid + g * kLT);
         if (c0 < C) {
             double xy[4], prev[4];
+            if (kLT < 512) {
+                const double2 w0 = *reinterpret_cast<const double2 *>(a.ln_w + c0), w1 = *reinterpret_cast<const double2 *>(a.ln_w + c0 + 2);
+                const double2 b0 = *reinterpret_cast<const double2 *>(a.ln_b + c0), b1 = *reinterpret_cast<const double2 *>(a.ln_b + c0 + 2);
+                lw[g][0] = w0.x; lw[g][1] = w0.y; lw[g][2] = w1.x; lw[g][3] = w1.y;
+                lb[g][0] = b0.x; lb[g][1] = b0.y; lb[g][2] = b1.x; lb[g][3] = b1.y;
+            }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 xy[i] = lw[g][i] * ((xv[g][i] - mean) / sd) + lb[g][i];
@@ -264,7 +272,7 @@ __global__ void __launch_bounds__(kLT) rows_ln_mix_quant_kernel(const LnQuantArg
         amax[m] = wmaxf(amax[m]);
         if ((tid & 63) == 0) redf[m * kLW + (tid >> 6)] = amax[m];
     }
-    lsum<NO>(z, red);                      // (its barriers also publish redf)
+    lsum<NO, kLW>(z, red);                      // (its barriers also publish redf)
     double S[NO], invS[NO], qsum[NO];
     const int KB = C >> 6;
 #pragma unroll
@@ -280,7 +288,7 @@ __global__ void __launch_bounds__(kLT) rows_ln_mix_quant_kernel(const LnQuantArg
             if (c0 < C) qsum[m] += emit_quad(xs[m][g], invS[m], c0, t, KB, a.dig[m]);
         }
     }
-    lsum<NO>(qsum, red);
+    lsum<NO, kLW>(qsum, red);
     if (tid == 0) {
 #pragma unroll
         for (int m = 0; m < NO; ++m) { a.S[m][t] = S[m]; a.qs[m][t] = qsum[m]; a.zp[m][t] = z[m]; }
@@ -857,14 +865,14 @@ int rows_embed(hipStream_t st, const int64_t *tokens, int64_t R, int V, int C, c
     return RWKV_OK;
 }
 
-bool rows_ln_width_supported(int64_t C) { return C % 4 == 0 && C <= 3 * 4 * kLT; }
+bool rows_ln_width_supported(int64_t C) { return C % 4 == 0 && C <= 3 * 4 * kLnMaxThreads; }
 
 int rows_ln_mix_quant(hipStream_t st, int n_mix, int64_t R, int C, bool sequence, const double *x, const double *ln_w,
                       const double *ln_b, const double *mu, const double *prev0, double *shift_dst,
                       int64_t prev_stride, const float *const *range, const double *const *offset,
                       const RowsOperand *out) {
     if (C % 64 != 0 || !rows_ln_width_supported(C))
-        return set_error(RWKV_ERR_SIZE, "rows_ln_mix_quant: width %d is not a multiple of 64 up to %d", C, 3 * 4 * kLT);
+        return set_error(RWKV_ERR_SIZE, "rows_ln_mix_quant: width %d is not a multiple of 64 up to %d", C, 3 * 4 * kLnMaxThreads);
     LnQuantArgs a;
     a.C = C; a.R = (int)R; a.sequence = sequence ? 1 : 0; a.x = x; a.ln_w = ln_w; a.ln_b = ln_b; a.mu = mu;
     a.prev0 = prev0; a.shift_dst = shift_dst; a.prev_stride = prev_stride;
@@ -874,12 +882,17 @@ int rows_ln_mix_quant(hipStream_t st, int n_mix, int64_t R, int C, bool sequence
         a.range[m] = range[k]; a.offset[m] = offset[k];
         a.dig[m] = out[k].dig; a.S[m] = out[k].S; a.qs[m] = out[k].qs; a.zp[m] = out[k].zp;
     }
-    const dim3 grid((unsigned)R), block(kLT);
-    const bool small = C <= 2 * 4 * kLT;
+    // few rows: 512 threads per row shorten the chain of dependent steps; many rows: 256 threads with twice
+    // the channels each keep more rows resident per compute unit
+    const bool many = R >= 128;
+    const dim3 grid((unsigned)R), block(many ? 256 : 512);
+    const bool small = many ? C <= 3 * 4 * 256 : C <= 2 * 4 * 512;
 #define RWKV_LNQ(NM)                                                                                  \
     do {                                                                                              \
-        if (small) hipLaunchKernelGGL((rows_ln_mix_quant_kernel<NM, 2>), grid, block, 0, st, a);      \
-        else hipLaunchKernelGGL((rows_ln_mix_quant_kernel<NM, 3>), grid, block, 0, st, a);            \
+        if (many && small) hipLaunchKernelGGL((rows_ln_mix_quant_kernel<NM, 3, 256>), grid, block, 0, st, a);   \
+        else if (many) hipLaunchKernelGGL((rows_ln_mix_quant_kernel<NM, 6, 256>), grid, block, 0, st, a);       \
+        else if (small) hipLaunchKernelGGL((rows_ln_mix_quant_kernel<NM, 2, 512>), grid, block, 0, st, a);      \
+        else hipLaunchKernelGGL((rows_ln_mix_quant_kernel<NM, 3, 512>), grid, block, 0, st, a);                 \
     } while (0)
     switch (n_mix) {
         case 0: RWKV_LNQ(0); break;
