@@ -558,24 +558,42 @@ __device__ __forceinline__ void gemm8_body(const GemmArgs a) {
     } while (0)
     // Step K multiplies block K out of buffer K & 1.  The barrier at its top says that block K is parked and
     // that every wavefront is done with block K - 1, whose buffer is then free: the NEXT block (registers FN,
-    // fetched kGemmAhead steps ago) is parked there right after the first operand reads, so its LDS writes
-    // run under this step's matrix instructions instead of standing between two steps.
+    // fetched kGemmAhead steps ago) is parked there fragment by fragment between this step's groups of matrix
+    // instructions, each register set refilled as soon as it is parked, so that LDS writes, global loads and
+    // LDS reads alternate in small pieces instead of queueing up in front of the first operand reads.
+#define RWKV_GEMM_MOVE(FN, I, V, B, O)                                                               \
+    if ((I) < kGemmLoads) { frag[B][wave + 4 * (I)][lane] = FN.V; FN.V = src[(I) < kGemmLoads ? (I) : 0][O]; }
 #define RWKV_GEMM_STEP(FN, K)                                                                        \
     {                                                                                                \
         const int buf_ = (K) & 1;                                                                    \
+        const size_t on_ = (size_t)((K) + 1 + kGemmAhead < nk ? (K) + 1 + kGemmAhead : nk - 1) * 64; \
         lds_barrier();                                                                               \
         v4i Bv_[kGN];                                                                                \
         _Pragma("unroll") for (int j = 0; j < kGN; ++j) {                                            \
             Bv_[j] = frag[buf_][16 + wn * kGN + j][lane];                                            \
         }                                                                                            \
         v4i Av_ = frag[buf_][wm * kGM][lane];                                                        \
-        RWKV_GEMM_PARK(FN, buf_ ^ 1);                                                                \
-        RWKV_GEMM_FETCH(FN, (K) + 1 + kGemmAhead);                                                   \
         _Pragma("unroll") for (int i = 0; i < kGM; ++i) {                                            \
             const v4i An_ = frag[buf_][wm * kGM + (i + 1 < kGM ? i + 1 : i)][lane];                  \
+            if (i == 0) RWKV_GEMM_MOVE(FN, 0, v0, buf_ ^ 1, on_)                                     \
+            if (i == 1) RWKV_GEMM_MOVE(FN, 1, v1, buf_ ^ 1, on_)                                     \
+            if (i == 2) RWKV_GEMM_MOVE(FN, 2, v2, buf_ ^ 1, on_)                                     \
+            if (i == 3) RWKV_GEMM_MOVE(FN, 3, v3, buf_ ^ 1, on_)                                     \
+            if (i == 4) RWKV_GEMM_MOVE(FN, 4, v4, buf_ ^ 1, on_)                                     \
+            if (i == 5) RWKV_GEMM_MOVE(FN, 5, v5, buf_ ^ 1, on_)                                     \
+            if (i == 6) RWKV_GEMM_MOVE(FN, 6, v6, buf_ ^ 1, on_)                                     \
             _Pragma("unroll") for (int j = 0; j < kGN; ++j)                                          \
                 acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Av_, Bv_[j], acc[i][j], 0, 0, 0);  \
             Av_ = An_;                                                                               \
+        }                                                                                            \
+        /* the order the scheduler is asked to keep: first operands, then per group of matrix */     \
+        /* instructions one LDS write, one LDS read and one global load */                          \
+        __builtin_amdgcn_sched_group_barrier(0x100, kGN + 2, 0);                                     \
+        _Pragma("unroll") for (int i = 0; i < kGM; ++i) {                                            \
+            if (i < kGemmLoads) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                   \
+            __builtin_amdgcn_sched_group_barrier(0x008, kGN, 0);                                     \
+            if (i + 2 < kGM) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                      \
+            if (i < kGemmLoads) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                   \
         }                                                                                            \
     }
     RWKV_GEMM_FETCH(fly0, 0); RWKV_GEMM_FETCH(fly1, 1); RWKV_GEMM_FETCH(fly2, 2);
@@ -592,6 +610,7 @@ __device__ __forceinline__ void gemm8_body(const GemmArgs a) {
     if (k0 < nk) RWKV_GEMM_STEP(fly1, k0)
     if (k0 + 1 < nk) RWKV_GEMM_STEP(fly2, k0 + 1)
 #undef RWKV_GEMM_STEP
+#undef RWKV_GEMM_MOVE
 #undef RWKV_GEMM_PARK
 #undef RWKV_GEMM_FETCH
     gemm_epilogue<kGM, kGN>(a, acc, mt0, nt0, mat, bz, lane);
@@ -667,22 +686,35 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         frag[B][wave][lane] = F.v0; frag[B][wave + 4][lane] = F.v1;                                  \
         frag[B][wave + 8][lane] = F.v2; frag[B][wave + 12][lane] = F.v3;                             \
     } while (0)
-    // (same step as gemm8_kernel: the next block is parked under this block's matrix instructions)
+    // (same step as gemm8_body: the next block is parked, and its registers refilled, piece by piece between
+    // this block's groups of matrix instructions)
+#define RWKV_SKINNY_MOVE(FN, I, V, B, O)                                                             \
+    { frag[B][wave + 4 * (I)][lane] = FN.V; FN.V = src[I][O]; }
 #define RWKV_SKINNY_STEP(FN, K)                                                                      \
     {                                                                                                \
         const int buf_ = (K) & 1;                                                                    \
+        const size_t on_ = (size_t)((K) + 1 + kSkinnyAhead < nk ? (K) + 1 + kSkinnyAhead : nk - 1) * 64; \
         lds_barrier();                                                                               \
         v4i Bv_[kSkinnyGN];                                                                          \
         _Pragma("unroll") for (int j = 0; j < kSkinnyGN; ++j)                                        \
             Bv_[j] = frag[buf_][kSkinnyMT + wave * kSkinnyGN + j][lane];                             \
         v4i Av_ = frag[buf_][0][lane];                                                               \
-        RWKV_SKINNY_PARK(FN, buf_ ^ 1);                                                              \
-        RWKV_SKINNY_FETCH(FN, (K) + 1 + kSkinnyAhead);                                               \
         _Pragma("unroll") for (int i = 0; i < kSkinnyMT; ++i) {                                      \
             const v4i An_ = frag[buf_][i + 1 < kSkinnyMT ? i + 1 : i][lane];                         \
+            if (i == 0) RWKV_SKINNY_MOVE(FN, 0, v0, buf_ ^ 1, on_)                                   \
+            if (i == 2) RWKV_SKINNY_MOVE(FN, 1, v1, buf_ ^ 1, on_)                                   \
+            if (i == 4) RWKV_SKINNY_MOVE(FN, 2, v2, buf_ ^ 1, on_)                                   \
+            if (i == 6) RWKV_SKINNY_MOVE(FN, 3, v3, buf_ ^ 1, on_)                                   \
             _Pragma("unroll") for (int j = 0; j < kSkinnyGN; ++j)                                    \
                 acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Av_, Bv_[j], acc[i][j], 0, 0, 0);  \
             Av_ = An_;                                                                               \
+        }                                                                                            \
+        __builtin_amdgcn_sched_group_barrier(0x100, kSkinnyGN + 2, 0);                               \
+        _Pragma("unroll") for (int i = 0; i < kSkinnyMT; ++i) {                                      \
+            if (i % 2 == 0) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                       \
+            __builtin_amdgcn_sched_group_barrier(0x008, kSkinnyGN, 0);                               \
+            if (i + 2 < kSkinnyMT) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                \
+            if (i % 2 == 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                       \
         }                                                                                            \
     }
     RWKV_SKINNY_FETCH(fly0, 0); RWKV_SKINNY_FETCH(fly1, 1); RWKV_SKINNY_FETCH(fly2, 2);
@@ -704,6 +736,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     if (k0 + 3 < nk) RWKV_SKINNY_STEP(fly4, k0 + 3)
     if (k0 + 4 < nk) RWKV_SKINNY_STEP(fly5, k0 + 4)
 #undef RWKV_SKINNY_STEP
+#undef RWKV_SKINNY_MOVE
 #undef RWKV_SKINNY_PARK
 #undef RWKV_SKINNY_FETCH
     gemm_epilogue<kSkinnyMT, kSkinnyGN>(a, acc, 0, nt0, mat, bz, lane);
