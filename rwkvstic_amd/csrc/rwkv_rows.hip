@@ -480,21 +480,22 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs &a, const v4i (&acc
     }
 }
 
-// One workgroup of the product: 64 tokens x 32*GN columns.  GN = 4 is the general shape (two workgroups per
-// compute unit); GN = 5 needs the whole register file of a SIMD for one wavefront and is used where it turns a
-// grid of 1.25 workgroups per compute unit into exactly one (2560 columns: 16 column blocks instead of 20).
-template <int GN>
+// One workgroup of the product: 64 tokens x 32*GN columns, 2*WM wavefronts as WM x 2, each 16/WM M-tiles x GN
+// N-tiles.  <4, 2> is the general shape (4 wavefronts, two workgroups per compute unit); <5, 4> (8 wavefronts
+// of 4 x 5 tiles, one workgroup per compute unit) is used where it turns a grid of 1.25 workgroups per compute
+// unit into exactly one (2560 columns: 16 column blocks instead of 20).
+template <int GN, int WM>
 __device__ __forceinline__ void gemm8_body(const GemmArgs a) {
     // Both operands of a contraction block are fetched once per workgroup (registers, kGemmAhead
     // blocks ahead), parked in LDS (two buffers, one barrier per block) and read from there by the
     // two wavefronts that need each fragment.
-    constexpr int kGN = GN, kNT = 2 * GN;
+    constexpr int kGN = GN, kNT = 2 * GN, kGM = 16 / WM, kNW = 2 * WM;    // (kGM shadows the 4-wavefront constant)
     constexpr int kGemmFrags = 16 + kNT;                // fragments of one contraction block: 16 M-tiles of digits, kNT N-tiles of weights
-    constexpr int kGemmLoads = (kGemmFrags + 3) / 4;    // per thread and contraction block (wave w fetches fragments w, w + 4, ...)
-    __shared__ v4i frag[2][4 * kGemmLoads][64];
+    constexpr int kGemmLoads = (kGemmFrags + kNW - 1) / kNW;    // per thread and contraction block (wave w fetches fragments w, w + kNW, ...)
+    __shared__ v4i frag[2][kNW * kGemmLoads][64];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int wm = wave & 1, wn = wave >> 1;
+    const int wm = wave % WM, wn = wave / WM;
     const int xcd = blockIdx.x % kXcds;
     int item = blockIdx.x / kXcds, bx, by, bz;
     if (a.by_rows) {                                    // (split, column block, row slot) of this XCD, row slot fastest
@@ -521,7 +522,7 @@ __device__ __forceinline__ void gemm8_body(const GemmArgs a) {
     const v4i *src[kGemmLoads];
 #pragma unroll
     for (int i = 0; i < kGemmLoads; ++i) {
-        const int f = wave + 4 * i;                     // fragment this thread helps to fetch
+        const int f = wave + kNW * i;                   // fragment this thread helps to fetch
         if (f < 16) {
             int mt = by * 16 + f;
             if (mt >= a.MT) mt = a.MT - 1;              // clamped: loads stay unconditional, results are dropped
@@ -541,20 +542,24 @@ __device__ __forceinline__ void gemm8_body(const GemmArgs a) {
     // the blocks in flight live in three separately named register sets: an array indexed by the
     // stage would be indexed dynamically once the loop is rotated, and end up in scratch memory
     static_assert(kGemmAhead == 3, "three named stages below");
-    static_assert(kGemmLoads == 6 || kGemmLoads == 7, "named members below");
+    static_assert(kGemmLoads >= 4 && kGemmLoads <= 7 && kGemmLoads <= kGM, "named members below, one parked per group of matrix instructions");
     struct Fly { v4i v0, v1, v2, v3, v4, v5, v6; };       // named members, not an array: they must stay registers
     Fly fly0, fly1, fly2;
 #define RWKV_GEMM_FETCH(F, K)                                                                        \
     do {                                                                                             \
         const size_t o_ = (size_t)((K) < nk ? (K) : nk - 1) * 64; /* past the end: the last block again (unused) */ \
-        F.v0 = src[0][o_]; F.v1 = src[1][o_]; F.v2 = src[2][o_]; F.v3 = src[3][o_]; F.v4 = src[4][o_]; F.v5 = src[5][o_]; \
-        if (kGemmLoads > 6) F.v6 = src[kGemmLoads - 1][o_];                                          \
+        F.v0 = src[0][o_]; F.v1 = src[1][o_]; F.v2 = src[2][o_]; F.v3 = src[3][o_];                  \
+        if (kGemmLoads > 4) F.v4 = src[kGemmLoads > 4 ? 4 : 0][o_];                                  \
+        if (kGemmLoads > 5) F.v5 = src[kGemmLoads > 5 ? 5 : 0][o_];                                  \
+        if (kGemmLoads > 6) F.v6 = src[kGemmLoads > 6 ? 6 : 0][o_];                                  \
     } while (0)
 #define RWKV_GEMM_PARK(F, B)                                                                         \
     do {                                                                                             \
-        frag[B][wave][lane] = F.v0; frag[B][wave + 4][lane] = F.v1; frag[B][wave + 8][lane] = F.v2;  \
-        frag[B][wave + 12][lane] = F.v3; frag[B][wave + 16][lane] = F.v4; frag[B][wave + 20][lane] = F.v5; \
-        if (kGemmLoads > 6) frag[B][wave + 4 * (kGemmLoads - 1)][lane] = F.v6;                       \
+        frag[B][wave][lane] = F.v0; frag[B][wave + kNW][lane] = F.v1; frag[B][wave + 2 * kNW][lane] = F.v2; \
+        frag[B][wave + 3 * kNW][lane] = F.v3;                                                        \
+        if (kGemmLoads > 4) frag[B][wave + (kGemmLoads > 4 ? 4 : 0) * kNW][lane] = F.v4;             \
+        if (kGemmLoads > 5) frag[B][wave + (kGemmLoads > 5 ? 5 : 0) * kNW][lane] = F.v5;             \
+        if (kGemmLoads > 6) frag[B][wave + (kGemmLoads > 6 ? 6 : 0) * kNW][lane] = F.v6;             \
     } while (0)
     // Step K multiplies block K out of buffer K & 1.  The barrier at its top says that block K is parked and
     // that every wavefront is done with block K - 1, whose buffer is then free: the NEXT block (registers FN,
@@ -562,7 +567,7 @@ __device__ __forceinline__ void gemm8_body(const GemmArgs a) {
     // instructions, each register set refilled as soon as it is parked, so that LDS writes, global loads and
     // LDS reads alternate in small pieces instead of queueing up in front of the first operand reads.
 #define RWKV_GEMM_MOVE(FN, I, V, B, O)                                                               \
-    if ((I) < kGemmLoads) { frag[B][wave + 4 * (I)][lane] = FN.V; FN.V = src[(I) < kGemmLoads ? (I) : 0][O]; }
+    if ((I) < kGemmLoads) { frag[B][wave + kNW * ((I) < kGemmLoads ? (I) : 0)][lane] = FN.V; FN.V = src[(I) < kGemmLoads ? (I) : 0][O]; }
 #define RWKV_GEMM_STEP(FN, K)                                                                        \
     {                                                                                                \
         const int buf_ = (K) & 1;                                                                    \
@@ -572,9 +577,9 @@ __device__ __forceinline__ void gemm8_body(const GemmArgs a) {
         _Pragma("unroll") for (int j = 0; j < kGN; ++j) {                                            \
             Bv_[j] = frag[buf_][16 + wn * kGN + j][lane];                                            \
         }                                                                                            \
-        v4i Av_ = frag[buf_][wm * kGM][lane];                                                        \
+        v4i Av_ = frag[buf_][wm * kGM][lane], Aw_ = frag[buf_][wm * kGM + 1][lane];                  \
         _Pragma("unroll") for (int i = 0; i < kGM; ++i) {                                            \
-            const v4i An_ = frag[buf_][wm * kGM + (i + 1 < kGM ? i + 1 : i)][lane];                  \
+            const v4i An_ = frag[buf_][wm * kGM + (i + 2 < kGM ? i + 2 : i)][lane];   /* two groups ahead */ \
             if (i == 0) RWKV_GEMM_MOVE(FN, 0, v0, buf_ ^ 1, on_)                                     \
             if (i == 1) RWKV_GEMM_MOVE(FN, 1, v1, buf_ ^ 1, on_)                                     \
             if (i == 2) RWKV_GEMM_MOVE(FN, 2, v2, buf_ ^ 1, on_)                                     \
@@ -584,15 +589,15 @@ __device__ __forceinline__ void gemm8_body(const GemmArgs a) {
             if (i == 6) RWKV_GEMM_MOVE(FN, 6, v6, buf_ ^ 1, on_)                                     \
             _Pragma("unroll") for (int j = 0; j < kGN; ++j)                                          \
                 acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Av_, Bv_[j], acc[i][j], 0, 0, 0);  \
-            Av_ = An_;                                                                               \
+            Av_ = Aw_; Aw_ = An_;                                                                    \
         }                                                                                            \
         /* the order the scheduler is asked to keep: first operands, then per group of matrix */     \
         /* instructions one LDS write, one LDS read and one global load */                          \
-        __builtin_amdgcn_sched_group_barrier(0x100, kGN + 2, 0);                                     \
+        __builtin_amdgcn_sched_group_barrier(0x100, kGN + 3, 0);                                     \
         _Pragma("unroll") for (int i = 0; i < kGM; ++i) {                                            \
             if (i < kGemmLoads) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                   \
             __builtin_amdgcn_sched_group_barrier(0x008, kGN, 0);                                     \
-            if (i + 2 < kGM) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                      \
+            if (i + 3 < kGM) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                      \
             if (i < kGemmLoads) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                   \
         }                                                                                            \
     }
@@ -617,10 +622,10 @@ __device__ __forceinline__ void gemm8_body(const GemmArgs a) {
 }
 
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) gemm8_kernel(const GemmArgs a) {
-    gemm8_body<4>(a);
+    gemm8_body<4, 2>(a);
 }
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) gemm8_wide_kernel(const GemmArgs a) {
-    gemm8_body<5>(a);
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) gemm8_wide_kernel(const GemmArgs a) {
+    gemm8_body<5, 4>(a);
 }
 
 // ---------------------------------------------------------------------------
@@ -987,7 +992,7 @@ int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, i
     g.tail = split > 1 ? -1 : op; g.R = (int)R; g.N = (int)N; g.gate = gate;
     const dim3 grid((unsigned)(kXcds * g.per_xcd * (g.by_rows ? gx : gy) * g.gz));
     if (skinny) hipLaunchKernelGGL(gemm8_skinny_kernel, grid, dim3(256), 0, st, g);
-    else if (wide) hipLaunchKernelGGL(gemm8_wide_kernel, grid, dim3(256), 0, st, g);
+    else if (wide) hipLaunchKernelGGL(gemm8_wide_kernel, grid, dim3(512), 0, st, g);
     else hipLaunchKernelGGL(gemm8_kernel, grid, dim3(256), 0, st, g);
     RWKV_CHECK_LAUNCH("gemm8_kernel");
     if (split == 1) return RWKV_OK;     // the tail was applied in the product's epilogue
