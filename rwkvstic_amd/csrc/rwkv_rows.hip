@@ -308,8 +308,9 @@ struct QuantArgs {
     double *S, *qs, *zp;        // [R]
 };
 
-constexpr int kQuantSeg = 5;        // 16-element segments a thread keeps in registers (rows up to 80 * kRT = 20480 long in one read)
-
+// kQuantSeg: 16-element segments a thread keeps in registers (rows up to 16 * kRT * kQuantSeg long in one
+// read): 3 covers 12288 with registers to spare for four workgroups per compute unit, 5 covers 20480.
+template <int kQuantSeg>
 __global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
     __shared__ double red[2 * kRW];
     __shared__ float redf[kRW];
@@ -399,6 +400,49 @@ __global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
     }
     rsum<1>(qsum, red);
     if (threadIdx.x == 0) { a.S[t] = S; a.qs[t] = qsum[0]; a.zp[t] = z[0]; }
+}
+
+// The same quantiser with a thread owning groups of four values (NSEG of them, 4 * kRT * NSEG values per row in
+// one read): every thread of the workgroup has work whatever the row length, and few registers are held.
+template <int NSEG>
+__global__ void __launch_bounds__(kRT) rows_quant4_kernel(const QuantArgs a) {
+    __shared__ double red[2 * kRW];
+    __shared__ float redf[kRW];
+    const int t = blockIdx.x, K = a.K, tid = threadIdx.x;
+    const double *row = a.in + (size_t)t * K;
+    float xs[NSEG][4];
+    float amax = 0.f;
+    double z[1] = {0.0};
+#pragma unroll
+    for (int g = 0; g < NSEG; ++g) {
+        const int c0 = 4 * (tid + g * kRT);
+        if (c0 < K) {
+            const double2 v0 = *reinterpret_cast<const double2 *>(row + c0), v1 = *reinterpret_cast<const double2 *>(row + c0 + 2);
+            const float4 r = *reinterpret_cast<const float4 *>(a.range + c0);
+            const double2 o0 = *reinterpret_cast<const double2 *>(a.offset + c0), o1 = *reinterpret_cast<const double2 *>(a.offset + c0 + 2);
+            xs[g][0] = (float)(v0.x * (double)r.x); xs[g][1] = (float)(v0.y * (double)r.y);
+            xs[g][2] = (float)(v1.x * (double)r.z); xs[g][3] = (float)(v1.y * (double)r.w);
+            amax = fmaxf(fmaxf(amax, fmaxf(fabsf(xs[g][0]), fabsf(xs[g][1]))), fmaxf(fabsf(xs[g][2]), fabsf(xs[g][3])));
+            z[0] += v0.x * o0.x; z[0] += v0.y * o0.y; z[0] += v1.x * o1.x; z[0] += v1.y * o1.y;
+        }
+    }
+    amax = wmaxf(amax);
+    if ((tid & 63) == 0) redf[tid >> 6] = amax;
+    rsum<1>(z, red);                       // (its barriers also publish redf)
+    amax = redf[0];
+#pragma unroll
+    for (int w = 1; w < kRW; ++w) amax = fmaxf(amax, redf[w]);
+    double S, invS;
+    row_scale(amax, S, invS);
+    const int KB = K >> 6;
+    double qsum[1] = {0.0};
+#pragma unroll
+    for (int g = 0; g < NSEG; ++g) {
+        const int c0 = 4 * (tid + g * kRT);
+        if (c0 < K) qsum[0] += emit_quad(xs[g], invS, c0, t, KB, a.dig);
+    }
+    rsum<1>(qsum, red);
+    if (tid == 0) { a.S[t] = S; a.qs[t] = qsum[0]; a.zp[t] = z[0]; }
 }
 
 // ---------------------------------------------------------------------------
@@ -949,7 +993,12 @@ int rows_quant(hipStream_t st, int64_t R, int64_t K, const double *in, const flo
                                       (long long)K);
     QuantArgs q;
     q.K = (int)K; q.in = in; q.range = range; q.offset = offset; q.dig = out.dig; q.S = out.S; q.qs = out.qs; q.zp = out.zp;
-    hipLaunchKernelGGL(rows_quant_kernel, dim3((unsigned)R), dim3(kRT), 0, st, q);
+    const dim3 grid((unsigned)R), block(kRT);
+    if (K <= 3 * 4 * kRT) hipLaunchKernelGGL(rows_quant4_kernel<3>, grid, block, 0, st, q);
+    else if (K <= 6 * 4 * kRT) hipLaunchKernelGGL(rows_quant4_kernel<6>, grid, block, 0, st, q);
+    else if (K <= 10 * 4 * kRT) hipLaunchKernelGGL(rows_quant4_kernel<10>, grid, block, 0, st, q);
+    else if (K <= 20 * 4 * kRT) hipLaunchKernelGGL(rows_quant4_kernel<20>, grid, block, 0, st, q);
+    else hipLaunchKernelGGL(rows_quant_kernel<3>, grid, block, 0, st, q);      // any length: a second read past 12288
     RWKV_CHECK_LAUNCH("rows_quant_kernel");
     return RWKV_OK;
 }
