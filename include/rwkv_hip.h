@@ -228,7 +228,11 @@ size_t rwkv_model_workspace_bytes(const rwkv_model *m, int64_t max_tokens);
  * float64 [L, 5, C] on the device, rows (att shift, ffn shift, aa, bb, pp),
  * updated in place.  WKV rows hold the max-shifted triple (see rwkv_wkv_f32);
  * the reference's empty state (0, 0, 0, 0, -1e30) is valid as is.
- * logits: float64 [V].  T == 1 takes the matvec path, T > 1 the GEMM path. */
+ * logits: float64 [V].  Path: T >= 4 with the M16 layout of every matrix and
+ * n_embd, n_ffn multiples of 64 takes the many-row (GEMM) kernels; fewer tokens
+ * go one at a time through the persistent single-token kernel where
+ * rwkv_model_has_fused_step, else as one-row prompts through the many-row
+ * kernels, and only without the M16 layout as one launch per phase. */
 int rwkv_model_forward(rwkv_model *m, rwkv_stream_t stream,
                        const int64_t *tokens, int64_t T,
                        double *state, double *logits,
