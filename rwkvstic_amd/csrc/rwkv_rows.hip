@@ -860,6 +860,11 @@ __global__ void __launch_bounds__(64) wkv_rows_kernel(const WkvRowsArgs a) {
 // replays its steps from that state, in parallel.  Same sums as the serial order up to float64 rounding.
 constexpr int kWkvChunk = 32;
 
+// The kernels read their inputs kWkvGroup steps ahead of the serial recurrence (registers, two groups): a
+// thread that fetched each step's k and v when it needed them would wait out a memory round trip per step.
+constexpr int kWkvGroup = 8;
+static_assert(kWkvChunk % kWkvGroup == 0, "whole groups");
+
 __global__ void __launch_bounds__(64) wkv_chunk_local_kernel(const WkvRowsArgs a, double *scr) {
     const int c = blockIdx.x * 64 + threadIdx.x, j = blockIdx.y;
     if (c >= a.C) return;
@@ -867,9 +872,23 @@ __global__ void __launch_bounds__(64) wkv_chunk_local_kernel(const WkvRowsArgs a
     const double w = a.w[c], u = a.u[c];
     const int t0 = j * kWkvChunk, t1 = min(t0 + kWkvChunk, a.R);
     double aa = 0.0, bb = 0.0, pp = -1e30;
-    for (int t = t0; t < t1; ++t) {
-        const size_t i = (size_t)t * C + c;
-        (void)wkv_step<double>(w, u, a.k[i], a.v[i], aa, bb, pp);
+    double kc[kWkvGroup], vc[kWkvGroup], kn[kWkvGroup], vn[kWkvGroup];
+#pragma unroll
+    for (int i = 0; i < kWkvGroup; ++i) {
+        const size_t o = (size_t)min(t0 + i, t1 - 1) * C + c;
+        kc[i] = a.k[o]; vc[i] = a.v[o];
+    }
+    for (int g = t0; g < t1; g += kWkvGroup) {
+#pragma unroll
+        for (int i = 0; i < kWkvGroup; ++i) {
+            const size_t o = (size_t)min(g + kWkvGroup + i, t1 - 1) * C + c;      // past the end: the last row again (unused)
+            kn[i] = a.k[o]; vn[i] = a.v[o];
+        }
+#pragma unroll
+        for (int i = 0; i < kWkvGroup; ++i)
+            if (g + i < t1) (void)wkv_step<double>(w, u, kc[i], vc[i], aa, bb, pp);
+#pragma unroll
+        for (int i = 0; i < kWkvGroup; ++i) { kc[i] = kn[i]; vc[i] = vn[i]; }
     }
     double *o = scr + (size_t)j * 3 * C;
     o[c] = aa; o[C + c] = bb; o[2 * C + c] = pp;
@@ -881,17 +900,35 @@ __global__ void __launch_bounds__(64) wkv_chunk_prefix_kernel(const WkvRowsArgs 
     const int C = a.C;
     const double w = a.w[c];
     double aa = a.state[c], bb = a.state[C + c], pp = a.state[2 * C + c];
-    for (int j = 0; j < n_chunks; ++j) {
-        double *o = scr + (size_t)j * 3 * C;
-        const double la = o[c], lb = o[C + c], lp = o[2 * C + c];
-        o[c] = aa; o[C + c] = bb; o[2 * C + c] = pp;              // incoming state of chunk j
-        const int n = min(kWkvChunk, a.R - j * kWkvChunk);
-        const double s = pp + (double)n * w;
-        const double p = fmax(s, lp);
-        const double f1 = exp(s - p), f2 = exp(lp - p);
-        aa = f1 * aa + f2 * la;
-        bb = f1 * bb + f2 * lb;
-        pp = p;
+    double la[kWkvGroup], lb[kWkvGroup], lp[kWkvGroup], na[kWkvGroup], nb[kWkvGroup], np[kWkvGroup];
+#pragma unroll
+    for (int i = 0; i < kWkvGroup; ++i) {
+        const double *o = scr + (size_t)min(i, n_chunks - 1) * 3 * C;
+        la[i] = o[c]; lb[i] = o[C + c]; lp[i] = o[2 * C + c];
+    }
+    for (int g = 0; g < n_chunks; g += kWkvGroup) {
+#pragma unroll
+        for (int i = 0; i < kWkvGroup; ++i) {
+            const double *o = scr + (size_t)min(g + kWkvGroup + i, n_chunks - 1) * 3 * C;
+            na[i] = o[c]; nb[i] = o[C + c]; np[i] = o[2 * C + c];
+        }
+#pragma unroll
+        for (int i = 0; i < kWkvGroup; ++i) {
+            const int j = g + i;
+            if (j < n_chunks) {
+                double *o = scr + (size_t)j * 3 * C;
+                o[c] = aa; o[C + c] = bb; o[2 * C + c] = pp;              // incoming state of chunk j
+                const int n = min(kWkvChunk, a.R - j * kWkvChunk);
+                const double s = pp + (double)n * w;
+                const double p = fmax(s, lp[i]);
+                const double f1 = exp(s - p), f2 = exp(lp[i] - p);
+                aa = f1 * aa + f2 * la[i];
+                bb = f1 * bb + f2 * lb[i];
+                pp = p;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kWkvGroup; ++i) { la[i] = na[i]; lb[i] = nb[i]; lp[i] = np[i]; }
     }
     a.state[c] = aa; a.state[C + c] = bb; a.state[2 * C + c] = pp;
 }
@@ -904,10 +941,27 @@ __global__ void __launch_bounds__(64) wkv_chunk_replay_kernel(const WkvRowsArgs 
     const int t0 = j * kWkvChunk, t1 = min(t0 + kWkvChunk, a.R);
     const double *in = scr + (size_t)j * 3 * C;
     double aa = in[c], bb = in[C + c], pp = in[2 * C + c];
-    for (int t = t0; t < t1; ++t) {
-        const size_t i = (size_t)t * C + c;
-        const double y = wkv_step<double>(w, u, a.k[i], a.v[i], aa, bb, pp);
-        a.out[i] = y * (1.0 / (1.0 + exp(-a.r[i])));
+    double kc[kWkvGroup], vc[kWkvGroup], rc[kWkvGroup], kn[kWkvGroup], vn[kWkvGroup], rn[kWkvGroup];
+#pragma unroll
+    for (int i = 0; i < kWkvGroup; ++i) {
+        const size_t o = (size_t)min(t0 + i, t1 - 1) * C + c;
+        kc[i] = a.k[o]; vc[i] = a.v[o]; rc[i] = a.r[o];
+    }
+    for (int g = t0; g < t1; g += kWkvGroup) {
+#pragma unroll
+        for (int i = 0; i < kWkvGroup; ++i) {
+            const size_t o = (size_t)min(g + kWkvGroup + i, t1 - 1) * C + c;
+            kn[i] = a.k[o]; vn[i] = a.v[o]; rn[i] = a.r[o];
+        }
+#pragma unroll
+        for (int i = 0; i < kWkvGroup; ++i) {
+            if (g + i < t1) {
+                const double y = wkv_step<double>(w, u, kc[i], vc[i], aa, bb, pp);
+                a.out[(size_t)(g + i) * C + c] = y * (1.0 / (1.0 + exp(-rc[i])));
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kWkvGroup; ++i) { kc[i] = kn[i]; vc[i] = vn[i]; rc[i] = rn[i]; }
     }
 }
 
