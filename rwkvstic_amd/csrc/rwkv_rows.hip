@@ -792,6 +792,65 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 }
 
 // ---------------------------------------------------------------------------
+// The same product for at most 8 rows (MT <= 2 M-tiles: a single token of a shape the persistent kernel does
+// not serve, a small batch): pure weight streaming.  No LDS staging and no barrier in the loop: workgroup =
+// one 16-column tile and one part of the contraction, its 4 wavefronts take every fourth block (together
+// they read the tile's blocks in order) and each keeps 8 blocks of weights in flight on its own, so that a
+// slow load holds up one wavefront, not the workgroup.  The digit fragments (L2-resident) are read by every
+// wavefront itself.  One cross-wavefront sum in LDS at the end, then the common epilogue.
+// ---------------------------------------------------------------------------
+constexpr int kVecMT = 2, kVecBlocks = 8;
+
+template <int MT>
+__global__ void __launch_bounds__(256) gemv16_kernel(const GemmArgs a) {
+    __shared__ v4i red[4][MT][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int item = blockIdx.x;
+    const int nt = item % a.NT; item /= a.NT;
+    const int bz = item % a.split, mat = item / a.split;
+    const signed char *dig = mat == 0 ? a.dig[0] : mat == 1 ? a.dig[1] : a.dig[2];
+    const uint8_t *w16 = mat == 0 ? a.w16[0] : mat == 1 ? a.w16[1] : a.w16[2];
+    const int kb0 = bz * a.kb_per_split;
+    int kb1 = kb0 + a.kb_per_split;
+    if (kb1 > a.KB) kb1 = a.KB;
+    const v4i *bsrc = reinterpret_cast<const v4i *>(w16 + (size_t)nt * a.KB * 1024) + lane;
+    const v4i *asrc[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+        asrc[m] = reinterpret_cast<const v4i *>(dig + (size_t)(m < a.MT ? m : a.MT - 1) * a.KB * 1024) + lane;
+    v4i acc[MT][1];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[m][0] = v4i{0, 0, 0, 0};
+    for (int k = kb0 + wave; k < kb1; k += 4 * kVecBlocks) {
+        v4i B[kVecBlocks], A[MT][kVecBlocks];
+#pragma unroll
+        for (int i = 0; i < kVecBlocks; ++i) {
+            const size_t o = (size_t)min(k + 4 * i, a.KB - 1) * 64;       // past the end: a block nobody multiplies
+            B[i] = bsrc[o];
+#pragma unroll
+            for (int m = 0; m < MT; ++m) A[m][i] = asrc[m][o];
+        }
+#pragma unroll
+        for (int i = 0; i < kVecBlocks; ++i) {
+            if (k + 4 * i < kb1) {          // uniform for the wavefront
+#pragma unroll
+                for (int m = 0; m < MT; ++m)
+                    acc[m][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[m][i], B[i], acc[m][0], 0, 0, 0);
+            }
+        }
+    }
+    // digit sums of at most a few hundred blocks: far inside int32
+#pragma unroll
+    for (int m = 0; m < MT; ++m) red[wave][m][lane] = acc[m][0];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[m][0] = red[0][m][lane] + red[1][m][lane] + red[2][m][lane] + red[3][m][lane];
+    gemm_epilogue<MT, 1>(a, acc, 0, nt, mat, bz, lane);
+}
+
+// ---------------------------------------------------------------------------
 // y[t, j] = S_t * tot + 128 * S_t * sum q_t + zp_t, then the phase's element-wise tail.
 // ---------------------------------------------------------------------------
 struct FinishArgs {
@@ -984,9 +1043,13 @@ constexpr int kGemmFillWgs = RWKV_GEMM_FILL;   // the contraction is split until
 // Upper bound of the number of contraction splits rows_matmul will choose for R rows and N columns:
 // each split writes its own slice of totals (summed by the tail kernel), so the buffer has that many.
 static int gemm_split_bound(int64_t R, int64_t N) {
-    const int64_t MT = ceil_div(R, 4);
-    const int64_t gx = ceil_div(ceil_div(N, 16), MT <= kSkinnyMT ? kSkinnyNT : kGemmNT), gy = ceil_div(MT, 16);
+    const int64_t MT = ceil_div(R, 4), NT = ceil_div(N, 16);
     int s = 1;
+    if (MT <= kVecMT) {
+        while (NT * s < 1024 && s < kMaxSplit) s *= 2;
+        return s;
+    }
+    const int64_t gx = ceil_div(NT, MT <= kSkinnyMT ? kSkinnyNT : kGemmNT), gy = ceil_div(MT, 16);
     while (gx * gy * s < kGemmFillWgs && s < kMaxSplit) s *= 2;
     return s;
 }
@@ -1072,32 +1135,48 @@ int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, i
     }
     g.tot = tot;
     g.MT = (int)ceil_div(R, 4); g.NT = (int)ceil_div(N, 16); g.KB = (int)(K / 64); g.ldd = g.NT * 16;
-    const bool skinny = g.MT <= kSkinnyMT;              // few rows: the weight-streaming variant
     const int gy = (int)ceil_div(g.MT, 16);
-    bool wide = false;
-    if (!skinny) {
-        // Rounds of workgroups on 256 compute units, in matrix instructions per step: two general workgroups
-        // share a compute unit (2 x 32), a wide one has it alone (40).
-        const int w4 = (int)ceil_div(g.NT, kGemmNT) * gy * n, w5 = (int)ceil_div(g.NT, kGemmWideNT) * gy * n;
-        const int rem = w4 % 512;
-        const int cost4 = (w4 / 512) * 64 + (rem == 0 ? 0 : rem <= 256 ? 32 : 64), cost5 = (int)ceil_div(w5, 256) * 40;
-        wide = w4 >= 256 && RWKV_GEMM_WIDE_NUM * cost5 < RWKV_GEMM_WIDE_DEN * cost4;
-    }
-    const int gx = (int)ceil_div(g.NT, skinny ? kSkinnyNT : wide ? kGemmWideNT : kGemmNT);
-    // Split the contraction until the grid has a few workgroups per compute unit.
+    g.R = (int)R; g.N = (int)N; g.gate = gate;
     int split = 1;
-    while (gx * gy * n * split < kGemmFillWgs && g.KB / (split * 2) >= 8 && split < kMaxSplit) split *= 2;
-    g.kb_per_split = (int)ceil_div(g.KB, split);
-    g.split = split;
-    g.slice = (size_t)g.MT * 4 * g.ldd;
-    g.gx = gx; g.gy = gy; g.gz = split * n; g.by_rows = gy >= kXcds;
-    g.per_xcd = ((g.by_rows ? gy : gx) + kXcds - 1) / kXcds;
-    g.tail = split > 1 ? -1 : op; g.R = (int)R; g.N = (int)N; g.gate = gate;
-    const dim3 grid((unsigned)(kXcds * g.per_xcd * (g.by_rows ? gx : gy) * g.gz));
-    if (skinny) hipLaunchKernelGGL(gemm8_skinny_kernel, grid, dim3(256), 0, st, g);
-    else if (wide) hipLaunchKernelGGL(gemm8_wide_kernel, grid, dim3(512), 0, st, g);
-    else hipLaunchKernelGGL(gemm8_kernel, grid, dim3(256), 0, st, g);
-    RWKV_CHECK_LAUNCH("gemm8_kernel");
+    if (g.MT <= kVecMT) {
+        // a handful of rows: one 16-column tile per workgroup, the contraction split until there are a few
+        // workgroups per compute unit (their integer slices are added by the tail kernel)
+        while (g.NT * n * split < 1024 && g.KB / (split * 2) >= 8 && split < kMaxSplit) split *= 2;
+        g.kb_per_split = (int)ceil_div(g.KB, split);
+        g.split = split;
+        g.slice = (size_t)g.MT * 4 * g.ldd;
+        g.gx = g.NT; g.gy = 1; g.gz = split * n; g.by_rows = 0; g.per_xcd = 0;
+        g.tail = split > 1 ? -1 : op;
+        const dim3 grid((unsigned)(g.NT * g.gz));
+        if (g.MT == 1) hipLaunchKernelGGL(gemv16_kernel<1>, grid, dim3(256), 0, st, g);
+        else hipLaunchKernelGGL(gemv16_kernel<2>, grid, dim3(256), 0, st, g);
+        RWKV_CHECK_LAUNCH("gemv16_kernel");
+    } else {
+        const bool skinny = g.MT <= kSkinnyMT;              // few rows: the weight-streaming variant
+        bool wide = false;
+        if (!skinny) {
+            // Rounds of workgroups on 256 compute units, in matrix instructions per step: two general workgroups
+            // share a compute unit (2 x 32), a wide one has it alone (40).
+            const int w4 = (int)ceil_div(g.NT, kGemmNT) * gy * n, w5 = (int)ceil_div(g.NT, kGemmWideNT) * gy * n;
+            const int rem = w4 % 512;
+            const int cost4 = (w4 / 512) * 64 + (rem == 0 ? 0 : rem <= 256 ? 32 : 64), cost5 = (int)ceil_div(w5, 256) * 40;
+            wide = w4 >= 256 && RWKV_GEMM_WIDE_NUM * cost5 < RWKV_GEMM_WIDE_DEN * cost4;
+        }
+        const int gx = (int)ceil_div(g.NT, skinny ? kSkinnyNT : wide ? kGemmWideNT : kGemmNT);
+        // Split the contraction until the grid has a few workgroups per compute unit.
+        while (gx * gy * n * split < kGemmFillWgs && g.KB / (split * 2) >= 8 && split < kMaxSplit) split *= 2;
+        g.kb_per_split = (int)ceil_div(g.KB, split);
+        g.split = split;
+        g.slice = (size_t)g.MT * 4 * g.ldd;
+        g.gx = gx; g.gy = gy; g.gz = split * n; g.by_rows = gy >= kXcds;
+        g.per_xcd = ((g.by_rows ? gy : gx) + kXcds - 1) / kXcds;
+        g.tail = split > 1 ? -1 : op;
+        const dim3 grid((unsigned)(kXcds * g.per_xcd * (g.by_rows ? gx : gy) * g.gz));
+        if (skinny) hipLaunchKernelGGL(gemm8_skinny_kernel, grid, dim3(256), 0, st, g);
+        else if (wide) hipLaunchKernelGGL(gemm8_wide_kernel, grid, dim3(512), 0, st, g);
+        else hipLaunchKernelGGL(gemm8_kernel, grid, dim3(256), 0, st, g);
+        RWKV_CHECK_LAUNCH("gemm8_kernel");
+    }
     if (split == 1) return RWKV_OK;     // the tail was applied in the product's epilogue
 
     f.R = (int)R; f.N = (int)N; f.ldd = g.ldd; f.slices = split; f.slice = g.slice; f.tot = tot; f.gate = gate;
