@@ -94,13 +94,18 @@ __device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + ex
 //   aa e^pp <- e^w (aa e^pp) + e^{w+k} v   (same for bb).
 template <typename F>
 __device__ __forceinline__ F wkv_step(F w, F u, F k, F v, F &aa, F &bb, F &pp) {
+    // Of each pair of exponentials one is e^0: with d = a - b, (e^{a - max}, e^{b - max}) is (1, e^{-d}) or
+    // (e^{d}, 1), so one call per pair gives the same bits as two.
     const F q = u + w + k;
-    const F p = fmax(pp, q);
-    const F e1 = exp(pp - p), e2 = exp(q - p);
+    const F d = pp - q;
+    const F e = exp(-fabs(d));
+    const F e1 = d >= F(0) ? F(1) : e, e2 = d >= F(0) ? e : F(1);
     const F y = (e1 * aa + e2 * v) / (e1 * bb + e2);
     const F s = pp + w, r = k + w;
+    const F d2 = s - r;
+    const F f = exp(-fabs(d2));
     const F p2 = fmax(s, r);
-    const F f1 = exp(s - p2), f2 = exp(r - p2);
+    const F f1 = d2 >= F(0) ? F(1) : f, f2 = d2 >= F(0) ? f : F(1);
     aa = f1 * aa + f2 * v;
     bb = f1 * bb + f2;
     pp = p2;

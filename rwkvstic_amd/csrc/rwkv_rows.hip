@@ -216,7 +216,9 @@ __global__ void __launch_bounds__(kLT) rows_ln_mix_quant_kernel(const LnQuantArg
         }
     }
     lsum<2, kLW>(q, red);
-    const double sd = sqrt(q[0] / (double)C + 1e-5), sdp = sqrt(q[1] / (double)C + 1e-5);
+    // (one reciprocal per row instead of a float64 division per channel: the last bit of a float64 is far below
+    // anything the float32 quantiser input can see)
+    const double rsd = 1.0 / sqrt(q[0] / (double)C + 1e-5), rsdp = 1.0 / sqrt(q[1] / (double)C + 1e-5);
     float xs[NO][NSEG][4];
     float amax[NO];
     double z[NO];
@@ -235,8 +237,8 @@ __global__ void __launch_bounds__(kLT) rows_ln_mix_quant_kernel(const LnQuantArg
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                xy[i] = lw[g][i] * ((xv[g][i] - mean) / sd) + lb[g][i];
-                if (NM > 0) prev[i] = need_prev ? lw[g][i] * ((pv[g][i] - meanp) / sdp) + lb[g][i] : pv[g][i];
+                xy[i] = lw[g][i] * ((xv[g][i] - mean) * rsd) + lb[g][i];
+                if (NM > 0) prev[i] = need_prev ? lw[g][i] * ((pv[g][i] - meanp) * rsdp) + lb[g][i] : pv[g][i];
             }
 #pragma unroll
             for (int m = 0; m < NO; ++m) {
