@@ -90,21 +90,21 @@ rows_embed_kernel(const int64_t *__restrict__ tokens, int V, int C, const float 
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ double emit_quad(const float (&x4)[4], double invS, int c0, int t, int KB,
                                             signed char *dig) {
-    unsigned pl[4] = {0u, 0u, 0u, 0u};
+    // q = sum_k d_k 256^k with signed digits d_k in [-128, 127]  <=>  q + 0x80808080 has the unsigned bytes
+    // d_k + 128, and b - 128 is b ^ 0x80 as a signed byte: two instructions give all four digits of a value.
+    unsigned u[4];
     double qsum = 0.0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        int q = __double2int_rn((double)x4[i] * invS);
+        const int q = __double2int_rn((double)x4[i] * invS);
         qsum += (double)q;
-        const int d3 = (int)(signed char)(q & 0xff); q = (q - d3) >> 8;
-        const int d2 = (int)(signed char)(q & 0xff); q = (q - d2) >> 8;
-        const int d1 = (int)(signed char)(q & 0xff); q = (q - d1) >> 8;
-        const int sh = 8 * i;
-        pl[0] |= (unsigned)(q & 0xff) << sh;
-        pl[1] |= (unsigned)(d1 & 0xff) << sh;
-        pl[2] |= (unsigned)(d2 & 0xff) << sh;
-        pl[3] |= (unsigned)(d3 & 0xff) << sh;
+        u[i] = ((unsigned)q + 0x80808080u) ^ 0x80808080u;
     }
+    // 4 x 4 byte transpose: one dword per digit plane, most significant first
+    const unsigned x0 = __builtin_amdgcn_perm(u[1], u[0], 0x05010400u), x1 = __builtin_amdgcn_perm(u[1], u[0], 0x07030602u);
+    const unsigned y0 = __builtin_amdgcn_perm(u[3], u[2], 0x05010400u), y1 = __builtin_amdgcn_perm(u[3], u[2], 0x07030602u);
+    const unsigned pl[4] = {__builtin_amdgcn_perm(y1, x1, 0x07060302u), __builtin_amdgcn_perm(y1, x1, 0x05040100u),
+                            __builtin_amdgcn_perm(y0, x0, 0x07060302u), __builtin_amdgcn_perm(y0, x0, 0x05040100u)};
     const int mt = t >> 2, m0 = (t & 3) * 4;
     const int kb = c0 >> 6, g = (c0 & 63) >> 4, j = (c0 & 15) >> 2;
     signed char *frag = dig + ((size_t)mt * KB + kb) * 1024 + (16 * g + m0) * 16 + 4 * j;
