@@ -480,11 +480,19 @@ struct GemmArgs {
 
 constexpr int kGM = 8;                   // M-tiles of accumulators per wavefront (GN N-tiles: 4, or 5 in the wide variant)
 constexpr int kGemmNT = 8, kGemmWideNT = 10;     // N-tiles per workgroup (two wavefronts side by side)
-constexpr int kGemmAhead = 3;           // contraction blocks on their way from memory
+#ifndef RWKV_WIDE_RING
+#define RWKV_WIDE_RING 4
+#endif
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global load
 // the wavefront has in flight, which would drain the prefetched contraction blocks at every step.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// 16 bytes per lane from global memory straight into LDS at lds_byte_offset + 16 * lane (the offset is uniform
+// for the wavefront and travels in M0; one wait state between writing M0 and the load that reads it).
+__device__ __forceinline__ void dma16(const v4i *g, unsigned lds_byte_offset) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(g), "s"(lds_byte_offset) : "memory");
+}
 
 // Accumulators of one wavefront (GM M-tiles x GN N-tiles from (mt0, nt0)) to totals or, when the
 // contraction is not split, straight through the product's tail.
@@ -530,15 +538,15 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs &a, const v4i (&acc
 // N-tiles.  <4, 2> is the general shape (4 wavefronts, two workgroups per compute unit); <5, 4> (8 wavefronts
 // of 4 x 5 tiles, one workgroup per compute unit) is used where it turns a grid of 1.25 workgroups per compute
 // unit into exactly one (2560 columns: 16 column blocks instead of 20).
-template <int GN, int WM>
+template <int GN, int WM, int RING>
 __device__ __forceinline__ void gemm8_body(const GemmArgs a) {
-    // Both operands of a contraction block are fetched once per workgroup (registers, kGemmAhead
-    // blocks ahead), parked in LDS (two buffers, one barrier per block) and read from there by the
-    // two wavefronts that need each fragment.
+    // Both operands of a contraction block are fetched once per workgroup into LDS and read from there by
+    // the wavefronts that need each fragment (one barrier per block).
     constexpr int kGN = GN, kNT = 2 * GN, kGM = 16 / WM, kNW = 2 * WM;    // (kGM shadows the 4-wavefront constant)
     constexpr int kGemmFrags = 16 + kNT;                // fragments of one contraction block: 16 M-tiles of digits, kNT N-tiles of weights
     constexpr int kGemmLoads = (kGemmFrags + kNW - 1) / kNW;    // per thread and contraction block (wave w fetches fragments w, w + kNW, ...)
-    __shared__ v4i frag[2][kNW * kGemmLoads][64];
+    constexpr int kSlots = kNW * kGemmLoads, kGemmRing = RING;
+    __shared__ v4i frag[kGemmRing][kSlots][64];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave % WM, wn = wave / WM;
@@ -585,93 +593,59 @@ __device__ __forceinline__ void gemm8_body(const GemmArgs a) {
 #pragma unroll
         for (int j = 0; j < kGN; ++j) acc[i][j] = v4i{0, 0, 0, 0};
 
-    // the blocks in flight live in three separately named register sets: an array indexed by the
-    // stage would be indexed dynamically once the loop is rotated, and end up in scratch memory
-    static_assert(kGemmAhead == 3, "three named stages below");
-    static_assert(kGemmLoads >= 4 && kGemmLoads <= 7 && kGemmLoads <= kGM, "named members below, one parked per group of matrix instructions");
-    struct Fly { v4i v0, v1, v2, v3, v4, v5, v6; };       // named members, not an array: they must stay registers
-    Fly fly0, fly1, fly2;
-#define RWKV_GEMM_FETCH(F, K)                                                                        \
+    // Contraction blocks travel from memory straight into a ring of kGemmRing LDS buffers (direct-to-LDS
+    // loads: no registers, no LDS write instructions); block K + kGemmRing - 1 is requested in step K, into the
+    // buffer block K - 1 has just left.  The compiler does not see these loads, so the waits are written here:
+    // before the barrier of step K a wavefront waits until only the requests of the blocks after K are still out.
+    const unsigned lds0 = (unsigned)(size_t)&frag[0][0][0] + (unsigned)wave * 1024u;
+#define RWKV_GEMM_DMA(SLOT, K)                                                                       \
     do {                                                                                             \
         const size_t o_ = (size_t)((K) < nk ? (K) : nk - 1) * 64; /* past the end: the last block again (unused) */ \
-        F.v0 = src[0][o_]; F.v1 = src[1][o_]; F.v2 = src[2][o_]; F.v3 = src[3][o_];                  \
-        if (kGemmLoads > 4) F.v4 = src[kGemmLoads > 4 ? 4 : 0][o_];                                  \
-        if (kGemmLoads > 5) F.v5 = src[kGemmLoads > 5 ? 5 : 0][o_];                                  \
-        if (kGemmLoads > 6) F.v6 = src[kGemmLoads > 6 ? 6 : 0][o_];                                  \
+        _Pragma("unroll") for (int i = 0; i < kGemmLoads; ++i)                                       \
+            dma16(src[i] + o_, lds0 + (unsigned)(((SLOT) * kSlots + kNW * i) * 1024));               \
     } while (0)
-#define RWKV_GEMM_PARK(F, B)                                                                         \
-    do {                                                                                             \
-        frag[B][wave][lane] = F.v0; frag[B][wave + kNW][lane] = F.v1; frag[B][wave + 2 * kNW][lane] = F.v2; \
-        frag[B][wave + 3 * kNW][lane] = F.v3;                                                        \
-        if (kGemmLoads > 4) frag[B][wave + (kGemmLoads > 4 ? 4 : 0) * kNW][lane] = F.v4;             \
-        if (kGemmLoads > 5) frag[B][wave + (kGemmLoads > 5 ? 5 : 0) * kNW][lane] = F.v5;             \
-        if (kGemmLoads > 6) frag[B][wave + (kGemmLoads > 6 ? 6 : 0) * kNW][lane] = F.v6;             \
-    } while (0)
-    // Step K multiplies block K out of buffer K & 1.  The barrier at its top says that block K is parked and
-    // that every wavefront is done with block K - 1, whose buffer is then free: the NEXT block (registers FN,
-    // fetched kGemmAhead steps ago) is parked there fragment by fragment between this step's groups of matrix
-    // instructions, each register set refilled as soon as it is parked, so that LDS writes, global loads and
-    // LDS reads alternate in small pieces instead of queueing up in front of the first operand reads.
-#define RWKV_GEMM_MOVE(FN, I, V, B, O)                                                               \
-    if ((I) < kGemmLoads) { frag[B][wave + kNW * ((I) < kGemmLoads ? (I) : 0)][lane] = FN.V; FN.V = src[(I) < kGemmLoads ? (I) : 0][O]; }
-#define RWKV_GEMM_STEP(FN, K)                                                                        \
+#define RWKV_GEMM_STEP(SLOT, K)                                                                      \
     {                                                                                                \
-        const int buf_ = (K) & 1;                                                                    \
-        const size_t on_ = (size_t)((K) + 1 + kGemmAhead < nk ? (K) + 1 + kGemmAhead : nk - 1) * 64; \
-        lds_barrier();                                                                               \
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" :: "n"((kGemmRing - 2) * kGemmLoads) : "memory"); \
+        RWKV_GEMM_DMA(((SLOT) + kGemmRing - 1) % kGemmRing, (K) + kGemmRing - 1);                    \
         v4i Bv_[kGN];                                                                                \
         _Pragma("unroll") for (int j = 0; j < kGN; ++j) {                                            \
-            Bv_[j] = frag[buf_][16 + wn * kGN + j][lane];                                            \
+            Bv_[j] = frag[SLOT][16 + wn * kGN + j][lane];                                            \
         }                                                                                            \
-        v4i Av_ = frag[buf_][wm * kGM][lane], Aw_ = frag[buf_][wm * kGM + 1][lane];                  \
+        v4i Av_ = frag[SLOT][wm * kGM][lane], Aw_ = frag[SLOT][wm * kGM + 1][lane];                  \
         _Pragma("unroll") for (int i = 0; i < kGM; ++i) {                                            \
-            const v4i An_ = frag[buf_][wm * kGM + (i + 2 < kGM ? i + 2 : i)][lane];   /* two groups ahead */ \
-            if (i == 0) RWKV_GEMM_MOVE(FN, 0, v0, buf_ ^ 1, on_)                                     \
-            if (i == 1) RWKV_GEMM_MOVE(FN, 1, v1, buf_ ^ 1, on_)                                     \
-            if (i == 2) RWKV_GEMM_MOVE(FN, 2, v2, buf_ ^ 1, on_)                                     \
-            if (i == 3) RWKV_GEMM_MOVE(FN, 3, v3, buf_ ^ 1, on_)                                     \
-            if (i == 4) RWKV_GEMM_MOVE(FN, 4, v4, buf_ ^ 1, on_)                                     \
-            if (i == 5) RWKV_GEMM_MOVE(FN, 5, v5, buf_ ^ 1, on_)                                     \
-            if (i == 6) RWKV_GEMM_MOVE(FN, 6, v6, buf_ ^ 1, on_)                                     \
+            const v4i An_ = frag[SLOT][wm * kGM + (i + 2 < kGM ? i + 2 : i)][lane];   /* two groups ahead */ \
             _Pragma("unroll") for (int j = 0; j < kGN; ++j)                                          \
                 acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Av_, Bv_[j], acc[i][j], 0, 0, 0);  \
             Av_ = Aw_; Aw_ = An_;                                                                    \
         }                                                                                            \
-        /* the order the scheduler is asked to keep: first operands, then per group of matrix */     \
-        /* instructions one LDS write, one LDS read and one global load */                          \
         __builtin_amdgcn_sched_group_barrier(0x100, kGN + 3, 0);                                     \
         _Pragma("unroll") for (int i = 0; i < kGM; ++i) {                                            \
-            if (i < kGemmLoads) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                   \
             __builtin_amdgcn_sched_group_barrier(0x008, kGN, 0);                                     \
             if (i + 3 < kGM) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                      \
-            if (i < kGemmLoads) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                   \
         }                                                                                            \
     }
-    RWKV_GEMM_FETCH(fly0, 0); RWKV_GEMM_FETCH(fly1, 1); RWKV_GEMM_FETCH(fly2, 2);
-    RWKV_GEMM_PARK(fly0, 0);
-    RWKV_GEMM_FETCH(fly0, kGemmAhead);
-    // whole rounds run without a branch between the steps: the compiler then counts exactly which loads
-    // a step has to wait for (with a test per step it drains every load in flight once per round)
+#pragma unroll
+    for (int s = 0; s + 1 < kGemmRing; ++s) RWKV_GEMM_DMA(s, s);
     int k0 = 0;
-    for (; k0 + kGemmAhead <= nk; k0 += kGemmAhead) {
-        RWKV_GEMM_STEP(fly1, k0)
-        RWKV_GEMM_STEP(fly2, k0 + 1)
-        RWKV_GEMM_STEP(fly0, k0 + 2)
+    for (; k0 + kGemmRing <= nk; k0 += kGemmRing) {     // whole turns of the ring: the buffer of a step is a constant
+#pragma unroll
+        for (int s = 0; s < kGemmRing; ++s) RWKV_GEMM_STEP(s, k0 + s)
     }
-    if (k0 < nk) RWKV_GEMM_STEP(fly1, k0)
-    if (k0 + 1 < nk) RWKV_GEMM_STEP(fly2, k0 + 1)
+#pragma unroll
+    for (int s = 0; s + 1 < kGemmRing; ++s)
+        if (k0 + s < nk) RWKV_GEMM_STEP(s, k0 + s)
 #undef RWKV_GEMM_STEP
-#undef RWKV_GEMM_MOVE
-#undef RWKV_GEMM_PARK
-#undef RWKV_GEMM_FETCH
+#undef RWKV_GEMM_DMA
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // nothing of this wavefront may still be writing LDS when it leaves
     gemm_epilogue<kGM, kGN>(a, acc, mt0, nt0, mat, bz, lane);
 }
 
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) gemm8_kernel(const GemmArgs a) {
-    gemm8_body<4, 2>(a);
+    gemm8_body<4, 2, 3>(a);
 }
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) gemm8_wide_kernel(const GemmArgs a) {
-    gemm8_body<5, 4>(a);
+    gemm8_body<5, 4, RWKV_WIDE_RING>(a);
 }
 
 // ---------------------------------------------------------------------------
