@@ -478,7 +478,6 @@ struct GemmArgs {
     const double *gate;
 };
 
-constexpr int kGM = 8;                   // M-tiles of accumulators per wavefront (GN N-tiles: 4, or 5 in the wide variant)
 constexpr int kGemmNT = 8, kGemmWideNT = 10;     // N-tiles per workgroup (two wavefronts side by side)
 #ifndef RWKV_WIDE_RING
 #define RWKV_WIDE_RING 4
@@ -535,14 +534,14 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs &a, const v4i (&acc
 }
 
 // One workgroup of the product: 64 tokens x 32*GN columns, 2*WM wavefronts as WM x 2, each 16/WM M-tiles x GN
-// N-tiles.  <4, 2> is the general shape (4 wavefronts, two workgroups per compute unit); <5, 4> (8 wavefronts
-// of 4 x 5 tiles, one workgroup per compute unit) is used where it turns a grid of 1.25 workgroups per compute
-// unit into exactly one (2560 columns: 16 column blocks instead of 20).
+// N-tiles, RING LDS buffers.  <4, 4, 3> is the general shape (8 wavefronts of 4 x 4 tiles, two workgroups per
+// compute unit); <5, 4, 4> (4 x 5 tiles, one workgroup per compute unit) is used where it turns a grid of 1.25
+// workgroups per compute unit into exactly one (2560 columns: 16 column blocks instead of 20).
 template <int GN, int WM, int RING>
 __device__ __forceinline__ void gemm8_body(const GemmArgs a) {
     // Both operands of a contraction block are fetched once per workgroup into LDS and read from there by
     // the wavefronts that need each fragment (one barrier per block).
-    constexpr int kGN = GN, kNT = 2 * GN, kGM = 16 / WM, kNW = 2 * WM;    // (kGM shadows the 4-wavefront constant)
+    constexpr int kGN = GN, kNT = 2 * GN, kGM = 16 / WM, kNW = 2 * WM;
     constexpr int kGemmFrags = 16 + kNT;                // fragments of one contraction block: 16 M-tiles of digits, kNT N-tiles of weights
     constexpr int kGemmLoads = (kGemmFrags + kNW - 1) / kNW;    // per thread and contraction block (wave w fetches fragments w, w + kNW, ...)
     constexpr int kSlots = kNW * kGemmLoads, kGemmRing = RING;
@@ -641,8 +640,8 @@ __device__ __forceinline__ void gemm8_body(const GemmArgs a) {
     gemm_epilogue<kGM, kGN>(a, acc, mt0, nt0, mat, bz, lane);
 }
 
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) gemm8_kernel(const GemmArgs a) {
-    gemm8_body<4, 2, 3>(a);
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) gemm8_kernel(const GemmArgs a) {
+    gemm8_body<4, 4, 3>(a);
 }
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) gemm8_wide_kernel(const GemmArgs a) {
     gemm8_body<5, 4, RWKV_WIDE_RING>(a);
@@ -1150,7 +1149,7 @@ int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, i
         const dim3 grid((unsigned)(kXcds * g.per_xcd * (g.by_rows ? gx : gy) * g.gz));
         if (skinny) hipLaunchKernelGGL(gemm8_skinny_kernel, grid, dim3(256), 0, st, g);
         else if (wide) hipLaunchKernelGGL(gemm8_wide_kernel, grid, dim3(512), 0, st, g);
-        else hipLaunchKernelGGL(gemm8_kernel, grid, dim3(256), 0, st, g);
+        else hipLaunchKernelGGL(gemm8_kernel, grid, dim3(512), 0, st, g);
         RWKV_CHECK_LAUNCH("gemm8_kernel");
     }
     if (split == 1) return RWKV_OK;     // the tail was applied in the product's epilogue
