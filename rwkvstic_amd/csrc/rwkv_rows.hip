@@ -449,10 +449,11 @@ __global__ void __launch_bounds__(kRT) rows_quant4_kernel(const QuantArgs a) {
 
 // ---------------------------------------------------------------------------
 // GEMM: tot[t, j] = sum_k q[t, k] * (code[k, j] - 128), exact in int64.
-// Workgroup = 4 wavefronts = 64 tokens x 128 columns; wavefront (wm, wn) holds
-// 8 M-tiles x 4 N-tiles of accumulators.  With few rows the contraction is split over
-// several workgroups; each split writes its own slice of integer totals and the tail
-// kernel adds the slices (integer sums: exact in any order).
+// Workgroup = 8 wavefronts = 64 tokens x 128 (or 160) columns; wavefront (wm, wn) holds
+// 4 M-tiles x 4 (or 5) N-tiles of accumulators; variants for at most 32 and at most 8 rows
+// follow.  With few rows the contraction is split over several workgroups; each split writes
+// its own slice of integer totals and the tail kernel adds the slices (integer sums: exact in
+// any order).
 //
 // Launch order.  Workgroups are handed to the 8 XCDs round robin, and each XCD has its own L2.  The
 // grid is 1-D and workgroup i works for XCD i % 8 on that XCD's own row blocks (row block r belongs
