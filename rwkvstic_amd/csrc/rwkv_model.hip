@@ -494,13 +494,15 @@ struct RowsWs {
     long long *tot;
 };
 
-size_t rows_tot_ws_bytes(int64_t R, int64_t C, int64_t n_wide) {
+// n_head > 0: one more product, of a single row with n_head columns (the head after a prompt)
+size_t rows_tot_ws_bytes(int64_t R, int64_t C, int64_t n_wide, int64_t n_head) {
     const size_t a = rows_tot_bytes(R, n_wide), b = 3 * rows_tot_bytes(R, C);     // k, v, r share a launch
-    return a > b ? a : b;
+    const size_t c = n_head > 0 ? rows_tot_bytes(1, n_head) : 0;
+    return a > b ? (a > c ? a : c) : (b > c ? b : c);
 }
 
 // n_wide = widest product output (n_ffn, or the vocabulary when every row needs logits)
-size_t rows_ws_bytes(int64_t R, int64_t C, int64_t F, int64_t n_wide) {
+size_t rows_ws_bytes(int64_t R, int64_t C, int64_t F, int64_t n_wide, int64_t n_head) {
     size_t n = 0;
     n += round_up((size_t)R * C * 8, 256) * 5;          // x, kvr[3], att
     n += round_up((size_t)R * F * 8, 256);              // h
@@ -508,11 +510,11 @@ size_t rows_ws_bytes(int64_t R, int64_t C, int64_t F, int64_t n_wide) {
     n += round_up(rows_wkv_scratch_bytes(R, C), 256);
     n += round_up((size_t)R * 8, 256) * 9;              // S, qs, zp of three operands
     n += round_up(rows_dig_bytes(R, F), 256) + 2 * round_up(rows_dig_bytes(R, C), 256);
-    n += round_up(rows_tot_ws_bytes(R, C, n_wide), 256);
+    n += round_up(rows_tot_ws_bytes(R, C, n_wide, n_head), 256);
     return n;
 }
 
-RowsWs rows_carve(void *ws, int64_t R, int64_t C, int64_t F, int64_t n_wide) {
+RowsWs rows_carve(void *ws, int64_t R, int64_t C, int64_t F, int64_t n_wide, int64_t n_head) {
     unsigned char *p = static_cast<unsigned char *>(ws);
     auto take = [&](size_t bytes) { void *q = p; p += round_up(bytes, 256); return q; };
     RowsWs w;
@@ -528,7 +530,7 @@ RowsWs rows_carve(void *ws, int64_t R, int64_t C, int64_t F, int64_t n_wide) {
         w.q[i].zp = (double *)take((size_t)R * 8);
         w.q[i].dig = (signed char *)take(rows_dig_bytes(R, i == 0 ? F : C));
     }
-    w.tot = (long long *)take(rows_tot_ws_bytes(R, C, n_wide));
+    w.tot = (long long *)take(rows_tot_ws_bytes(R, C, n_wide, n_head));
     return w;
 }
 
@@ -614,12 +616,22 @@ int rows_sequence(rwkv_model *m, hipStream_t st, const int64_t *tokens, int64_t 
     const int64_t C = m->d.n_embd, F = m->d.n_ffn;
     unsigned char *rows_base = static_cast<unsigned char *>(workspace) + round_up(ws_doubles(C, F) * sizeof(double), 256);
     const int64_t Rmax = T < kRowsChunk ? T : kRowsChunk;
-    const RowsWs rw = rows_carve(rows_base, Rmax, C, F, F);
+    const RowsWs rw = rows_carve(rows_base, Rmax, C, F, F, m->d.n_vocab);
     for (int64_t t0 = 0; t0 < T; t0 += kRowsChunk) {
         const int64_t R = T - t0 < kRowsChunk ? T - t0 : kRowsChunk;
         int rc = rows_layers(m, st, tokens + t0, R, true, state, 0, rw);
         if (rc) return rc;
-        if (t0 + R == T) rc = head_logits(m, st, rw.x + (size_t)(R - 1) * C, logits);
+        if (t0 + R == T) {
+            // ln_out and the head on the last row (opt.py:72-74), as a one-row product with integer sums
+            const rwkv_model_desc &d = m->d;
+            const float *rg[1] = {d.head.range};
+            const double *of[1] = {d.head.offset};
+            rc = rows_ln_mix_quant(st, 0, 1, (int)C, false, rw.x + (size_t)(R - 1) * C, d.ln_out_w, d.ln_out_b, nullptr,
+                                   nullptr, nullptr, 0, rg, of, rw.q);
+            if (rc) return rc;
+            const RowsProduct ph = {rw.q[0], d.head.packed16, logits};
+            rc = rows_products(st, 1, &ph, rw.tot, 1, C, d.n_vocab, ROW_STORE, nullptr);
+        }
         if (rc) return rc;
     }
     return RWKV_OK;
@@ -708,7 +720,7 @@ size_t rwkv_model_workspace_bytes(const rwkv_model *m, int64_t max_tokens) {
     size_t n = round_up(ws_doubles(m->d.n_embd, m->d.n_ffn) * sizeof(double), 256);
     if (use_rows(m, max_tokens)) {
         const int64_t R = max_tokens < kRowsChunk ? max_tokens : kRowsChunk;
-        n += rows_ws_bytes(R, m->d.n_embd, m->d.n_ffn, m->d.n_ffn);
+        n += rows_ws_bytes(R, m->d.n_embd, m->d.n_ffn, m->d.n_ffn, m->d.n_vocab);
     }
     return n;
 }
@@ -716,7 +728,7 @@ size_t rwkv_model_workspace_bytes(const rwkv_model *m, int64_t max_tokens) {
 size_t rwkv_model_batch_workspace_bytes(const rwkv_model *m, int64_t batch) {
     if (!m || batch <= 0 || !rows_supported(m)) return 0;
     const int64_t wide = m->d.n_ffn > m->d.n_vocab ? m->d.n_ffn : m->d.n_vocab;
-    return rows_ws_bytes(batch, m->d.n_embd, m->d.n_ffn, wide);
+    return rows_ws_bytes(batch, m->d.n_embd, m->d.n_ffn, wide, 0);
 }
 
 int rwkv_model_forward(rwkv_model *m, rwkv_stream_t stream, const int64_t *tokens, int64_t T, double *state,
@@ -752,7 +764,7 @@ int rwkv_model_forward_batch(rwkv_model *m, rwkv_stream_t stream, const int64_t 
     const hipStream_t st = (hipStream_t)stream;
     const rwkv_model_desc &d = m->d;
     const int64_t C = d.n_embd, F = d.n_ffn, V = d.n_vocab;
-    const RowsWs rw = rows_carve(workspace, batch, C, F, F > V ? F : V);
+    const RowsWs rw = rows_carve(workspace, batch, C, F, F > V ? F : V, 0);
     int rc = rows_layers(m, st, tokens, batch, false, states, d.n_layer * 5 * C, rw);
     if (rc) return rc;
     const float *rg[1] = {d.head.range};
