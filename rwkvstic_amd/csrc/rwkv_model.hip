@@ -588,22 +588,6 @@ int rows_layers(rwkv_model *m, hipStream_t st, const int64_t *tokens, int64_t R,
     return RWKV_OK;
 }
 
-// logits[V] of one residual row through ln_out and the head (opt.py:72-74)
-int head_logits(rwkv_model *m, hipStream_t st, const double *xrow, double *logits) {
-    const rwkv_model_desc &d = m->d;
-    const int C = (int)d.n_embd, V = (int)d.n_vocab;
-    const int c_kb = (int)ceil_div(C, kBlockRows);
-    const size_t red_bytes = 3 * kWaves * 8 + 3 * kWaves * 8 * 4;
-    LnMatArgs h;
-    h.C = C; h.mode = EPI_LOGITS; h.x = const_cast<double *>(xrow); h.ln_w = d.ln_out_w; h.ln_b = d.ln_out_b;
-    h.mix = nullptr; h.shift = nullptr; h.k = to_dev(d.head); h.r = h.k; h.out_k = logits; h.out_r = nullptr;
-    h.ln_tmp = nullptr;
-    hipLaunchKernelGGL(ln_matvec_kernel, dim3((unsigned)ceil_div(V, kTileCols)), dim3(kThreads),
-                       (size_t)c_kb * kBlockRows * 4 + red_bytes, st, h);
-    RWKV_CHECK_LAUNCH("head");
-    return RWKV_OK;
-}
-
 // Which path a sequence of T tokens takes: the many-row kernels for prompts, and for single tokens too when
 // the persistent single-token kernel does not serve the shape (their integer products beat one launch per
 // phase with float32 sums both in time and in accuracy).
