@@ -216,6 +216,21 @@ def test_prompt_gemm_path_matches_token_steps(tiny, n_prompt):
     assert ((a[:, 2] - b[:, 2]).abs() <= 1e-6 * torch.maximum(b[:, 2].abs(), b[:, 3]) + 1e-30).all()
 
 
+def test_prompt_longer_than_one_pass(tiny):
+    """A prompt of more rows than one pass of the many-row kernels takes (1024): the state is carried from pass to
+    pass inside one call; against the CPU oracle and against the same prompt fed as two calls."""
+    ref, hip = tiny
+    toks = synth.random_tokens(1100, V=512, seed=12).tolist()
+    lr, sr = ref.forward(toks, ref.emptyState.clone())
+    lg, sg = hip.forward(toks, hip.emptyState.clone())
+    _say(f"1100-token prompt |dlogits| vs oracle {(lg.cpu() - lr).abs().max().item():.2e}")
+    assert (lg.cpu() - lr).abs().max() < LOGIT_TOL and int(lg.argmax()) == int(lr.argmax())
+    _state_close(sg, sr)
+    _, s2 = hip.forward(toks[:700], hip.emptyState.clone())
+    l2, s2 = hip.forward(toks[700:], s2)
+    assert (lg - l2).abs().max() < 1e-5 and (sg[:, :2] - s2[:, :2]).abs().max() < 1e-6
+
+
 def test_prompt_gemm_path_mid_shape_vs_fp64_oracle():
     """C=256, F=1024, ragged vocabulary; 70 tokens (18 M-tiles: a partial 64-token workgroup tile)."""
     from rwkvstic_amd.model import HipRWKV
