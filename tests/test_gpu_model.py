@@ -244,14 +244,14 @@ def test_prompt_gemm_path_mid_shape_vs_fp64_oracle():
     _state_close(sg, sr, tol=STATE_TOL)
 
 
-def test_forward_batch_matches_per_sequence_steps(tiny):
+@pytest.mark.parametrize("B", [5, 20])      # 5: the products of at most 8 rows; 20: the 9..32-row variant
+def test_forward_batch_matches_per_sequence_steps(tiny, B):
     ref, hip = tiny
-    B = 5
     states, toks = [], []
     for b in range(B):
         s = hip.emptyState.clone()
         if b:                                     # sequence 0 starts from the empty state
-            _, s = hip.forward(synth.random_tokens(3 + b, V=512, seed=30 + b).tolist(), s)
+            _, s = hip.forward(synth.random_tokens(3 + b % 7, V=512, seed=30 + b).tolist(), s)
         states.append(s)
         toks.append(int(synth.random_tokens(1, V=512, seed=40 + b)[0]))
     batch_state = torch.stack(states).contiguous()
