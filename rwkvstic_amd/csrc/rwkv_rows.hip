@@ -775,9 +775,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 // slow load holds up one wavefront, not the workgroup.  The digit fragments (L2-resident) are read by every
 // wavefront itself.  One cross-wavefront sum in LDS at the end, then the common epilogue.
 // ---------------------------------------------------------------------------
-constexpr int kVecMT = 2, kVecBlocks = 8;
+constexpr int kVecMT = 2;
 
-template <int MT>
+// kVecBlocks: weight blocks a wavefront has in flight
+template <int MT, int kVecBlocks>
 __global__ void __launch_bounds__(256) gemv16_kernel(const GemmArgs a) {
     __shared__ v4i red[4][MT][64];
     const int lane = threadIdx.x & 63;
@@ -1007,6 +1008,7 @@ __global__ void __launch_bounds__(64) wkv_chunk_replay_kernel(const WkvRowsArgs 
 // ---------------------------------------------------------------------------
 size_t rows_dig_bytes(int64_t R, int64_t K) { return (size_t)(ceil_div(R, 4) * (K / 64) * 1024); }
 size_t rows_wkv_scratch_bytes(int64_t R, int64_t C) { return (size_t)(ceil_div(R, kWkvChunk) * 3 * C * 8); }
+constexpr int kVecFillWgs = 256;        // products of at most 8 rows: the contraction is split until there are this many workgroups
 constexpr int kMaxSplit = 8;
 #ifndef RWKV_GEMM_WIDE_NUM
 #define RWKV_GEMM_WIDE_NUM 10
@@ -1022,7 +1024,7 @@ static int gemm_split_bound(int64_t R, int64_t N) {
     const int64_t MT = ceil_div(R, 4), NT = ceil_div(N, 16);
     int s = 1;
     if (MT <= kVecMT) {
-        while (NT * s < 1024 && s < kMaxSplit) s *= 2;
+        while (NT * s < kVecFillWgs && s < kMaxSplit) s *= 2;
         return s;
     }
     const int64_t gx = ceil_div(NT, MT <= kSkinnyMT ? kSkinnyNT : kGemmNT), gy = ceil_div(MT, 16);
@@ -1115,17 +1117,17 @@ int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, i
     g.R = (int)R; g.N = (int)N; g.gate = gate;
     int split = 1;
     if (g.MT <= kVecMT) {
-        // a handful of rows: one 16-column tile per workgroup, the contraction split until there are a few
-        // workgroups per compute unit (their integer slices are added by the tail kernel)
-        while (g.NT * n * split < 1024 && g.KB / (split * 2) >= 8 && split < kMaxSplit) split *= 2;
+        // a handful of rows: one 16-column tile per workgroup; only products with fewer tiles than compute
+        // units split the contraction (their integer slices are added by the tail kernel)
+        while (g.NT * n * split < kVecFillWgs && g.KB / (split * 2) >= 8 && split < kMaxSplit) split *= 2;
         g.kb_per_split = (int)ceil_div(g.KB, split);
         g.split = split;
         g.slice = (size_t)g.MT * 4 * g.ldd;
         g.gx = g.NT; g.gy = 1; g.gz = split * n; g.by_rows = 0; g.per_xcd = 0;
         g.tail = split > 1 ? -1 : op;
         const dim3 grid((unsigned)(g.NT * g.gz));
-        if (g.MT == 1) hipLaunchKernelGGL(gemv16_kernel<1>, grid, dim3(256), 0, st, g);
-        else hipLaunchKernelGGL(gemv16_kernel<2>, grid, dim3(256), 0, st, g);
+        if (g.MT == 1) hipLaunchKernelGGL((gemv16_kernel<1, 8>), grid, dim3(256), 0, st, g);
+        else hipLaunchKernelGGL((gemv16_kernel<2, 8>), grid, dim3(256), 0, st, g);
         RWKV_CHECK_LAUNCH("gemv16_kernel");
     } else {
         const bool skinny = g.MT <= kSkinnyMT;              // few rows: the weight-streaming variant
