@@ -34,8 +34,9 @@ int rows_ln_mix_quant(hipStream_t st, int n_mix, int64_t R, int C, bool sequence
                       int64_t prev_stride, const float *const *range, const double *const *offset,
                       const RowsOperand *out);
 // Rows of float64 values quantised for a matrix with the given per-input-channel range / offset.
+// scratch: 16 * R * ceil(K / 3072) bytes (any buffer free until the product starts, e.g. its totals), or null.
 int rows_quant(hipStream_t st, int64_t R, int64_t K, const double *in, const float *range, const double *offset,
-               const RowsOperand &out);
+               const RowsOperand &out, double *scratch);
 // n (<= kRowsMaxProducts) products of the same shape [R, K] x [K, N] and tail in one launch;
 // tot: n * rows_tot_bytes(R, N) bytes of scratch.
 int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, int64_t R, int64_t K, int64_t N, int op,

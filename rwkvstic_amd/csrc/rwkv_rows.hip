@@ -447,6 +447,78 @@ __global__ void __launch_bounds__(kRT) rows_quant4_kernel(const QuantArgs a) {
     if (tid == 0) { a.S[t] = S; a.qs[t] = qsum[0]; a.zp[t] = z[0]; }
 }
 
+// A handful of long rows (one token of a wide ffn): one workgroup per row would pull the whole row and its
+// range / offset vectors through a single compute unit.  Two launches instead, G workgroups per row: the first
+// leaves each part's max |xs| and zero-point share in `part`, the second turns them into the row's scale and
+// writes the digits of its part.  The sum of the fixed-point values is added up with atomics: integers below
+// 2^53, exact in any order.
+constexpr int kQuantPartSeg = 3;        // groups of four values per thread: parts of up to 3072 values
+
+struct QuantPartArgs {
+    QuantArgs q;
+    int G, quads_per_part;
+    double *part;               // [R][G][2]: max |xs|, zero-point share
+};
+
+template <bool EMIT>
+__global__ void __launch_bounds__(kRT) rows_quant_part_kernel(const QuantPartArgs a) {
+    __shared__ double red[2 * kRW];
+    __shared__ float redf[kRW];
+    const int g = blockIdx.x, t = blockIdx.y, K = a.q.K, tid = threadIdx.x;
+    const double *row = a.q.in + (size_t)t * K;
+    const int q0 = g * a.quads_per_part, q1 = min(q0 + a.quads_per_part, K >> 2);
+    float xs[kQuantPartSeg][4];
+    float amax = 0.f;
+    double z[1] = {0.0};
+#pragma unroll
+    for (int s = 0; s < kQuantPartSeg; ++s) {
+        const int qi = q0 + tid + s * kRT;
+        if (qi < q1) {
+            const int c0 = 4 * qi;
+            const double2 v0 = *reinterpret_cast<const double2 *>(row + c0), v1 = *reinterpret_cast<const double2 *>(row + c0 + 2);
+            const float4 r = *reinterpret_cast<const float4 *>(a.q.range + c0);
+            xs[s][0] = (float)(v0.x * (double)r.x); xs[s][1] = (float)(v0.y * (double)r.y);
+            xs[s][2] = (float)(v1.x * (double)r.z); xs[s][3] = (float)(v1.y * (double)r.w);
+            if (!EMIT) {
+                const double2 o0 = *reinterpret_cast<const double2 *>(a.q.offset + c0), o1 = *reinterpret_cast<const double2 *>(a.q.offset + c0 + 2);
+                amax = fmaxf(fmaxf(amax, fmaxf(fabsf(xs[s][0]), fabsf(xs[s][1]))), fmaxf(fabsf(xs[s][2]), fabsf(xs[s][3])));
+                z[0] += v0.x * o0.x; z[0] += v0.y * o0.y; z[0] += v1.x * o1.x; z[0] += v1.y * o1.y;
+            }
+        }
+    }
+    double *part = a.part + (size_t)t * a.G * 2;
+    if (!EMIT) {
+        amax = wmaxf(amax);
+        if ((tid & 63) == 0) redf[tid >> 6] = amax;
+        rsum<1>(z, red);                   // (its barriers also publish redf)
+        if (tid == 0) {
+            amax = redf[0];
+#pragma unroll
+            for (int w = 1; w < kRW; ++w) amax = fmaxf(amax, redf[w]);
+            part[2 * g] = (double)amax; part[2 * g + 1] = z[0];
+            if (g == 0) a.q.qs[t] = 0.0;
+        }
+        return;
+    }
+    float am = 0.f;
+    double zp = 0.0;
+    for (int i = 0; i < a.G; ++i) { am = fmaxf(am, (float)part[2 * i]); zp += part[2 * i + 1]; }     // fixed order
+    double S, invS;
+    row_scale(am, S, invS);
+    const int KB = K >> 6;
+    double qsum[1] = {0.0};
+#pragma unroll
+    for (int s = 0; s < kQuantPartSeg; ++s) {
+        const int qi = q0 + tid + s * kRT;
+        if (qi < q1) qsum[0] += emit_quad(xs[s], invS, 4 * qi, t, KB, a.q.dig);
+    }
+    rsum<1>(qsum, red);
+    if (tid == 0) {
+        atomicAdd(a.q.qs + t, qsum[0]);
+        if (g == 0) { a.q.S[t] = S; a.q.zp[t] = zp; }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // GEMM: tot[t, j] = sum_k q[t, k] * (code[k, j] - 128), exact in int64.
 // Workgroup = 8 wavefronts = 64 tokens x 128 (or 160) columns; wavefront (wm, wn) holds
@@ -1083,12 +1155,22 @@ int rows_ln_mix_quant(hipStream_t st, int n_mix, int64_t R, int C, bool sequence
 }
 
 int rows_quant(hipStream_t st, int64_t R, int64_t K, const double *in, const float *range, const double *offset,
-               const RowsOperand &out) {
+               const RowsOperand &out, double *scratch) {
     if (K % 64 != 0) return set_error(RWKV_ERR_SIZE, "rows_quant: contraction length %lld is not a multiple of 64",
                                       (long long)K);
     QuantArgs q;
     q.K = (int)K; q.in = in; q.range = range; q.offset = offset; q.dig = out.dig; q.S = out.S; q.qs = out.qs; q.zp = out.zp;
     const dim3 grid((unsigned)R), block(kRT);
+    if (scratch && R <= 8 && K >= 8192) {
+        QuantPartArgs pa;
+        pa.q = q; pa.G = (int)ceil_div(K, 4 * kRT * kQuantPartSeg); pa.quads_per_part = (int)ceil_div(K / 4, pa.G);
+        pa.part = scratch;
+        const dim3 pg((unsigned)pa.G, (unsigned)R);
+        hipLaunchKernelGGL(rows_quant_part_kernel<false>, pg, block, 0, st, pa);
+        hipLaunchKernelGGL(rows_quant_part_kernel<true>, pg, block, 0, st, pa);
+        RWKV_CHECK_LAUNCH("rows_quant_part_kernel");
+        return RWKV_OK;
+    }
     if (K <= 3 * 4 * kRT) hipLaunchKernelGGL(rows_quant4_kernel<3>, grid, block, 0, st, q);
     else if (K <= 6 * 4 * kRT) hipLaunchKernelGGL(rows_quant4_kernel<6>, grid, block, 0, st, q);
     else if (K <= 10 * 4 * kRT) hipLaunchKernelGGL(rows_quant4_kernel<10>, grid, block, 0, st, q);

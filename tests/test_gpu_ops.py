@@ -256,7 +256,8 @@ def test_pack_m16_round_trip(ops):
 # with ragged rows, ragged columns and a contraction that ends inside a round of the pipeline
 @pytest.mark.parametrize("T,K,N", [(1, 64, 16), (5, 256, 100), (64, 2560, 2560), (130, 2560, 10240),
                                    (33, 10240, 2560), (8, 2560, 50277), (1000, 192, 2560), (1024, 320, 2500),
-                                   (3, 20544, 32),      # rows too long for the register-resident quantiser
+                                   (3, 20544, 32),      # a few long rows: the two-launch quantiser
+                                   (9, 20544, 32),      # rows too long for the register-resident quantiser
                                    (20, 2560, 2560), (32, 640, 5000)])   # 9..32 rows: the few-row variant with LDS staging
 def test_gemm8_matches_fp64_dense(ops, T, K, N):
     """Prompt GEMM (matmul.py:56-57 without its bfloat16 rounding) against the float64 dense product."""
