@@ -250,6 +250,15 @@ int rwkv_gemm8(rwkv_stream_t stream, int64_t T, int64_t n_in, int64_t n_out,
                const double *offset, double *y,
                void *workspace, size_t workspace_bytes);
 
+/* Diagnostics: the launch plan rwkv_gemm8 / the model's many-row path follows for
+ * n_products (1..3) products x[T, n_in] x matrix[n_in, n_out] sharing a launch
+ * (k, v, r do; matmul.py:86-94): plan = {kernel variant (0: at most 8 rows, 1: 9-32
+ * rows, 2: 64 x 128 tiles, 3: 64 x 160 tiles), grid x, grid y, splits of the
+ * contraction}, and in *tot_bytes_per_product the bytes of integer totals the
+ * workspace reserves per product.  Host-only: launches nothing. */
+int rwkv_gemm8_plan(int64_t T, int64_t n_in, int64_t n_out, int n_products,
+                    int plan[4], size_t *tot_bytes_per_product);
+
 /* One token for each of `batch` independent sequences (the reference has no
  * batched entry point on this path: it would call myRWKV.forward, opt.py:61-76,
  * once per sequence).  tokens[batch]; states[batch][n_layer][5][n_embd] updated

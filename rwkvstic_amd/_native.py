@@ -21,7 +21,7 @@ EXPORTS = (
     "rwkv_model_create", "rwkv_model_destroy", "rwkv_model_workspace_bytes",
     "rwkv_model_has_fused_step", "rwkv_model_check", "rwkv_model_set_trace",
     "rwkv_model_forward", "rwkv_model_decode_greedy", "rwkv_argmax_f64",
-    "rwkv_gemm8_workspace_bytes", "rwkv_gemm8",
+    "rwkv_gemm8_workspace_bytes", "rwkv_gemm8", "rwkv_gemm8_plan",
     "rwkv_model_batch_workspace_bytes", "rwkv_model_forward_batch",
 )
 
@@ -100,6 +100,7 @@ def lib() -> C.CDLL:
     L.rwkv_gemm8_workspace_bytes.restype = sz
     L.rwkv_gemm8_workspace_bytes.argtypes = [i64, i64, i64]
     L.rwkv_gemm8.argtypes = [vp, i64, i64, i64, vp, vp, vp, vp, vp, vp, sz]
+    L.rwkv_gemm8_plan.argtypes = [i64, i64, i64, ci, C.POINTER(ci * 4), C.POINTER(sz)]
     L.rwkv_model_batch_workspace_bytes.restype = sz
     L.rwkv_model_batch_workspace_bytes.argtypes = [vp, i64]
     L.rwkv_model_forward_batch.argtypes = [vp, vp, vp, i64, vp, vp, vp, sz]

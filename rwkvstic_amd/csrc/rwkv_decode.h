@@ -74,7 +74,7 @@ struct DModel {
 // the first launch; they belong to one model handle (one token step in flight at a time).
 struct DecodeBuffers {
     u64 *X;                 // [C]       residual stream
-    u64 *XR;                // [11][G]   per workgroup: sum x, sum x^2, then per matrix max |x P|, sum x PO (hi, lo)
+    u64 *XR;                // [13][G]   per workgroup: sum x (hi, lo), sum x^2 (hi, lo), then per matrix max |x P|, sum x PO (hi, lo)
     u64 *A;                 // [C]       fp32(wkv * sigmoid(r) * range_o)
     u64 *AR;                // [3][G]    per workgroup: max |A|, zero-point share (hi, lo)
     u64 *H;                 // [F]       fp32(relu(k)^2 * range_v)
@@ -105,6 +105,10 @@ size_t decode_block_bytes(int64_t L, int64_t C, int64_t F, int64_t V);
 // Fills `block` (device, decode_block_bytes, zero-filled by the caller) and the two descriptors.
 // Synchronises the device (model creation only).
 int decode_setup(void *block, const DSetup &s, DModel *dm, DecodeBuffers *db);
+
+// Zero-fills the exchange buffers on the stream (a kernel, so the call may be captured); the next launch must
+// use epoch 1.
+int decode_clear_exchange(hipStream_t st, const DModel &m, const DecodeBuffers &b);
 
 // One token: token[0] -> logits[V], state [L,5,C] updated in place.  epoch0 must grow by
 // decode_epochs_per_token() between launches on the same buffers and never be 0.

@@ -49,6 +49,7 @@
 // their own loads.
 #include "rwkv_decode.h"
 
+#include <mutex>
 #include <type_traits>
 #include <vector>
 
@@ -59,7 +60,8 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 constexpr int kBW = 8;                 // back (streaming) waves per workgroup
 constexpr int kRealJobs = 13;          // tile jobs per layer: k v r | o | ffn_r, 4 x ffn_k | 4 quarters of ffn_v
 constexpr unsigned kSpinLimit = 1u << 20;
-constexpr int kLnRows = 2 + 3 * 3;     // rows of the XR record table
+constexpr int kStatRows = 4;           // XR rows 0-3: sum x and sum x^2 of a workgroup's channels, each as a (hi, lo) pair of float32
+constexpr int kLnRows = kStatRows + 3 * 3;     // rows of the XR record table
 constexpr int kEarlyDiv = 4;           // gathers start when all but G / kEarlyDiv workgroups have published (measured flat from G/20 to G)
 constexpr int kHeadCsPerThread = 4;    // head column sums a front thread fetches: 16 per head tile of the workgroup
 
@@ -355,17 +357,20 @@ __device__ __forceinline__ void publish_ln_input(u64 *X, u64 *XR, int G, int g, 
                                                  const float (&P)[NM], const double (&PO)[NM]) {
     put_word(X + 16 * g + n, epoch, (float)x);
     const double sx = row16_sum(x), sxx = row16_sum(x * x);
-    float val = (n == 0) ? (float)sx : (float)sxx;
+    // The sums travel as (hi, lo) float32 pairs: a single float32 would carry an error of 6e-8 of sum x^2 into
+    // the variance, which is far smaller than sum x^2 when the mean dwarfs the spread.
+    const float sxh = (float)sx, sxxh = (float)sxx;
+    float val = n == 0 ? sxh : (n == 1 ? (float)(sx - (double)sxh) : (n == 2 ? sxxh : (float)(sxx - (double)sxxh)));
 #pragma unroll
     for (int m = 0; m < NM; ++m) {
         const float mx = row16_max(fabsf((float)(x * (double)P[m])));
         const double so = row16_sum(x * PO[m]);
         const float hi = (float)so, lo = (float)(so - (double)hi);
-        if (n == 2 + 3 * m) val = mx;
-        if (n == 3 + 3 * m) val = hi;
-        if (n == 4 + 3 * m) val = lo;
+        if (n == kStatRows + 3 * m) val = mx;
+        if (n == kStatRows + 1 + 3 * m) val = hi;
+        if (n == kStatRows + 2 + 3 * m) val = lo;
     }
-    if (n < 2 + 3 * NM) put_word(XR + (size_t)n * G + g, epoch, val);
+    if (n < kStatRows + 3 * NM) put_word(XR + (size_t)n * G + g, epoch, val);
 }
 
 // The same for an epilogue wave whose four DPP rows all hold the same 16 channels (lane n of every
@@ -387,13 +392,14 @@ __device__ __forceinline__ void publish_ln_input_rows(u64 *X, u64 *XR, int G, in
     float val = (float)x;
     bool on = row == 0;
     if (row >= 1 && row <= NM && n < 3) {
-        dst = XR + (size_t)(2 + 3 * (row - 1) + n) * G + g;
+        dst = XR + (size_t)(kStatRows + 3 * (row - 1) + n) * G + g;
         val = n == 0 ? mc : (n == 1 ? hi : lo);
         on = true;
     }
-    if (row == 1 && (n == 3 || n == 4)) {
+    if (row == 1 && n >= 3 && n < 3 + kStatRows) {             // the statistics as (hi, lo) pairs, see publish_ln_input
         dst = XR + (size_t)(n - 3) * G + g;
-        val = n == 3 ? (float)sx : (float)sxx;
+        const float sxh = (float)sx, sxxh = (float)sxx;
+        val = n == 3 ? sxh : (n == 4 ? (float)(sx - (double)sxh) : (n == 5 ? sxxh : (float)(sxx - (double)sxxh)));
         on = true;
     }
     if (on) put_word(dst, epoch, val);
@@ -520,10 +526,10 @@ __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, co
     u64 w[NQT][4];
     const xtab_t xt = make_xtab(a.b.X, C);
     if (fx.wave == 0) {
-        RowPoll<2, G> r;
-        r.poll(fx, a.b.XR, epoch, seq, 2 * (G / kEarlyDiv), [&] { issue_quads<FT, NQT>(xt, fx.tid, 0, NQ, w); });
+        RowPoll<kStatRows, G> r;
+        r.poll(fx, a.b.XR, epoch, seq, kStatRows * (G / kEarlyDiv), [&] { issue_quads<FT, NQT>(xt, fx.tid, 0, NQ, w); });
         if (tp && fx.tid == 0) tp[0] = wall_clock64();
-        const double s0 = wave_sum_dpp(r.lane_sum(fx, 0)), s1 = wave_sum_dpp(r.lane_sum(fx, 1));
+        const double s0 = wave_sum_dpp(r.lane_sum(fx, 0) + r.lane_sum(fx, 1)), s1 = wave_sum_dpp(r.lane_sum(fx, 2) + r.lane_sum(fx, 3));
         const double mean = s0 * (1.0 / (double)C);
         double var = s1 * (1.0 / (double)C) - mean * mean;
         if (var < 0.0) var = 0.0;
@@ -535,7 +541,7 @@ __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, co
         const int m = fx.wave - 1;
         if (m < NM) {
             RowPoll<3, G> r;
-            r.poll(fx, a.b.XR + (size_t)(2 + 3 * m) * G, epoch);
+            r.poll(fx, a.b.XR + (size_t)(kStatRows + 3 * m) * G, epoch);
             const float mx = wave_max_dpp(r.lane_max(fx, 0));
             const double so = wave_sum_dpp(r.lane_sum(fx, 1) + r.lane_sum(fx, 2));
             if (fx.lane == 0) { stat[2 + 2 * m] = (double)mx; stat[3 + 2 * m] = so; }
@@ -1178,6 +1184,9 @@ bool decode_supported(int64_t L, int64_t C, int64_t F, int64_t V) {
 
 unsigned decode_epochs_per_token(int64_t L) { return (unsigned)(4 * L + 1); }
 
+// 8-byte words of the exchange buffers (X, XR, A, AR, H, HR), one contiguous range starting at X
+static size_t exchange_words(int64_t C, int64_t F) { return (size_t)(2 * C + F + (kLnRows + 6) * (C / 16)); }
+
 namespace {
 struct BlockPlan {
     size_t layers, prep, P32, Q32, PO, sc, X0, cs, ownrec, jt, scp, amax, xchg, abort, total;
@@ -1201,7 +1210,7 @@ BlockPlan plan_block(int64_t L, int64_t C, int64_t F, int64_t V) {
     p.jt = take(G * (size_t)(L + 1) * 16 * sizeof(u64));
     p.scp = take((size_t)L * (C / 512) * sizeof(DScal));
     p.amax = take((size_t)G * (sizeof(double) + sizeof(int)));
-    p.xchg = take(((size_t)2 * C + F + (size_t)(kLnRows + 6) * G) * sizeof(u64));
+    p.xchg = take(exchange_words(C, F) * sizeof(u64));
     p.abort = take(256);
     p.total = off;
     return p;
@@ -1294,21 +1303,43 @@ int decode_setup(void *block, const DSetup &s, DModel *dm, DecodeBuffers *db) {
     return RWKV_OK;
 }
 
+__global__ void __launch_bounds__(256) fill_zero_kernel(u64 *p, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0;
+}
+
+int decode_clear_exchange(hipStream_t st, const DModel &m, const DecodeBuffers &b) {
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(64), dim3(256), 0, st, b.X, exchange_words(m.C, m.F));
+    RWKV_CHECK_LAUNCH("fill_zero_kernel");
+    return RWKV_OK;
+}
+
+constexpr int kMaxDevices = 64;
+
 template <int KW, int FW>
 static int launch_one(hipStream_t st, const DArgs &args, bool with_prep) {
     const bool trace = args.b.trace != nullptr;
     const int lds = DecodeLds<KW, FW>::total(args.m.L, trace);
     if (lds > 160 * 1024) return set_error(RWKV_ERR_SIZE, "decode kernel: %d layers need %d bytes of LDS", args.m.L, lds);
-    static int configured = 0;
-    if (configured < lds) {     // the attribute only ever grows
-        RWKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_kernel<KW, FW, false>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        RWKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_kernel<KW, FW, true>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        configured = lds;
+    // the dynamic LDS limit is a per-device attribute of the function; it only ever grows
+    static std::mutex mu;
+    static int configured[kMaxDevices] = {};
+    int dev = 0;
+    RWKV_CHECK_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return set_error(RWKV_ERR_DEVICE, "decode kernel: device index %d", dev);
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        if (configured[dev] < lds) {
+            RWKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_kernel<KW, FW, false>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+            RWKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_kernel<KW, FW, true>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+            configured[dev] = lds;
+        }
     }
-    if (with_prep)
+    if (with_prep) {
         hipLaunchKernelGGL(prep_kernel, dim3((unsigned)(args.m.L * (args.m.C / kPrepThreads) + 1)), dim3(kPrepThreads), 0, st, args);
+        RWKV_CHECK_LAUNCH("prep_kernel");
+    }
     if (trace)
         hipLaunchKernelGGL((decode_kernel<KW, FW, true>), dim3((unsigned)args.m.G), dim3((FW + kBW) * 64), lds, st, args);
     else

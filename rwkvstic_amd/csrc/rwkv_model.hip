@@ -498,7 +498,10 @@ struct RowsWs {
 size_t rows_tot_ws_bytes(int64_t R, int64_t C, int64_t n_wide, int64_t n_head) {
     const size_t a = rows_tot_bytes(R, n_wide), b = 3 * rows_tot_bytes(R, C);     // k, v, r share a launch
     const size_t c = n_head > 0 ? rows_tot_bytes(1, n_head) : 0;
-    return a > b ? (a > c ? a : c) : (b > c ? b : c);
+    // the quantisers of the att output and of h park their partial records here before the product starts
+    const size_t q = rows_quant_scratch_bytes(R, n_wide > C ? n_wide : C);
+    const size_t m = a > b ? (a > c ? a : c) : (b > c ? b : c);
+    return m > q ? m : q;
 }
 
 // n_wide = widest product output (n_ffn, or the vocabulary when every row needs logits)
@@ -621,8 +624,21 @@ int rows_sequence(rwkv_model *m, hipStream_t st, const int64_t *tokens, int64_t 
     return RWKV_OK;
 }
 
+// The exchange words carry a 32-bit epoch that grows with every token step.  Before the counter would wrap
+// (after some 2^32 / (4 L + 1) steps) the exchange buffers are cleared and the count starts again at 1, so no
+// step ever runs under a tag an older word could still carry, and never under tag 0 (cleared memory).
+int fused_epochs(rwkv_model *m, hipStream_t st, int64_t steps) {
+    const uint64_t need = (uint64_t)steps * decode_epochs_per_token(m->d.n_layer);
+    if (need >= 0xffffffffull) return set_error(RWKV_ERR_SIZE, "too many token steps in one call");
+    if ((uint64_t)m->epoch + need < 0xffffffffull) return RWKV_OK;
+    RWKV_TRY(decode_clear_exchange(st, m->dm, m->db));
+    m->epoch = 1;
+    return RWKV_OK;
+}
+
 // One token through the persistent kernel (argument checks done by the caller).
 int fused_token(rwkv_model *m, hipStream_t st, const int64_t *token, double *state, double *logits) {
+    RWKV_TRY(fused_epochs(m, st, 1));
     const int rc = decode_launch(st, m->dm, m->db, m->epoch, token, state, logits);
     m->epoch += decode_epochs_per_token(m->d.n_layer);
     return rc;
@@ -695,7 +711,13 @@ int rwkv_model_check(rwkv_model *m) {
     if (!m->fused) return RWKV_OK;
     unsigned flag = 0;
     RWKV_CHECK_HIP(hipMemcpy(&flag, m->db.abort_flag, sizeof(flag), hipMemcpyDeviceToHost));
-    if (flag) return set_error(RWKV_ERR_HIP, "a single-token launch gave up waiting for another workgroup");
+    if (flag) {
+        // reported once: the flag is cleared so that later token steps run again (every wait of the kernel also
+        // leaves when it sees the flag, so a set flag would cut every following step short)
+        RWKV_CHECK_HIP(hipMemset(m->db.abort_flag, 0, sizeof(flag)));
+        return set_error(RWKV_ERR_HIP, "a single-token launch gave up waiting for another workgroup; logits and "
+                                       "state written since the last check are invalid");
+    }
     return RWKV_OK;
 }
 
@@ -789,8 +811,18 @@ int rwkv_gemm8(rwkv_stream_t stream, int64_t T, int64_t n_in, int64_t n_out, con
 
 size_t rwkv_gemm8_workspace_bytes(int64_t T, int64_t n_in, int64_t n_out) {
     if (T <= 0 || n_in <= 0 || n_out <= 0) return 0;
-    return round_up((size_t)T * 8, 256) * 3 + round_up(rows_dig_bytes(T, n_in), 256) +
-           round_up(rows_tot_bytes(T, n_out), 256);
+    const size_t tot = rows_tot_bytes(T, n_out), qs = rows_quant_scratch_bytes(T, n_in);   // share one area
+    return round_up((size_t)T * 8, 256) * 3 + round_up(rows_dig_bytes(T, n_in), 256) + round_up(tot > qs ? tot : qs, 256);
+}
+
+int rwkv_gemm8_plan(int64_t T, int64_t n_in, int64_t n_out, int n_products, int plan[4], size_t *tot_bytes_per_product) {
+    RWKV_CHECK_ARG(plan && tot_bytes_per_product, "rwkv_gemm8_plan: null pointer");
+    RWKV_CHECK_ARG(T > 0 && n_in > 0 && n_out > 0 && n_products >= 1 && n_products <= kRowsMaxProducts,
+                   "rwkv_gemm8_plan: bad sizes");
+    if (n_in % 64) return set_error(RWKV_ERR_SIZE, "rwkv_gemm8_plan: n_in must be a multiple of 64");
+    rows_plan_describe(T, n_in, n_out, n_products, plan);
+    *tot_bytes_per_product = rows_tot_bytes(T, n_out);
+    return RWKV_OK;
 }
 
 int rwkv_model_decode_greedy(rwkv_model *m, rwkv_stream_t stream, int64_t *tokens, int64_t n, double *state,
@@ -800,6 +832,7 @@ int rwkv_model_decode_greedy(rwkv_model *m, rwkv_stream_t stream, int64_t *token
     RWKV_CHECK_ARG(n > 0, "rwkv_model_decode_greedy: n must be positive");
     const Workspace w = carve(workspace, m->d.n_embd, m->d.n_ffn);
     if (m->fused) {
+        if ((rc = fused_epochs(m, (hipStream_t)stream, n))) return rc;
         rc = decode_launch_greedy((hipStream_t)stream, m->dm, m->db, m->epoch, tokens, n, state, logits);
         m->epoch += (unsigned)n * decode_epochs_per_token(m->d.n_layer);
         return rc;

@@ -22,6 +22,9 @@ constexpr int kRowsMaxProducts = 3;     // products of equal shape and tail that
 size_t rows_dig_bytes(int64_t R, int64_t K);
 size_t rows_tot_bytes(int64_t R, int64_t N);        // integer totals of ONE product (times the products in a launch)
 size_t rows_wkv_scratch_bytes(int64_t R, int64_t C);
+size_t rows_quant_scratch_bytes(int64_t R, int64_t K);   // what rows_quant writes into its scratch area (0: unused)
+// The plan rows_products follows for n products [R, K] x [K, N]: out = {kernel kind, grid x, grid y, splits}.
+void rows_plan_describe(int64_t R, int64_t K, int64_t N, int n, int out[4]);
 bool rows_ln_width_supported(int64_t C);            // widths the fused LayerNorm + mix + quantise kernel holds in registers
 
 int rows_embed(hipStream_t st, const int64_t *tokens, int64_t R, int V, int C, const float *emb, const double *w,
@@ -34,7 +37,7 @@ int rows_ln_mix_quant(hipStream_t st, int n_mix, int64_t R, int C, bool sequence
                       int64_t prev_stride, const float *const *range, const double *const *offset,
                       const RowsOperand *out);
 // Rows of float64 values quantised for a matrix with the given per-input-channel range / offset.
-// scratch: 16 * R * ceil(K / 3072) bytes (any buffer free until the product starts, e.g. its totals), or null.
+// scratch: rows_quant_scratch_bytes(R, K) bytes (any buffer free until the product starts, e.g. its totals), or null.
 int rows_quant(hipStream_t st, int64_t R, int64_t K, const double *in, const float *range, const double *offset,
                const RowsOperand &out, double *scratch);
 // n (<= kRowsMaxProducts) products of the same shape [R, K] x [K, N] and tail in one launch;

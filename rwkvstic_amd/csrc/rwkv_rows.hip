@@ -1090,21 +1090,61 @@ constexpr int kMaxSplit = 8;
 #define RWKV_GEMM_FILL 256
 #endif
 constexpr int kGemmFillWgs = RWKV_GEMM_FILL;   // the contraction is split until the grid has this many workgroups
-// Upper bound of the number of contraction splits rows_matmul will choose for R rows and N columns:
-// each split writes its own slice of totals (summed by the tail kernel), so the buffer has that many.
+
+// Which kernel serves n products of MT row tiles x NT column tiles over KB contraction blocks, its grid and
+// the number of contraction splits.  The ONE place these are decided: the launches and the sizing of the
+// totals buffer both call it, so the buffer always holds every slice the kernel writes.
+enum { PLAN_VEC = 0, PLAN_SKINNY, PLAN_GENERAL, PLAN_WIDE };
+struct ProductPlan { int kind, gx, gy, split; };
+static ProductPlan plan_products(int64_t MT, int64_t NT, int64_t KB, int n) {
+    ProductPlan p;
+    p.split = 1;
+    if (MT <= kVecMT) {
+        // a handful of rows: one 16-column tile per workgroup; only products with fewer tiles than compute
+        // units split the contraction (their integer slices are added by the tail kernel)
+        p.kind = PLAN_VEC; p.gx = (int)NT; p.gy = 1;
+        while (NT * n * p.split < kVecFillWgs && KB / (p.split * 2) >= 8 && p.split < kMaxSplit) p.split *= 2;
+        return p;
+    }
+    p.gy = (int)ceil_div(MT, 16);
+    p.kind = MT <= kSkinnyMT ? PLAN_SKINNY : PLAN_GENERAL;      // few rows: the weight-streaming variant
+    if (p.kind == PLAN_GENERAL) {
+        // Rounds of workgroups on 256 compute units, in matrix instructions per step: two general workgroups
+        // share a compute unit (2 x 32), a wide one has it alone (40).
+        const int64_t w4 = ceil_div(NT, kGemmNT) * p.gy * n, w5 = ceil_div(NT, kGemmWideNT) * p.gy * n;
+        const int64_t rem = w4 % 512;
+        const int64_t cost4 = (w4 / 512) * 64 + (rem == 0 ? 0 : rem <= 256 ? 32 : 64), cost5 = ceil_div(w5, 256) * 40;
+        if (w4 >= 256 && RWKV_GEMM_WIDE_NUM * cost5 < RWKV_GEMM_WIDE_DEN * cost4) p.kind = PLAN_WIDE;
+    }
+    p.gx = (int)ceil_div(NT, p.kind == PLAN_SKINNY ? kSkinnyNT : p.kind == PLAN_WIDE ? kGemmWideNT : kGemmNT);
+    // Split the contraction until the grid has a few workgroups per compute unit.
+    while ((int64_t)p.gx * p.gy * n * p.split < kGemmFillWgs && KB / (p.split * 2) >= 8 && p.split < kMaxSplit) p.split *= 2;
+    return p;
+}
+// Upper bound of the splits plan_products chooses for R rows and N columns, whatever the contraction length and
+// the number of products in the launch: a longer contraction only lifts the limit on the split, so the
+// plan for an unbounded one bounds every real one.
 static int gemm_split_bound(int64_t R, int64_t N) {
     const int64_t MT = ceil_div(R, 4), NT = ceil_div(N, 16);
     int s = 1;
-    if (MT <= kVecMT) {
-        while (NT * s < kVecFillWgs && s < kMaxSplit) s *= 2;
-        return s;
+    for (int n = 1; n <= kRowsMaxProducts; ++n) {
+        const int sp = plan_products(MT, NT, (int64_t)1 << 40, n).split;
+        if (sp > s) s = sp;
     }
-    const int64_t gx = ceil_div(NT, MT <= kSkinnyMT ? kSkinnyNT : kGemmNT), gy = ceil_div(MT, 16);
-    while (gx * gy * s < kGemmFillWgs && s < kMaxSplit) s *= 2;
     return s;
 }
 size_t rows_tot_bytes(int64_t R, int64_t N) {
     return (size_t)(ceil_div(R, 4) * 4 * round_up(N, 16) * 8) * (size_t)gemm_split_bound(R, N);
+}
+// What rows_quant keeps in its scratch area for R rows of K values (0: that shape does not use it).
+static bool quant_uses_parts(int64_t R, int64_t K) { return R <= 8 && K >= 8192; }
+size_t rows_quant_scratch_bytes(int64_t R, int64_t K) {
+    if (!quant_uses_parts(R, K)) return 0;
+    return (size_t)(R * ceil_div(K, 4 * kRT * kQuantPartSeg) * 2 * 8);
+}
+void rows_plan_describe(int64_t R, int64_t K, int64_t N, int n, int out[4]) {
+    const ProductPlan p = plan_products(ceil_div(R, 4), ceil_div(N, 16), K / 64, n);
+    out[0] = p.kind; out[1] = p.gx; out[2] = p.gy; out[3] = p.split;
 }
 
 int rows_embed(hipStream_t st, const int64_t *tokens, int64_t R, int V, int C, const float *emb, const double *w,
@@ -1161,7 +1201,7 @@ int rows_quant(hipStream_t st, int64_t R, int64_t K, const double *in, const flo
     QuantArgs q;
     q.K = (int)K; q.in = in; q.range = range; q.offset = offset; q.dig = out.dig; q.S = out.S; q.qs = out.qs; q.zp = out.zp;
     const dim3 grid((unsigned)R), block(kRT);
-    if (scratch && R <= 8 && K >= 8192) {
+    if (scratch && quant_uses_parts(R, K)) {
         QuantPartArgs pa;
         pa.q = q; pa.G = (int)ceil_div(K, 4 * kRT * kQuantPartSeg); pa.quads_per_part = (int)ceil_div(K / 4, pa.G);
         pa.part = scratch;
@@ -1197,43 +1237,25 @@ int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, i
     g.MT = (int)ceil_div(R, 4); g.NT = (int)ceil_div(N, 16); g.KB = (int)(K / 64); g.ldd = g.NT * 16;
     const int gy = (int)ceil_div(g.MT, 16);
     g.R = (int)R; g.N = (int)N; g.gate = gate;
-    int split = 1;
-    if (g.MT <= kVecMT) {
-        // a handful of rows: one 16-column tile per workgroup; only products with fewer tiles than compute
-        // units split the contraction (their integer slices are added by the tail kernel)
-        while (g.NT * n * split < kVecFillWgs && g.KB / (split * 2) >= 8 && split < kMaxSplit) split *= 2;
-        g.kb_per_split = (int)ceil_div(g.KB, split);
-        g.split = split;
-        g.slice = (size_t)g.MT * 4 * g.ldd;
-        g.gx = g.NT; g.gy = 1; g.gz = split * n; g.by_rows = 0; g.per_xcd = 0;
-        g.tail = split > 1 ? -1 : op;
+    const ProductPlan pl = plan_products(g.MT, g.NT, g.KB, n);
+    const int split = pl.split;
+    g.kb_per_split = (int)ceil_div(g.KB, split);
+    g.split = split;
+    g.slice = (size_t)g.MT * 4 * g.ldd;
+    g.gz = split * n;
+    g.tail = split > 1 ? -1 : op;
+    if (pl.kind == PLAN_VEC) {
+        g.gx = g.NT; g.gy = 1; g.by_rows = 0; g.per_xcd = 0;
         const dim3 grid((unsigned)(g.NT * g.gz));
         if (g.MT == 1) hipLaunchKernelGGL((gemv16_kernel<1, 8>), grid, dim3(256), 0, st, g);
         else hipLaunchKernelGGL((gemv16_kernel<2, 8>), grid, dim3(256), 0, st, g);
         RWKV_CHECK_LAUNCH("gemv16_kernel");
     } else {
-        const bool skinny = g.MT <= kSkinnyMT;              // few rows: the weight-streaming variant
-        bool wide = false;
-        if (!skinny) {
-            // Rounds of workgroups on 256 compute units, in matrix instructions per step: two general workgroups
-            // share a compute unit (2 x 32), a wide one has it alone (40).
-            const int w4 = (int)ceil_div(g.NT, kGemmNT) * gy * n, w5 = (int)ceil_div(g.NT, kGemmWideNT) * gy * n;
-            const int rem = w4 % 512;
-            const int cost4 = (w4 / 512) * 64 + (rem == 0 ? 0 : rem <= 256 ? 32 : 64), cost5 = (int)ceil_div(w5, 256) * 40;
-            wide = w4 >= 256 && RWKV_GEMM_WIDE_NUM * cost5 < RWKV_GEMM_WIDE_DEN * cost4;
-        }
-        const int gx = (int)ceil_div(g.NT, skinny ? kSkinnyNT : wide ? kGemmWideNT : kGemmNT);
-        // Split the contraction until the grid has a few workgroups per compute unit.
-        while (gx * gy * n * split < kGemmFillWgs && g.KB / (split * 2) >= 8 && split < kMaxSplit) split *= 2;
-        g.kb_per_split = (int)ceil_div(g.KB, split);
-        g.split = split;
-        g.slice = (size_t)g.MT * 4 * g.ldd;
-        g.gx = gx; g.gy = gy; g.gz = split * n; g.by_rows = gy >= kXcds;
-        g.per_xcd = ((g.by_rows ? gy : gx) + kXcds - 1) / kXcds;
-        g.tail = split > 1 ? -1 : op;
-        const dim3 grid((unsigned)(kXcds * g.per_xcd * (g.by_rows ? gx : gy) * g.gz));
-        if (skinny) hipLaunchKernelGGL(gemm8_skinny_kernel, grid, dim3(256), 0, st, g);
-        else if (wide) hipLaunchKernelGGL(gemm8_wide_kernel, grid, dim3(512), 0, st, g);
+        g.gx = pl.gx; g.gy = gy; g.by_rows = gy >= kXcds;
+        g.per_xcd = ((g.by_rows ? gy : pl.gx) + kXcds - 1) / kXcds;
+        const dim3 grid((unsigned)(kXcds * g.per_xcd * (g.by_rows ? pl.gx : gy) * g.gz));
+        if (pl.kind == PLAN_SKINNY) hipLaunchKernelGGL(gemm8_skinny_kernel, grid, dim3(256), 0, st, g);
+        else if (pl.kind == PLAN_WIDE) hipLaunchKernelGGL(gemm8_wide_kernel, grid, dim3(512), 0, st, g);
         else hipLaunchKernelGGL(gemm8_kernel, grid, dim3(512), 0, st, g);
         RWKV_CHECK_LAUNCH("gemm8_kernel");
     }

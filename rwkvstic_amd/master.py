@@ -106,7 +106,15 @@ class RWKVMaster:
                 break
             if stopStrings and text.endswith(tuple(stopStrings)):
                 break
+        self._raise_if_aborted()
         return {"logits": logits, "state": ostate, "output": text}
+
+    def _raise_if_aborted(self):
+        """A model whose token kernel can give up waiting (bounded waits) reports it here, once the results
+        have been pulled to the host anyway: nothing computed since the last check is valid then."""
+        check = getattr(self.model, "check", None)
+        if callable(check):
+            check()
 
     # ------------------------------------------------------------------ prompt (rwkvMaster.py:58-105)
     def loadContext(self, newctx="", ctx="\n\n", statex=None, progressCallBack: Callable = lambda x: x,
@@ -120,6 +128,7 @@ class RWKVMaster:
             chunk = new_ids[i:i + max(1, batch)]
             _, state = self.model.forward(chunk, state)
             progressCallBack(chunk)
+        self._raise_if_aborted()
         self.myState = _clone(state)
         return new_ids, _clone(state)
 

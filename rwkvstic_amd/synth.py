@@ -2,7 +2,10 @@
 
 There are no pretrained weights offline, so every test and benchmark runs on
 models drawn here: matrices and embedding ~N(0, 0.02), ``time_decay`` ~U(-5, 1),
-``time_first`` ~U(-1, 1), every ``time_mix_*`` ~U(0, 1), LayerNorm gamma=1 beta=0.
+``time_first`` ~U(-1, 1), every ``time_mix_*`` ~U(0, 1); LayerNorm gamma=1 beta=0 with
+``ln="identity"`` (the benchmark configurations), or gamma ~U(0.5, 1.5), beta ~N(0, 0.1)
+drawn separately for every LayerNorm with ``ln="random"`` (what a trained checkpoint looks like
+to the kernels: every weight and bias path carries a non-trivial value).
 The key names and shapes are the ones ``OptRWKV`` reads
 (reference src/rwkvstic/agnostic/backends/opt.py:34-48, modules/block.py:13-47).
 """
@@ -21,11 +24,17 @@ SHAPES = {
 
 
 def iter_tensors(layers: int, C: int, F: int, V: int, seed: int = 0,
-                 device: str = "cpu") -> Iterator[Tuple[str, torch.Tensor]]:
+                 device: str = "cpu", ln: str = "identity") -> Iterator[Tuple[str, torch.Tensor]]:
     """Yield ``(key, tensor)`` pairs one at a time (large shapes never need the
     whole float32 checkpoint resident)."""
+    if ln not in ("identity", "random"):
+        raise ValueError("ln must be 'identity' or 'random'")
     g = torch.Generator(device=device)
     g.manual_seed(seed)
+    # LayerNorm parameters come from a generator of their own, so that the matrices of a seed are the same
+    # in both modes
+    gl = torch.Generator(device=device)
+    gl.manual_seed(seed + 104729)
 
     def normal(*shape):
         return torch.randn(*shape, generator=g, device=device, dtype=torch.float32) * 0.02
@@ -33,8 +42,15 @@ def iter_tensors(layers: int, C: int, F: int, V: int, seed: int = 0,
     def uniform(lo, hi, *shape):
         return torch.rand(*shape, generator=g, device=device, dtype=torch.float32) * (hi - lo) + lo
 
-    ones = lambda: torch.ones(C, dtype=torch.float32, device=device)
-    zeros = lambda: torch.zeros(C, dtype=torch.float32, device=device)
+    def ones():
+        if ln == "random":
+            return torch.rand(C, generator=gl, device=device, dtype=torch.float32) + 0.5
+        return torch.ones(C, dtype=torch.float32, device=device)
+
+    def zeros():
+        if ln == "random":
+            return torch.randn(C, generator=gl, device=device, dtype=torch.float32) * 0.1
+        return torch.zeros(C, dtype=torch.float32, device=device)
 
     yield "emb.weight", normal(V, C)
     yield "blocks.0.ln0.weight", ones()
@@ -65,9 +81,9 @@ def iter_tensors(layers: int, C: int, F: int, V: int, seed: int = 0,
 
 
 def make_state_dict(layers: int, C: int, F: int | None = None, V: int = 50277,
-                    seed: int = 0, device: str = "cpu") -> Dict[str, torch.Tensor]:
+                    seed: int = 0, device: str = "cpu", ln: str = "identity") -> Dict[str, torch.Tensor]:
     F = 4 * C if F is None else F
-    return dict(iter_tensors(layers, C, F, V, seed, device))
+    return dict(iter_tensors(layers, C, F, V, seed, device, ln))
 
 
 def random_tokens(n: int, V: int = 50277, seed: int = 0) -> torch.Tensor:

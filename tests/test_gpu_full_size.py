@@ -26,7 +26,7 @@ def model3b():
     from rwkvstic_amd.model import HipRWKV
     L, C, F, V = synth.SHAPES["3B"]
     _say("building the 3B-shape model")
-    m = HipRWKV(synth.iter_tensors(L, C, F, V, seed=0, device="cuda"), device="cuda:0")
+    m = HipRWKV(synth.iter_tensors(L, C, F, V, seed=0, device="cuda", ln="random"), device="cuda:0")
     assert m.fused_step
     return m
 
@@ -70,7 +70,7 @@ def test_3b_fused_and_phase_kernels_agree_on_decode(model3b):
     from rwkvstic_amd.model import HipRWKV
     m = model3b
     L, C, F, V = synth.SHAPES["3B"]
-    plain = HipRWKV(synth.iter_tensors(L, C, F, V, seed=0, device="cuda"), device="cuda:0", fused=False)
+    plain = HipRWKV(synth.iter_tensors(L, C, F, V, seed=0, device="cuda", ln="random"), device="cuda:0", fused=False)
     assert not plain.fused_step
     sa, sb = m.emptyState.clone(), plain.emptyState.clone()
     for t in synth.random_tokens(4, V=V, seed=12).tolist():
@@ -108,7 +108,7 @@ def test_3b_width_two_layers_against_oracle():
     """Full width and vocabulary, 2 layers: what the CPU oracle finishes in seconds."""
     from rwkvstic_amd.model import HipRWKV
     _, C, F, V = synth.SHAPES["3B"]
-    sd = synth.make_state_dict(2, C, F, V, seed=3)
+    sd = synth.make_state_dict(2, C, F, V, seed=3, ln="random")
     ref = O.OracleModel(sd)
     exact = O.OracleModel(sd, matmul_dtype=torch.float64)
     hip = HipRWKV(sd)
@@ -135,7 +135,7 @@ def test_14b_width_two_layers_prompt_chunks_batch_and_oracle():
     kernels (their few-row product variant), one step of a batch of independent states, all against the CPU oracle."""
     from rwkvstic_amd.model import HipRWKV
     _, C, F, V = synth.SHAPES["14B"]
-    sd = synth.make_state_dict(2, C, F, V, seed=4)
+    sd = synth.make_state_dict(2, C, F, V, seed=4, ln="random")
     ref = O.OracleModel(sd)
     exact = O.OracleModel(sd, matmul_dtype=torch.float64)
     hip = HipRWKV(sd)

@@ -35,7 +35,7 @@ def _state_close(st_gpu, st_ref, tol=NOISY_STATE_TOL):
 @pytest.fixture(scope="module")
 def tiny():
     from rwkvstic_amd.model import HipRWKV
-    sd = synth.make_state_dict(layers=3, C=64, V=512, seed=5)
+    sd = synth.make_state_dict(layers=3, C=64, V=512, seed=5, ln="random")
     return O.OracleModel(sd), HipRWKV(sd)
 
 
@@ -72,7 +72,7 @@ def test_tiny_chunked_prefill_matches_oracle_and_single_steps(tiny):
 def test_ragged_shape_model():
     """C not a multiple of 128, V not a multiple of 8, F != 4C."""
     from rwkvstic_amd.model import HipRWKV
-    sd = synth.make_state_dict(layers=2, C=72, F=200, V=301, seed=8)
+    sd = synth.make_state_dict(layers=2, C=72, F=200, V=301, seed=8, ln="random")
     ref, hip = O.OracleModel(sd), HipRWKV(sd)
     toks = synth.random_tokens(6, V=301, seed=1).tolist()
     sr, sg = ref.emptyState.clone(), hip.emptyState.clone()
@@ -110,8 +110,9 @@ def test_169m_shape_greedy_128_tokens():
     """The plumbing configuration: 12 layers, C=768, F=3072, V=50277; 32-token prompt, 128 greedy tokens."""
     from rwkvstic_amd.model import HipRWKV
     L, C, F, V = synth.SHAPES["169M"]
-    sd = synth.make_state_dict(L, C, F, V, seed=0)
+    sd = synth.make_state_dict(L, C, F, V, seed=0)          # the configuration as stated: LayerNorm weight 1, bias 0
     ref, hip = O.OracleModel(sd), HipRWKV(sd)
+    exact = O.OracleModel(sd, matmul_dtype=torch.float64)
     assert hip.weight_bytes() == 130_625_280
     prompt = synth.random_tokens(32, V=V, seed=0).tolist()
     _say("169M oracle greedy (CPU) ...")
@@ -131,14 +132,23 @@ def test_169m_shape_greedy_128_tokens():
     assert toks_g == toks_r, "greedy tokens differ from the CPU oracle"
     assert worst <= LOGIT_TOL
     _state_close(st, st_r)
+    # the 1e-4 bound on the state holds against the same network with exact (float64) accumulation: the float32
+    # path above is itself only reproducible to NOISY_STATE_TOL
+    _say("169M oracle with float64 accumulation, same tokens ...")
+    st_e = exact.emptyState.clone()
+    _, st_e = exact.forward(prompt, st_e)
+    for t in toks_g:
+        le, st_e = exact.forward([t], st_e)
+    assert (lg.cpu() - le).abs().max() < 1e-4
+    _state_close(st, st_e, tol=STATE_TOL)
 
 
 # ------------------------------------------------------------------ persistent single-token kernel
-@pytest.mark.parametrize("C,L,V", [(1024, 2, 1999), (2560, 2, 5003), (2048, 1, 1600)])
+@pytest.mark.parametrize("C,L,V", [(1024, 2, 1999), (2560, 2, 5003), (2048, 1, 1600), (4096, 1, 1777)])
 def test_fused_step_matches_oracle_and_phase_kernels(C, L, V):
     from rwkvstic_amd.model import HipRWKV
     _say(f"fused step C={C} L={L} V={V}")
-    sd = synth.make_state_dict(L, C, 4 * C, V, seed=C + L)
+    sd = synth.make_state_dict(L, C, 4 * C, V, seed=C + L, ln="random")
     ref = O.OracleModel(sd)
     exact = O.OracleModel(sd, matmul_dtype=torch.float64)
     hip = HipRWKV(sd)
@@ -158,7 +168,12 @@ def test_fused_step_matches_oracle_and_phase_kernels(C, L, V):
         e_pl = float((lg - lp).abs().max())
         _say(f"  token {i}: |fused-fp32 oracle| {e_ref:.2e}  |fused-fp64 oracle| {e_ex:.2e}  |fused-phase| {e_pl:.2e}"
              f"  (|fp32 oracle-fp64 oracle| {float((lr - le).abs().max()):.2e})")
-        assert e_ref < LOGIT_TOL and e_pl < LOGIT_TOL
+        # Against the float32 CPU path the bound is 1e-3, unless that path's own float32 summation noise (its
+        # distance from the same network with exact accumulation, printed above) is already of that size, as at
+        # C=4096 with LayerNorm weights up to 1.5: then the kernel must sit within 5e-4 of the noise, and the
+        # comparison that binds is the 1e-4 one against exact accumulation.
+        noise = float((lr - le).abs().max())
+        assert e_ref < max(LOGIT_TOL, noise + 5e-4) and e_pl < LOGIT_TOL
         assert e_ex < 1e-4
         assert int(lg.argmax()) == int(lr.argmax())
     _state_close(sg, sr)
@@ -171,12 +186,87 @@ def test_fused_step_matches_oracle_and_phase_kernels(C, L, V):
     assert torch.equal(l2, lg) and torch.equal(s2, sg)
 
 
+def test_fused_kernel_128_greedy_tokens_match_both_oracles():
+    """The kernel the benchmark times, held to the parity statement itself: after a 32-token prompt, 128 greedy
+    tokens through the persistent single-token kernel are the oracle's tokens, every logits vector is within
+    1e-3 of the float32 CPU path, and the final state within 1e-4 of the same network with exact accumulation
+    (its WKV sums and sigmoids are float32 where block.py:72 and operators.cu:21-36 are float64: this is the run
+    that bounds the drift)."""
+    from rwkvstic_amd.model import HipRWKV
+    L, C, V = 4, 1024, 2003
+    sd = synth.make_state_dict(L, C, 4 * C, V, seed=321, ln="random")
+    ref, exact, hip = O.OracleModel(sd), O.OracleModel(sd, matmul_dtype=torch.float64), HipRWKV(sd)
+    assert hip.fused_step
+    prompt = synth.random_tokens(32, V=V, seed=6).tolist()
+    toks_r, logits_r, st_r = ref.greedy(prompt, 128)
+    st = hip.emptyState.clone()
+    for t in prompt:                                   # the prompt too goes token by token through the kernel
+        lg, st = hip.forward([t], st)
+    toks_g, worst = [], 0.0
+    for i in range(128):
+        worst = max(worst, float((lg.cpu() - logits_r[i]).abs().max()))
+        t = int(lg.argmax())
+        toks_g.append(t)
+        lg, st = hip.forward([t], st)
+    hip.check()
+    worst = max(worst, float((lg.cpu() - logits_r[128]).abs().max()))
+    _say(f"fused kernel, 160 tokens: worst logit max-abs vs float32 oracle {worst:.3e}")
+    assert toks_g == toks_r
+    assert worst <= LOGIT_TOL
+    _state_close(st, st_r)
+    st_e = exact.emptyState.clone()
+    for t in prompt + toks_g:
+        le, st_e = exact.forward([t], st_e)
+    e_ex = float((lg.cpu() - le).abs().max())
+    _say(f"fused kernel, 160 tokens: final logits vs float64-accumulation oracle {e_ex:.3e}")
+    assert e_ex < 1e-4
+    _state_close(st, st_e, tol=STATE_TOL)
+    # the device-side greedy loop produces the same 128 tokens
+    s2 = hip.emptyState.clone()
+    for t in prompt[:-1]:
+        _, s2 = hip.forward([t], s2)
+    toks_d, _, s2 = hip.decode_greedy(prompt[-1], 128, s2)
+    hip.check()
+    assert toks_d.tolist() == toks_r
+
+
+@pytest.mark.parametrize("kind", ["offset", "outliers"])
+def test_fused_kernel_layernorm_with_large_mean(kind):
+    """LayerNorm inputs whose mean dwarfs their spread (every channel of the residual stream shifted by +30
+    through the ln0 bias) or with a few huge channels: the statistics travel between workgroups as partial sums,
+    and a variance formed as E[x^2] - mean^2 from rounded partials would lose digits here (layernorm.py:11-20
+    subtracts the mean first)."""
+    from rwkvstic_amd.model import HipRWKV
+    L, C, V = 2, 1024, 1500
+    sd = synth.make_state_dict(L, C, 4 * C, V, seed=99, ln="random")
+    if kind == "offset":
+        sd["blocks.0.ln0.bias"] = sd["blocks.0.ln0.bias"] + 30.0
+    else:
+        sd["blocks.0.ln0.bias"][[3, 500, 1023]] += torch.tensor([300.0, -250.0, 400.0])
+    exact, hip = O.OracleModel(sd, matmul_dtype=torch.float64), HipRWKV(sd)
+    assert hip.fused_step
+    toks = synth.random_tokens(8, V=V, seed=8).tolist()
+    se, sg = exact.emptyState.clone(), hip.emptyState.clone()
+    for t in toks:
+        le, se = exact.forward([t], se)
+        lg, sg = hip.forward([t], sg)
+    hip.check()
+    err = float((lg.cpu() - le).abs().max())
+    _say(f"large-mean LayerNorm ({kind}): |dlogits| vs float64-accumulation oracle {err:.3e}")
+    assert err < 1e-4
+    _state_close(sg, se, tol=STATE_TOL)
+    # the many-row path on the same model
+    lp, sp = hip.forward(toks, hip.emptyState.clone())
+    assert float((lp.cpu() - le).abs().max()) < 1e-4
+    _state_close(sp, se, tol=STATE_TOL)
+
+
 def test_fused_greedy_device_loop_matches_host_loop():
     """rwkv_model_decode_greedy on the persistent kernel: argmax and the preparation of the next step run in one
     launch between the token kernels; tokens, logits and state must equal forward() + host argmax, bit for bit
     (rwkvMaster.py:28-56 with the sampler replaced by argmax)."""
     from rwkvstic_amd.model import HipRWKV
-    sd = synth.make_state_dict(2, 1024, 4096, 1999, seed=77)
+    sd = synth.make_state_dict(2, 1024, 4096, 1999, seed=77, ln="random")
     hip = HipRWKV(sd)
     assert hip.fused_step
     s1 = hip.emptyState.clone()
@@ -234,7 +324,7 @@ def test_prompt_longer_than_one_pass(tiny):
 def test_prompt_gemm_path_mid_shape_vs_fp64_oracle():
     """C=256, F=1024, ragged vocabulary; 70 tokens (18 M-tiles: a partial 64-token workgroup tile)."""
     from rwkvstic_amd.model import HipRWKV
-    sd = synth.make_state_dict(layers=2, C=256, F=1024, V=1203, seed=21)
+    sd = synth.make_state_dict(layers=2, C=256, F=1024, V=1203, seed=21, ln="random")
     ref, hip = O.OracleModel(sd, matmul_dtype=torch.float64), HipRWKV(sd)
     toks = synth.random_tokens(70, V=1203, seed=2).tolist()
     lr, sr = ref.forward(toks, ref.emptyState.clone())
@@ -274,7 +364,7 @@ def test_rwkv_shell_loads_checkpoint_file_and_generates(tmp_path, tiny):
     """RWKV(path) -> RWKVMaster surface (load.py:18,42-47; rwkvMaster.py:28-105) over the HIP model."""
     from rwkvstic_amd.master import RWKV, greedy
     ref, hip = tiny
-    sd = synth.make_state_dict(layers=3, C=64, V=512, seed=5)
+    sd = synth.make_state_dict(layers=3, C=64, V=512, seed=5, ln="random")
     path = str(tmp_path / "tiny.pth")
     torch.save(sd, path)
     r = RWKV(path, sampler=greedy)
@@ -298,7 +388,7 @@ def test_quantized_tree_round_trip_and_oracle_layout(tmp_path, tiny):
     from rwkvstic_amd.master import RWKV, greedy
     from rwkvstic_amd.model import HipRWKV
     ref, hip = tiny
-    sd = synth.make_state_dict(layers=3, C=64, V=512, seed=5)
+    sd = synth.make_state_dict(layers=3, C=64, V=512, seed=5, ln="random")
     tree = hip.quantized_tree()
     assert tree["emptyState"].shape == (3, 5, 64) and tree["emb.w"].shape == (512, 64)
     assert tree["blocks.0.attmix"].shape == (3, 1, 64) and tree["blocks.2.ffnmix"].shape == (2, 1, 64)

@@ -164,7 +164,7 @@ def test_wkv_first_step_from_empty_state_is_v():
 # ---------------------------------------------------------------- model
 @pytest.fixture(scope="module")
 def tiny():
-    sd = synth.make_state_dict(layers=3, C=64, V=512, seed=5)
+    sd = synth.make_state_dict(layers=3, C=64, V=512, seed=5, ln="random")
     return sd, O.OracleModel(sd)
 
 
