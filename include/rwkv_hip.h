@@ -64,6 +64,21 @@ int rwkv_mm8_one(rwkv_stream_t stream, int64_t n_in, int64_t n_out,
                  float *y, const float *r,
                  void *workspace, size_t workspace_bytes);
 
+/* rwkv_mm8_one without a workspace argument and without any allocation, for
+ * callers that cannot allocate device memory: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart
+ * in the reference.  The partial sums go to a fixed array inside the library's
+ * device image (rwkv_mm8_one_static_max_bytes() = 12 MiB per GPU, held until
+ * the process ends); shapes that need more
+ * (rwkv_mm8_workspace_bytes(n_in, n_out, 1) > the maximum) are rejected with
+ * RWKV_ERR_SIZE.  Same arithmetic, same kernels and bit-identical results as
+ * rwkv_mm8_one.  All calls on one GPU share the array: calls that overlap on
+ * one GPU (two streams, two threads) race; calls on one stream do not. */
+size_t rwkv_mm8_one_static_max_bytes(void);
+int rwkv_mm8_one_static(rwkv_stream_t stream, int64_t n_in, int64_t n_out,
+                        const float *x, const uint8_t *w, int64_t w_stride,
+                        float *y, const float *r);
+
 /* mm8_three (wrapper.cpp:82-127, operators32.cu:44-104): three independent
  * (x, w, r, y) problems sharing n_in and n_out in one launch. */
 int rwkv_mm8_three(rwkv_stream_t stream, int64_t n_in, int64_t n_out,

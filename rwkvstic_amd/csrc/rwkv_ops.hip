@@ -2,6 +2,8 @@
 // and the reference-layout mm8_one / mm8_three drop-ins.
 #include "rwkv_common.h"
 
+#include <mutex>
+
 namespace rwkv {
 
 // ---------------------------------------------------------------------------
@@ -271,6 +273,34 @@ static int mm8_ref_launch(hipStream_t st, int nm, int64_t n_in, int64_t n_out,
     return RWKV_OK;
 }
 
+// ---------------------------------------------------------------------------
+// Scratch for callers that cannot hand over (or allocate) a workspace: a fixed array in the library's own
+// device image.  Every GPU the library runs on holds its own copy, at its own address, until the process
+// ends; the array's name below is only the host-side handle of the symbol, the device address comes from
+// hipGetSymbolAddress, once per device, with that device current.
+// ---------------------------------------------------------------------------
+constexpr size_t kStaticScratchBytes = (size_t)12 << 20;     // the [5120 x 50277] head of the 14B shape needs 8.05 MB
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kScratchMaxDevices = 64;
+static std::mutex scratch_mu;
+static void *scratch_ptr[kScratchMaxDevices] = {};
+
+static int static_scratch(void **out) {
+    int dev = 0;
+    RWKV_CHECK_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kScratchMaxDevices) return set_error(RWKV_ERR_DEVICE, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(scratch_mu);
+    if (!scratch_ptr[dev]) {
+        void *p = nullptr;
+        RWKV_CHECK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return set_error(RWKV_ERR_HIP, "hipGetSymbolAddress returned a null address for the scratch array");
+        scratch_ptr[dev] = p;
+    }
+    *out = scratch_ptr[dev];
+    return RWKV_OK;
+}
+
 }  // namespace rwkv
 
 using namespace rwkv;
@@ -290,6 +320,24 @@ int rwkv_mm8_one(rwkv_stream_t stream, int64_t n_in, int64_t n_out, const float 
     float *ys[3] = {y, y, y};
     const float *rs[3] = {r, r, r};
     return mm8_ref_launch((hipStream_t)stream, 1, n_in, n_out, xs, ws_, st, ys, rs, workspace, workspace_bytes);
+}
+
+size_t rwkv_mm8_one_static_max_bytes(void) { return kStaticScratchBytes; }
+
+int rwkv_mm8_one_static(rwkv_stream_t stream, int64_t n_in, int64_t n_out, const float *x, const uint8_t *w,
+                        int64_t w_stride, float *y, const float *r) {
+    RWKV_CHECK_ARG(n_in > 0 && n_out > 0 && n_in < (1 << 30) && n_out < (1 << 30), "mm8: bad sizes");
+    const size_t need = rwkv_mm8_workspace_bytes(n_in, n_out, 1);
+    if (need > kStaticScratchBytes)
+        return set_error(RWKV_ERR_SIZE, "rwkv_mm8_one_static: [%lld x %lld] needs %zu bytes of scratch, the built-in "
+                                        "array holds %zu; use rwkv_mm8_one with a workspace",
+                         (long long)n_in, (long long)n_out, need, kStaticScratchBytes);
+    void *ws = nullptr;
+    const int rc = static_scratch(&ws);
+    if (rc) return rc;
+    // every partial sum the reduce kernel reads is written by the partial kernel of the same call: nothing of
+    // an earlier call's contents is read, so the array needs no clearing
+    return rwkv_mm8_one(stream, n_in, n_out, x, w, w_stride, y, r, ws, kStaticScratchBytes);
 }
 
 int rwkv_mm8_three(rwkv_stream_t stream, int64_t n_in, int64_t n_out,
