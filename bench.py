@@ -68,6 +68,55 @@ def cpu_baseline(shape, threads: int):
     }
 
 
+def phase_trace(model, L: int, C: int) -> int:
+    """Where a token step of the persistent kernel spends its time: every workgroup stamps its phase boundaries
+    (100 MHz wall clock); the table gives, per boundary, the spread over the workgroups relative to the earliest
+    workgroup's start of the layer.  "X:stats" / "X:scale" = the records of the other workgroups have arrived,
+    "X:digits" = gathered and written as digit planes, "X:mfma" = the back waves have parked the tile sums,
+    "finX" = epilogue done and results published."""
+    import numpy as np
+    import torch
+    from rwkvstic_amd import _native as N
+    if not model.fused_step:
+        print("phase trace: this shape does not run the persistent kernel", file=sys.stderr)
+        return 2
+    G, per = C // 16, 24
+    st = model.emptyState.clone()
+    for t in range(5):
+        _, st = model.forward([t + 3], st)
+    buf = torch.zeros(G * L * per, dtype=torch.int64, device="cuda")
+    N.check(N.lib().rwkv_model_set_trace(model._handle, buf.data_ptr()))
+    model.forward([77], st)
+    torch.cuda.synchronize()
+    model.check()
+    N.check(N.lib().rwkv_model_set_trace(model._handle, None))
+    t = buf.cpu().numpy().astype("float64").reshape(G, L, per) * 0.01          # microseconds
+    names = ["start", "A:stats", "A:digits", "A:mfma", "finA", "B:scale", "B:digits", "B:mfma", "finB",
+             "C:stats", "C:digits", "C:mfma", "finC", "D:scale", "D:digits", "D:mfma"]
+    print("phases: A = att k, v, r   B = att output   C = ffn key + receptance   D = ffn value   (microseconds)")
+    for l in sorted({min(L - 1, 1), L // 2, L - 2 if L > 2 else L - 1}):
+        base = t[:, l, 0].min()
+        print(f"layer {l}")
+        prev = 0.0
+        for i, name in enumerate(names):
+            v = t[:, l, i] - base
+            med = float(np.median(v))
+            print(f"  {name:9s} min {v.min():6.2f}  med {med:6.2f}  max {v.max():6.2f}   (+{med - prev:5.2f} after the previous boundary)")
+            prev = med
+    if L > 3:
+        print(f"per layer, workgroup 0, layers 1..{L - 2}: {(t[0, L - 1, 0] - t[0, 1, 0]) / (L - 2):.2f} us")
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    one = torch.tensor([5], device="cuda")
+    e0.record()
+    for _ in range(50):
+        model.forward(one, st)
+    e1.record()
+    torch.cuda.synchronize()
+    model.check()
+    print(f"token step without stamps: {e0.elapsed_time(e1) / 50 * 1e3:.1f} us")
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -79,6 +128,10 @@ def main() -> int:
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="before the workload, copy this many MiB device to device once (a kernel of known HBM "
                          "traffic: the yardstick for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
+    ap.add_argument("--phase-trace", action="store_true",
+                    help="instead of the benchmark: one token step of the persistent kernel with its 100 MHz phase "
+                         "stamps switched on (rwkv_model_set_trace), printed as a table of min / median / max over "
+                         "the workgroups per phase boundary, for three layers")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (batch-1 decode of one model replica); "
@@ -101,6 +154,9 @@ def main() -> int:
 
     stream = torch.cuda.current_stream()
     ev = lambda: torch.cuda.Event(enable_timing=True)
+
+    if args.phase_trace:
+        return phase_trace(model, L, C)
 
     if args.calibrate_copy_mib > 0:
         n = args.calibrate_copy_mib << 20

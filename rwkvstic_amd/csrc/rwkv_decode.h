@@ -100,11 +100,13 @@ bool decode_supported(int64_t L, int64_t C, int64_t F, int64_t V);
 unsigned decode_epochs_per_token(int64_t L);
 constexpr int kTraceStampsPerLayer = 24;
 
-// Bytes of the single device allocation that holds tables, constants and exchange buffers.
+// Bytes of the single device allocation that holds tables and constants, and of the exchange buffers.
 size_t decode_block_bytes(int64_t L, int64_t C, int64_t F, int64_t V);
-// Fills `block` (device, decode_block_bytes, zero-filled by the caller) and the two descriptors.
+size_t decode_exchange_bytes(int64_t C, int64_t F);
+// Fills `block` (device, decode_block_bytes, zero-filled by the caller) and the two descriptors; `exchange`
+// (device, decode_exchange_bytes, zero-filled by the caller) becomes the exchange buffers.
 // Synchronises the device (model creation only).
-int decode_setup(void *block, const DSetup &s, DModel *dm, DecodeBuffers *db);
+int decode_setup(void *block, void *exchange, const DSetup &s, DModel *dm, DecodeBuffers *db);
 
 // Zero-fills the exchange buffers on the stream (a kernel, so the call may be captured); the next launch must
 // use epoch 1.

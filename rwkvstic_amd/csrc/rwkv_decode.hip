@@ -60,13 +60,13 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 constexpr int kBW = 8;                 // back (streaming) waves per workgroup
 constexpr int kRealJobs = 13;          // tile jobs per layer: k v r | o | ffn_r, 4 x ffn_k | 4 quarters of ffn_v
 constexpr unsigned kSpinLimit = 1u << 20;
-constexpr int kStatRows = 4;           // XR rows 0-3: sum x and sum x^2 of a workgroup's channels, each as a (hi, lo) pair of float32
+constexpr int kStatRows = 2;           // XR rows 0-1: sum x of a workgroup's 16 channels, and their squared deviations from the workgroup's own mean
 constexpr int kLnRows = kStatRows + 3 * 3;     // rows of the XR record table
 constexpr int kEarlyDiv = 4;           // gathers start when all but G / kEarlyDiv workgroups have published (measured flat from G/20 to G)
 constexpr int kHeadCsPerThread = 4;    // head column sums a front thread fetches: 16 per head tile of the workgroup
 
 // LDS flag words
-enum { FLAG_ARRIVED = 0, FLAG_SCALE = 1, FLAG_ABORT = 2, FLAG_COUNT = 4 };
+enum { FLAG_ARRIVED = 0, FLAG_SCALE = 1, FLAG_ABORT = 2, FLAG_ALL = 3, FLAG_COUNT = 4 };
 
 // Pointers that were themselves loaded from memory are "flat" to the compiler, and a flat load
 // counts against the LDS counter as well as the vector-memory counter: every wait for an LDS read
@@ -267,6 +267,19 @@ struct RowPoll {
                 if ((2 * (fx.lane + 64 * k) + j) / G == r) acc += (double)v[k][j];
         return acc;
     }
+    // this lane's share of sum over the words w of row r of 16 (w / 16 - mean)^2
+    __device__ __forceinline__ double lane_group_dev2(const Front &fx, int r, double mean) const {
+        double acc = 0.0;
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                if ((2 * (fx.lane + 64 * k) + j) / G == r && 2 * (fx.lane + 64 * k) + j < NR * G) {
+                    const double d = (double)v[k][j] * (1.0 / 16.0) - mean;
+                    acc += 16.0 * d * d;
+                }
+        return acc;
+    }
     __device__ __forceinline__ float lane_max(const Front &fx, int r) const {
         float acc = 0.f;
 #pragma unroll
@@ -356,11 +369,14 @@ template <int NM>
 __device__ __forceinline__ void publish_ln_input(u64 *X, u64 *XR, int G, int g, int n, unsigned epoch, double x,
                                                  const float (&P)[NM], const double (&PO)[NM]) {
     put_word(X + 16 * g + n, epoch, (float)x);
-    const double sx = row16_sum(x), sxx = row16_sum(x * x);
-    // The sums travel as (hi, lo) float32 pairs: a single float32 would carry an error of 6e-8 of sum x^2 into
-    // the variance, which is far smaller than sum x^2 when the mean dwarfs the spread.
-    const float sxh = (float)sx, sxxh = (float)sxx;
-    float val = n == 0 ? sxh : (n == 1 ? (float)(sx - (double)sxh) : (n == 2 ? sxxh : (float)(sxx - (double)sxxh)));
+    // The statistics travel as float32: the sum of the 16 channels and the sum of their squared deviations
+    // from the workgroup's OWN mean.  The consumer combines the groups (the parallel form of the variance),
+    // so no term is a difference of two numbers that are large against the spread, whatever the mean.
+    const double sx = row16_sum(x);
+    const float sxf = (float)sx;
+    const double dev = x - (double)sxf * (1.0 / 16.0);
+    const double m2 = row16_sum(dev * dev);
+    float val = n == 0 ? sxf : (float)m2;
 #pragma unroll
     for (int m = 0; m < NM; ++m) {
         const float mx = row16_max(fabsf((float)(x * (double)P[m])));
@@ -384,7 +400,9 @@ __device__ __forceinline__ void publish_ln_input_rows(u64 *X, u64 *XR, int G, in
                                                       float Pm, double POm) {
     static_assert(NM >= 1 && NM <= 3, "one row per product");
     const double sx = row16_sum(x);
-    const double sxx = row16_sum(x * x);
+    const float sxf = (float)sx;
+    const double dev = x - (double)sxf * (1.0 / 16.0);
+    const double m2 = row16_sum(dev * dev);
     const double so = row16_sum(x * POm);
     const float mc = row16_max(fabsf((float)(x * (double)Pm)));
     const float hi = (float)so, lo = (float)(so - (double)hi);
@@ -396,10 +414,9 @@ __device__ __forceinline__ void publish_ln_input_rows(u64 *X, u64 *XR, int G, in
         val = n == 0 ? mc : (n == 1 ? hi : lo);
         on = true;
     }
-    if (row == 1 && n >= 3 && n < 3 + kStatRows) {             // the statistics as (hi, lo) pairs, see publish_ln_input
+    if (row == 1 && (n == 3 || n == 4)) {                      // the statistics, see publish_ln_input
         dst = XR + (size_t)(n - 3) * G + g;
-        const float sxh = (float)sx, sxxh = (float)sxx;
-        val = n == 3 ? sxh : (n == 4 ? (float)(sx - (double)sxh) : (n == 5 ? sxxh : (float)(sxx - (double)sxxh)));
+        val = n == 3 ? sxf : (float)m2;
         on = true;
     }
     if (on) put_word(dst, epoch, val);
@@ -529,10 +546,10 @@ __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, co
         RowPoll<kStatRows, G> r;
         r.poll(fx, a.b.XR, epoch, seq, kStatRows * (G / kEarlyDiv), [&] { issue_quads<FT, NQT>(xt, fx.tid, 0, NQ, w); });
         if (tp && fx.tid == 0) tp[0] = wall_clock64();
-        const double s0 = wave_sum_dpp(r.lane_sum(fx, 0) + r.lane_sum(fx, 1)), s1 = wave_sum_dpp(r.lane_sum(fx, 2) + r.lane_sum(fx, 3));
-        const double mean = s0 * (1.0 / (double)C);
-        double var = s1 * (1.0 / (double)C) - mean * mean;
-        if (var < 0.0) var = 0.0;
+        // groups of 16 channels combined: mean of the group sums, variance from the groups' own squared
+        // deviations plus the spread of the group means
+        const double mean = wave_sum_dpp(r.lane_sum(fx, 0)) * (1.0 / (double)C);
+        const double var = wave_sum_dpp(r.lane_sum(fx, 1) + r.lane_group_dev2(fx, 0, mean)) * (1.0 / (double)C);
         const double rsd = 1.0 / sqrt(var + 1e-5);                 // layernorm.py:15-20
         if (fx.lane == 0) { stat[0] = mean; stat[1] = rsd; }
     } else {
@@ -1108,6 +1125,11 @@ __global__ void build_jobtab_kernel(const DLayer *__restrict__ layers, const uin
             const int tile = g + G * j;
             p = w_head + (size_t)(tile < v_tiles ? tile : 0) * TB;
         }
+#ifdef RWKV_DIAG_HOT_WEIGHTS
+        // Diagnostic build only (results are wrong): every job streams the same cache-resident tile, which
+        // takes HBM out of the picture and leaves the time of the dependency chain between the workgroups.
+        p = w_head;
+#endif
         jt[(size_t)g * (L + 1) * 16 + i] = (u64) reinterpret_cast<uintptr_t>(p);
     }
 }
@@ -1189,7 +1211,7 @@ static size_t exchange_words(int64_t C, int64_t F) { return (size_t)(2 * C + F +
 
 namespace {
 struct BlockPlan {
-    size_t layers, prep, P32, Q32, PO, sc, X0, cs, ownrec, jt, scp, amax, xchg, abort, total;
+    size_t layers, prep, P32, Q32, PO, sc, X0, cs, ownrec, jt, scp, amax, abort, total;
     size_t cs_layer_ints;
 };
 BlockPlan plan_block(int64_t L, int64_t C, int64_t F, int64_t V) {
@@ -1210,7 +1232,6 @@ BlockPlan plan_block(int64_t L, int64_t C, int64_t F, int64_t V) {
     p.jt = take(G * (size_t)(L + 1) * 16 * sizeof(u64));
     p.scp = take((size_t)L * (C / 512) * sizeof(DScal));
     p.amax = take((size_t)G * (sizeof(double) + sizeof(int)));
-    p.xchg = take(exchange_words(C, F) * sizeof(u64));
     p.abort = take(256);
     p.total = off;
     return p;
@@ -1218,8 +1239,9 @@ BlockPlan plan_block(int64_t L, int64_t C, int64_t F, int64_t V) {
 }  // namespace
 
 size_t decode_block_bytes(int64_t L, int64_t C, int64_t F, int64_t V) { return plan_block(L, C, F, V).total; }
+size_t decode_exchange_bytes(int64_t C, int64_t F) { return (size_t)round_up((int64_t)(exchange_words(C, F) * sizeof(u64)), 256); }
 
-int decode_setup(void *block, const DSetup &s, DModel *dm, DecodeBuffers *db) {
+int decode_setup(void *block, void *exchange, const DSetup &s, DModel *dm, DecodeBuffers *db) {
     const int64_t L = s.L, C = s.C, F = s.F, V = s.V;
     if (!decode_supported(L, C, F, V)) return set_error(RWKV_ERR_SIZE, "decode_setup: unsupported shape");
     const BlockPlan p = plan_block(L, C, F, V);
@@ -1290,7 +1312,7 @@ int decode_setup(void *block, const DSetup &s, DModel *dm, DecodeBuffers *db) {
                        dm->P32, dm->PO, (int)L, (int)C, (int)F, (int)G, reinterpret_cast<u64 *>(base + p.ownrec));
     RWKV_CHECK_LAUNCH("build_ownrec_kernel");
 
-    u64 *x = reinterpret_cast<u64 *>(base + p.xchg);
+    u64 *x = static_cast<u64 *>(exchange);
     db->X = x; x += C;
     db->XR = x; x += (size_t)kLnRows * G;
     db->A = x; x += C;

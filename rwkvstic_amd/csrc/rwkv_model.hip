@@ -27,6 +27,7 @@
 #include "rwkv_decode.h"
 #include "rwkv_rows.h"
 
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -347,7 +348,9 @@ struct rwkv_model {
     int device = 0;
     rwkv::DModel dm{};
     rwkv::DecodeBuffers db{};
-    void *dev_block = nullptr;     // one allocation: layer table + exchange vectors + abort flag
+    void *dev_block = nullptr;     // one allocation: layer table, constants, abort flag
+    void *xchg_block = nullptr;    // exchange vectors (uncached device memory from the pool below)
+    size_t xchg_bytes = 0;
     unsigned epoch = 0;
 };
 
@@ -449,6 +452,34 @@ int check_forward_args(const rwkv_model *m, const void *tokens, const double *st
 
 rwkv::DQ to_dq(const rwkv_qmat &q) { return rwkv::DQ{q.packed16, q.range, q.offset}; }
 
+// The exchange vectors of the persistent kernel live in uncached device memory: every access to them is
+// an agent-coherent one that must not be served from an XCD's own L2, and on uncached pages such accesses
+// go straight to the memory side, which shortens the polls (measured: a chip-wide flag barrier under a
+// running weight stream takes 4.4 us on uncached pages against 6.0 us on ordinary ones).  Uncached
+// allocations are never freed while the process lives (freeing one that a kernel has read has left later
+// allocations with wrong contents on this platform): blocks go back to a per-device pool and are reused.
+#define RWKV_TRY(expr) do { const int rc_ = (expr); if (rc_) return rc_; } while (0)
+
+struct XchgBlock { int device; size_t bytes; void *ptr; bool busy; };
+std::mutex xchg_mu;
+std::vector<XchgBlock> xchg_pool;
+
+int xchg_acquire(int device, size_t bytes, void **out) {
+    std::lock_guard<std::mutex> lock(xchg_mu);
+    for (XchgBlock &b : xchg_pool)
+        if (!b.busy && b.device == device && b.bytes >= bytes) { b.busy = true; *out = b.ptr; return RWKV_OK; }
+    void *p = nullptr;
+    RWKV_CHECK_HIP(hipExtMallocWithFlags(&p, bytes, hipDeviceMallocUncached));
+    xchg_pool.push_back(XchgBlock{device, bytes, p, true});
+    *out = p;
+    return RWKV_OK;
+}
+void xchg_release(void *p) {
+    std::lock_guard<std::mutex> lock(xchg_mu);
+    for (XchgBlock &b : xchg_pool)
+        if (b.ptr == p) b.busy = false;
+}
+
 // Device-side copy of the layer table plus the exchange vectors of the
 // persistent single-token kernel.  Leaves m->fused false when the shape or the
 // supplied layouts do not allow that kernel.
@@ -463,6 +494,9 @@ int setup_fused(rwkv_model *m) {
     const size_t total = decode_block_bytes(d.n_layer, d.n_embd, d.n_ffn, d.n_vocab);
     RWKV_CHECK_HIP(hipMalloc(&m->dev_block, total));
     RWKV_CHECK_HIP(hipMemset(m->dev_block, 0, total));
+    m->xchg_bytes = decode_exchange_bytes(d.n_embd, d.n_ffn);
+    RWKV_TRY(xchg_acquire(m->device, m->xchg_bytes, &m->xchg_block));
+    RWKV_CHECK_HIP(hipMemset(m->xchg_block, 0, m->xchg_bytes));
     std::vector<DLayerSrc> src((size_t)d.n_layer);
     for (size_t l = 0; l < src.size(); ++l) {
         const rwkv_layer_desc &ld = m->layers[l];
@@ -477,7 +511,7 @@ int setup_fused(rwkv_model *m) {
     s.emb = d.emb; s.ln0_w = d.ln0_w; s.ln0_b = d.ln0_b; s.lnout_w = d.ln_out_w; s.lnout_b = d.ln_out_b;
     s.head = to_dq(d.head);
     s.layers = src.data();
-    const int rc = decode_setup(m->dev_block, s, &m->dm, &m->db);
+    const int rc = decode_setup(m->dev_block, m->xchg_block, s, &m->dm, &m->db);
     if (rc) return rc;
     m->epoch = 1;      // tag 0 is what the zero-filled exchange buffers hold
     m->fused = true;
@@ -546,8 +580,6 @@ bool rows_supported(const rwkv_model *m) {
             return false;
     return true;
 }
-
-#define RWKV_TRY(expr) do { const int rc_ = (expr); if (rc_) return rc_; } while (0)
 
 // R rows through every layer.  sequence: rows are consecutive tokens of one sequence whose state is
 // `state` [L,5,C]; otherwise row b is one token of sequence b with state at state + b * state_stride.
@@ -686,7 +718,7 @@ int rwkv_model_create(const rwkv_model_desc *desc, rwkv_model **out) {
     m->d.layers = m->layers.data();
     m->device = dev;
     rc = setup_fused(m);
-    if (rc) { delete m; return rc; }
+    if (rc) { rwkv_model_destroy(m); return rc; }
     *out = m;
     return RWKV_OK;
 }
@@ -694,6 +726,7 @@ int rwkv_model_create(const rwkv_model_desc *desc, rwkv_model **out) {
 void rwkv_model_destroy(rwkv_model *m) {
     if (!m) return;
     if (m->dev_block) (void)hipFree(m->dev_block);
+    if (m->xchg_block) xchg_release(m->xchg_block);
     delete m;
 }
 
