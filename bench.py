@@ -71,9 +71,7 @@ def cpu_baseline(shape, threads: int):
 def phase_trace(model, L: int, C: int) -> int:
     """Where a token step of the persistent kernel spends its time: every workgroup stamps its phase boundaries
     (100 MHz wall clock); the table gives, per boundary, the spread over the workgroups relative to the earliest
-    workgroup's start of the layer.  "X:stats" / "X:scale" = the records of the other workgroups have arrived,
-    "X:digits" = gathered and written as digit planes, "X:mfma" = the back waves have parked the tile sums,
-    "finX" = epilogue done and results published."""
+    workgroup's start of the layer."""
     import numpy as np
     import torch
     from rwkvstic_amd import _native as N
@@ -91,14 +89,19 @@ def phase_trace(model, L: int, C: int) -> int:
     model.check()
     N.check(N.lib().rwkv_model_set_trace(model._handle, None))
     t = buf.cpu().numpy().astype("float64").reshape(G, L, per) * 0.01          # microseconds
-    names = ["start", "A:stats", "A:digits", "A:mfma", "finA", "B:scale", "B:digits", "B:mfma", "finB",
-             "C:stats", "C:digits", "C:mfma", "finC", "D:scale", "D:digits", "D:mfma"]
+    names = {0: "start", 16: "A:polled", 1: "A:stats", 2: "A:digits", 3: "A:mfma", 20: "A:sums", 4: "finA",
+             17: "B:polled", 5: "B:scale", 6: "B:digits", 7: "B:mfma", 21: "B:sums", 8: "finB",
+             18: "C:polled", 9: "C:stats", 10: "C:digits", 11: "C:mfma", 12: "finC",
+             19: "D:polled", 13: "D:scale", 14: "D:digits", 15: "D:mfma", 22: "D:sums"}
     print("phases: A = att k, v, r   B = att output   C = ffn key + receptance   D = ffn value   (microseconds)")
+    print("X:polled = the polling wave holds every workgroup's first records; X:stats / X:scale = all records reduced "
+          "(workgroup barrier); X:digits = gathered and written as digit planes; X:mfma = tile sums parked by the "
+          "weight-streaming waves; X:sums = the owner wave has combined them; finX = results published")
     for l in sorted({min(L - 1, 1), L // 2, L - 2 if L > 2 else L - 1}):
         base = t[:, l, 0].min()
         print(f"layer {l}")
         prev = 0.0
-        for i, name in enumerate(names):
+        for i, name in names.items():
             v = t[:, l, i] - base
             med = float(np.median(v))
             print(f"  {name:9s} min {v.min():6.2f}  med {med:6.2f}  max {v.max():6.2f}   (+{med - prev:5.2f} after the previous boundary)")

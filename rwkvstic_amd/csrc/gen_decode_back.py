@@ -40,6 +40,7 @@ DEFER = int(os.environ.get("RWKV_BACK_DEFER", "1"))
 # per-phase windows for the reloads that follow the barrier of the att k/v/r, att output, ffn key and ffn value phases
 WINDOWS = [int(x) for x in os.environ.get("RWKV_BACK_WINDOWS", ",".join([str(WINDOW)] * 4)).split(",")]
 BURST = int(os.environ.get("RWKV_BACK_BURST", "0"))      # the first BURST reloads after a phase's barrier go out back to back
+PACE = int(os.environ.get("RWKV_BACK_PACE", "0"))        # s_sleep units (64 cycles) in front of every deferred reload: the reloads of a phase go out at a steady rate instead of as fast as the window allows
 SLEEP = int(os.environ.get("RWKV_BACK_SLEEP", "0"))      # s_sleep units (64 cycles) between a phase's barrier and its reloads   # weight loads a wave keeps in flight while it reloads slots
 
 
@@ -226,6 +227,8 @@ def gen(KW, R, NV, NSH):
             e(f"s_sleep {SLEEP}")
         for i, p in enumerate(deferred):
             assert issued_loads == p + R
+            if PACE and i >= BURST:
+                e(f"s_sleep {PACE}")
             layer_reload(p, max(BURST, WINDOWS[ph]) if i < BURST else WINDOWS[ph])
             issued_loads += 1
     # end of layer: next layer's addresses become current; fetch the layer after

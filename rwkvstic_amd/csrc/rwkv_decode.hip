@@ -62,7 +62,10 @@ constexpr int kRealJobs = 13;          // tile jobs per layer: k v r | o | ffn_r
 constexpr unsigned kSpinLimit = 1u << 20;
 constexpr int kStatRows = 2;           // XR rows 0-1: sum x of a workgroup's 16 channels, and their squared deviations from the workgroup's own mean
 constexpr int kLnRows = kStatRows + 3 * 3;     // rows of the XR record table
-constexpr int kEarlyDiv = 4;           // gathers start when all but G / kEarlyDiv workgroups have published (measured flat from G/20 to G)
+#ifndef RWKV_EARLY_DIV
+#define RWKV_EARLY_DIV 4
+#endif
+constexpr int kEarlyDiv = RWKV_EARLY_DIV;           // gathers start when all but G / kEarlyDiv workgroups have published (measured flat from G/20 to G)
 constexpr int kHeadCsPerThread = 4;    // head column sums a front thread fetches: 16 per head tile of the workgroup
 
 // LDS flag words
