@@ -23,26 +23,40 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E vendor peak
 
 # HBM bytes per launch of the single-token kernel from rocprofv3 counters (FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB,
-# both scaled by a 1 GiB device copy in the same run): a measured constant per shape, not something this script
-# can read live.  Shapes without a counter run report null.
-PMC_TRAFFIC_BYTES = {"3B": 2_964_600_000}
+# both scaled by a 1 GiB device copy in the same run; profiles/decode_kernel_3B_b1_hbm_traffic.md): a measured
+# constant per shape, not something this script can read live.  It is tied to the kernel sources it was measured on
+# by their digest (csrc_digest() below): with any other sources the bench reports null instead of a stale figure.
+PMC_TRAFFIC = {"3B": {"bytes": 2_964_600_000, "csrc_digest": "unmeasured"}}
 
 
-def cpu_baseline(shape, threads: int):
-    """The CPU oracle (the reference's torch CPU path restated) on this box's host cores, on a
-    bounded sample: the shape's embedding + 2 layers + head, decoding 6 tokens at batch 1; the per-layer
-    time is scaled to the full layer count."""
+def csrc_digest() -> str:
+    """sha256 over the kernel sources of the library, in name order (what `traffic` was measured on)."""
+    import hashlib
+    d = os.path.join(ROOT, "rwkvstic_amd", "csrc")
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(d)):
+        if name.endswith((".hip", ".h", ".inc", ".py")):
+            h.update(name.encode())
+            h.update(open(os.path.join(d, name), "rb").read())
+    return h.hexdigest()[:16]
+
+
+def cpu_baseline(shape, threads: int, layers_timed: int):
+    """The CPU oracle (the reference's torch CPU path restated: float32 matmul on a per-call uint8 -> float32 cast,
+    float64 element-wise, Python WKV step) on this box's host cores, decoding at batch 1 on a bounded sample:
+    `layers_timed` of the shape's layers (0 = all) + embedding + head, 1 untimed and 3 timed tokens; the layer time
+    is scaled to the full depth.  The matrices are drawn directly as codes (oracle QMat.synthetic): the cost of the
+    path does not depend on their values and running the quantiser over the model would take longer than the
+    sample itself."""
     import torch
     from oracle import rwkv_oracle as O
     from rwkvstic_amd import synth
     L, C, F, V = shape
     torch.set_num_threads(threads)
-    Ls = min(2, L)
-    sd = synth.make_state_dict(Ls, C, F, V, seed=1)
-    m = O.OracleModel(sd)
-    del sd
+    Ls = L if layers_timed <= 0 else min(layers_timed, L)
+    m = O.OracleModel.synthetic(Ls, C, F, V, seed=1)
     state = m.emptyState.clone()
-    toks = synth.random_tokens(7, V=V, seed=2).tolist()
+    toks = synth.random_tokens(4, V=V, seed=2).tolist()
     m.forward([toks[0]], state)                       # warm-up
     t_layers = t_rest = 0.0
     n = 0
@@ -61,11 +75,101 @@ def cpu_baseline(shape, threads: int):
         t_rest += (t1 - t0) + (t3 - t2)
         n += 1
     per_token = (t_layers / n) * (L / Ls) + t_rest / n
+    scaled = "" if Ls == L else f", layer time scaled x{L / Ls:g}"
     return {
         "value": round(1.0 / per_token, 3), "unit": "tokens/s", "cores": threads, "kind": "port",
         "sample": f"oracle (torch CPU fp32 matmul on uint8->fp32 cast, fp64 elementwise), shape C={C} F={F} V={V}: "
-                  f"{Ls} of {L} layers + head timed over {n} decode tokens at batch 1, layer time scaled x{L // Ls}",
+                  f"{Ls} of {L} layers + head timed over {n} decode tokens at batch 1{scaled}",
     }
+
+
+def calibrate_copy(mib: int) -> None:
+    """One device-to-device copy of `mib` MiB (a kernel of known HBM traffic: the yardstick for rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE readings of the same run)."""
+    if mib <= 0:
+        return
+    import torch
+    n = mib << 20
+    src = torch.full((n,), 3, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    dst.copy_(src)                    # one copy kernel: reads n bytes, writes n bytes
+    torch.cuda.synchronize()
+    del src, dst
+
+
+def isolated_matvec(device="cuda"):
+    """BASELINE configuration 1: the quantised matrix-vector product on its own (rwkv_mm8_packed, general
+    four-vector form) at the three 3B shapes, batch 1 and 8.  Each call reads a different matrix out of a pool
+    of at least 512 MB, so no matrix is served from L2 or the 256 MB memory-side cache: GB/s = in x out bytes
+    per call / time per call over HIP events."""
+    import torch
+    from rwkvstic_amd import ops
+    out = []
+    pool = torch.randint(0, 256, (640 << 20,), dtype=torch.uint8, device=device)       # random bytes are valid packed codes
+    g = torch.Generator(device=device).manual_seed(3)
+    for n_in, n_out in ((2560, 2560), (2560, 10240), (10240, 2560)):
+        nbytes = n_in * n_out
+        n_mats = pool.numel() // nbytes
+        r_row = torch.rand(n_in, generator=g, device=device) * 9e-4 + 1e-4
+        m_row = (torch.randn(n_in, generator=g, device=device) * 0.01).double()
+        r_col = torch.rand(n_out, generator=g, device=device) * 9e-4 + 1e-4
+        m_col = torch.randn(n_out, generator=g, device=device) * 0.01
+        for B in (1, 8):
+            x = torch.randn(B, n_in, generator=g, device=device)
+            y = torch.empty(B, n_out, dtype=torch.float64, device=device)
+            calls = 2 * n_mats
+
+            def run(k):
+                for i in range(k):
+                    off = (i % n_mats) * nbytes
+                    ops.mm8_packed(x, pool[off:off + nbytes], n_in, n_out, r_row, m_row, r_col, m_col, out=y)
+            run(n_mats)
+            torch.cuda.synchronize()
+            # the calls are recorded into a HIP graph and replayed, so that the time is the kernels' and not
+            # the host's launch rate (about 10 us per call from Python, more than the smaller products take)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                run(calls)
+            graph.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) / calls * 1e3
+            out.append({"shape": f"{n_in}x{n_out}", "batch": B, "us_per_call": round(us, 2),
+                        "GB_per_s": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                        "distinct_matrices": n_mats})
+    return out
+
+
+def isolated_wkv(device="cuda"):
+    """BASELINE configuration 2: rwkv_wkv_f32 at B=8, T=1024, C=2560 (k, v read and y written once: 251.7 MB)."""
+    import torch
+    from rwkvstic_amd import ops
+    B, T, C = 8, 1024, 2560
+    g = torch.Generator(device=device).manual_seed(4)
+    k = torch.randn(B, T, C, generator=g, device=device)
+    v = torch.randn(B, T, C, generator=g, device=device)
+    w = -torch.exp(torch.rand(C, generator=g, device=device) * 9 - 8)
+    u = torch.rand(C, generator=g, device=device) * 2 - 1
+    us = []
+    for _ in range(4):
+        aa, bb = torch.zeros(B, C, device=device), torch.zeros(B, C, device=device)
+        pp = torch.full((B, C), -1e38, device=device)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        ops.wkv_f32(w, u, k, v, aa, bb, pp)
+        e1.record()
+        torch.cuda.synchronize()
+        us.append(e0.elapsed_time(e1) * 1e3)
+    best = sorted(us[1:])[len(us[1:]) // 2]
+    nbytes = 3 * B * T * C * 4
+    return {"shape": f"B={B} T={T} C={C}", "us": round(best, 1), "GB_per_s": round(nbytes / best / 1e3, 1),
+            "bytes": nbytes}
 
 
 def phase_trace(model, L: int, C: int) -> int:
@@ -128,6 +232,11 @@ def main() -> int:
     ap.add_argument("--shape", default="3B", choices=["169M", "3B", "14B"])
     ap.add_argument("--prefill", type=int, default=1024)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-baseline-layers", type=int, default=8,
+                    help="layers of the shape the CPU baseline times (0 = all of them; the rest is scaled)")
+    ap.add_argument("--no-isolated", action="store_true", help="skip the isolated matvec / WKV measurements")
+    ap.add_argument("--isolated-only", action="store_true",
+                    help="only the isolated matvec and WKV kernels (for profiling them on their own)")
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="before the workload, copy this many MiB device to device once (a kernel of known HBM "
                          "traffic: the yardstick for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
@@ -146,6 +255,11 @@ def main() -> int:
     from rwkvstic_amd.model import HipRWKV
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.isolated_only:
+        torch.cuda.set_device(0)
+        calibrate_copy(args.calibrate_copy_mib)
+        print(json.dumps({"isolated_matvec": isolated_matvec(), "isolated_wkv": isolated_wkv()}), flush=True)
+        return 0
     shape = synth.SHAPES[args.shape]
     L, C, F, V = shape
     torch.cuda.set_device(0)
@@ -161,14 +275,7 @@ def main() -> int:
     if args.phase_trace:
         return phase_trace(model, L, C)
 
-    if args.calibrate_copy_mib > 0:
-        n = args.calibrate_copy_mib << 20
-        src = torch.full((n,), 3, dtype=torch.uint8, device="cuda")
-        dst = torch.empty_like(src)
-        torch.cuda.synchronize()
-        dst.copy_(src)                    # one elementwise copy kernel: reads n bytes, writes n bytes
-        torch.cuda.synchronize()
-        del src, dst
+    calibrate_copy(args.calibrate_copy_mib)
 
     # ---- prefill -------------------------------------------------------------
     prompt = synth.random_tokens(args.prefill, V=V, seed=0).cuda()
@@ -199,6 +306,7 @@ def main() -> int:
     ms_per_step = wall_ms / args.steps
     tok_s = args.steps / (wall_ms / 1e3)
     assert bool(torch.isfinite(logits).all()), "non-finite logits"
+    model.check()            # raises if a token step gave up waiting (its results would be stale): no number then
 
     # ---- the dominant kernel on its own: single-token forward calls, HIP events on the launch stream
     nk = min(64, args.steps)
@@ -213,7 +321,11 @@ def main() -> int:
     e1.record(stream)
     torch.cuda.synchronize()
     step_us = e0.elapsed_time(e1) / nk * 1e3
+    model.check()
     achieved = wbytes / (step_us * 1e-6) / 1e9
+    traffic = PMC_TRAFFIC.get(args.shape)
+    digest = csrc_digest()
+    traffic_now = traffic["bytes"] if (traffic and model.fused_step and traffic["csrc_digest"] == digest) else None
     out = {
         "metric": "decode tokens/s @ RWKV-4 3B-shape fp32i8 B=1" if args.shape == "3B"
                   else f"decode tokens/s @ RWKV-4 {args.shape}-shape fp32i8 B=1",
@@ -230,12 +342,16 @@ def main() -> int:
                                else "decode token step (all phase kernels of one token)",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": PMC_TRAFFIC_BYTES.get(args.shape) if model.fused_step else None,
+                     "traffic": traffic_now, "traffic_measured_on_csrc": traffic["csrc_digest"] if traffic else None,
+                     "csrc_digest": digest,
                      "launch_us": round(step_us, 2), "decode_loop_us_per_token": round(dev_ms / args.steps * 1e3, 2)},
     }
+    if not args.no_isolated:
+        out["isolated_matvec"] = isolated_matvec()
+        out["isolated_wkv"] = isolated_wkv()
     if not args.no_cpu_baseline:
         threads = min(16, os.cpu_count() or 1)
-        out["cpu_baseline"] = cpu_baseline(shape, threads)
+        out["cpu_baseline"] = cpu_baseline(shape, threads, args.cpu_baseline_layers)
     print(json.dumps(out), flush=True)
     return 0
 

@@ -187,6 +187,24 @@ class QMat:
     def __call__(self, x: Tensor) -> Tensor:
         return mm8_naive(x, self.codes, self.range, self.offset, self.dtype)
 
+    @classmethod
+    def synthetic(cls, n_in: int, n_out: int, gen: torch.Generator, dtype: torch.dtype = torch.float32) -> "QMat":
+        """A matrix given directly by random codes, ranges and offsets (what quantising an ~N(0, 0.02) matrix
+        yields in size and spread), for timing the arithmetic at sizes where running the quantiser over a whole
+        model would dominate the run; the cost of ``__call__`` does not depend on the values."""
+        self = cls.__new__(cls)
+        seed = int(torch.randint(1, 2 ** 31 - 1, (1,), generator=gen))
+        # bytes of a multiplicative hash of the index: filled at memory speed (the random generators take
+        # minutes for the 3 GB of a whole model), and as good as random for what the timing needs
+        n8 = (n_in * n_out + 7) // 8
+        h = (torch.arange(n8, dtype=torch.int64) + seed) * -7046029254386353131
+        h ^= h >> 29
+        self.codes = h.view(torch.uint8)[:n_in * n_out].reshape(n_in, n_out)
+        self.range = torch.rand(n_in, generator=gen, dtype=torch.float32) * 2e-4 + 5e-4
+        self.offset = (torch.rand(n_in, generator=gen, dtype=torch.float64) - 0.5) * 0.02 - 0.08
+        self.n_in, self.n_out, self.dtype = n_in, n_out, dtype
+        return self
+
 
 class OracleModel:
     """CPU restatement of ``myRWKV`` (agnostic/backends/opt.py:27-84)."""
@@ -227,6 +245,32 @@ class OracleModel:
         # opt.py:31-32, 80
         self.emptyState = torch.tensor(
             self.layers * [[[0.0] * self.dims] * 4 + [[-1e30] * self.dims]], dtype=f64)
+
+    @classmethod
+    def synthetic(cls, layers: int, C: int, F: int, V: int, seed: int = 0) -> "OracleModel":
+        """The network at full depth with every matrix drawn as codes (``QMat.synthetic``) and unit LayerNorms:
+        the same arithmetic, op for op, as a quantised checkpoint, built in seconds.  For timing only."""
+        g = torch.Generator().manual_seed(seed)
+        f64 = torch.float64
+        self = cls.__new__(cls)
+        self.matmul_dtype = torch.float32
+        self.dims, self.layers = C, layers
+        self.emb = torch.randn(V, C, generator=g, dtype=torch.float32) * 0.02
+        ones, zeros = torch.ones(C, dtype=f64), torch.zeros(C, dtype=f64)
+        self.ln_in, self.ln_out = (ones, zeros), (ones, zeros)
+        self.head = QMat.synthetic(C, V, g)
+        self.blocks = []
+        for _ in range(layers):
+            self.blocks.append(dict(
+                ln1=(ones, zeros), ln2=(ones, zeros),
+                att_k=QMat.synthetic(C, C, g), att_v=QMat.synthetic(C, C, g), att_r=QMat.synthetic(C, C, g),
+                att_o=QMat.synthetic(C, C, g), ffn_k=QMat.synthetic(C, F, g), ffn_r=QMat.synthetic(C, C, g),
+                ffn_v=QMat.synthetic(F, C, g),
+                attmix=torch.rand(3, 1, C, generator=g, dtype=f64), ffnmix=torch.rand(2, 1, C, generator=g, dtype=f64),
+                time_first=torch.rand(C, generator=g, dtype=f64) * 2 - 1,
+                time_decay=(torch.rand(C, generator=g, dtype=f64) * 6 - 5).exp().neg()))
+        self.emptyState = torch.tensor(layers * [[[0.0] * C] * 4 + [[-1e30] * C]], dtype=f64)
+        return self
 
     # block.py:56-102
     def block_forward(self, blk: dict, x: Tensor, state: Tensor) -> Tensor:

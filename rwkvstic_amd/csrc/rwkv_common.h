@@ -117,16 +117,19 @@ __device__ __forceinline__ F wkv_step(F w, F u, F k, F v, F &aa, F &bb, F &pp) {
 // carried in float64 while aa, bb, the exponentials and the output stay float32.
 __device__ __forceinline__ float wkv_step_f32(double w, double u, float k, float v,
                                               float &aa, float &bb, double &pp) {
-    const double q = u + w + (double)k;
-    const double p = fmax(pp, q);
-    const float e1 = expf((float)(pp - p)), e2 = expf((float)(q - p));
+    // as in wkv_step: of each pair of exponentials one is e^0, so one call per pair gives the same bits as two
+    // (the float32 rounding of a difference and of its negative are each other's negatives)
+    const double d = pp - (u + w + (double)k);
+    const float e = expf(-fabsf((float)d));
+    const float e1 = d >= 0.0 ? 1.f : e, e2 = d >= 0.0 ? e : 1.f;
     const float y = (e1 * aa + e2 * v) / (e1 * bb + e2);
     const double s = pp + w, r = (double)k + w;
-    const double p2 = fmax(s, r);
-    const float f1 = expf((float)(s - p2)), f2 = expf((float)(r - p2));
+    const double d2 = s - r;
+    const float f = expf(-fabsf((float)d2));
+    const float f1 = d2 >= 0.0 ? 1.f : f, f2 = d2 >= 0.0 ? f : 1.f;
     aa = f1 * aa + f2 * v;
     bb = f1 * bb + f2;
-    pp = p2;
+    pp = fmax(s, r);
     return y;
 }
 

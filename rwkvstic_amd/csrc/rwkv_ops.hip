@@ -72,9 +72,13 @@ mm8_packed_kernel(int n_in, int n_out, int n_kb, int kc_blocks,
 }
 
 // ---------------------------------------------------------------------------
-// WKV: one thread per (b, c); k/v loads are independent of the recurrence, so
-// the compiler can hoist them ahead of the dependent exp chain (unroll 4).
+// WKV: one thread per (b, c), state in registers.  The recurrence is a serial chain of T steps per thread, and
+// with B * C threads there is about one wavefront per compute unit, so nothing else hides a load: k and v are
+// therefore fetched a whole group of steps ahead of the step that uses them (kWkvAhead independent loads in
+// flight per thread), and the chain itself, not the memory latency, sets the pace.
 // ---------------------------------------------------------------------------
+constexpr int kWkvAhead = 16;
+
 __global__ void __launch_bounds__(64)
 wkv_f32_kernel(int B, int T, int C, const float *__restrict__ w, const float *__restrict__ u,
                const float *__restrict__ k, const float *__restrict__ v, float *__restrict__ y,
@@ -86,10 +90,24 @@ wkv_f32_kernel(int B, int T, int C, const float *__restrict__ w, const float *__
     const double wc = (double)w[c], uc = (double)u[c];
     float a = aa[idx], bsum = bb[idx];
     double p = (double)pp[idx];
-#pragma unroll 4
-    for (int t = 0; t < T; ++t) {
-        const size_t o = base + (size_t)t * C;
-        y[o] = wkv_step_f32(wc, uc, k[o], v[o], a, bsum, p);
+    float kc[kWkvAhead], vc[kWkvAhead], kn[kWkvAhead], vn[kWkvAhead];
+#pragma unroll
+    for (int i = 0; i < kWkvAhead; ++i) {
+        const size_t o = base + (size_t)min(i, T - 1) * C;
+        kc[i] = k[o]; vc[i] = v[o];
+    }
+    for (int t0 = 0; t0 < T; t0 += kWkvAhead) {
+#pragma unroll
+        for (int i = 0; i < kWkvAhead; ++i) {           // the next group (clamped at the end: re-reads the last row)
+            const size_t o = base + (size_t)min(t0 + kWkvAhead + i, T - 1) * C;
+            kn[i] = k[o]; vn[i] = v[o];
+        }
+#pragma unroll
+        for (int i = 0; i < kWkvAhead; ++i) {
+            if (t0 + i < T) y[base + (size_t)(t0 + i) * C] = wkv_step_f32(wc, uc, kc[i], vc[i], a, bsum, p);
+        }
+#pragma unroll
+        for (int i = 0; i < kWkvAhead; ++i) { kc[i] = kn[i]; vc[i] = vn[i]; }
     }
     aa[idx] = a; bb[idx] = bsum; pp[idx] = (float)p;
 }

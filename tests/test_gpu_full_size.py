@@ -172,3 +172,52 @@ def test_14b_width_two_layers_prompt_chunks_batch_and_oracle():
         assert float((sb[b, :, :2] - s1[:, :2]).abs().max()) < 1e-4, b
     lo, _ = exact.forward([toks[0]], se)
     assert float((lb[0].cpu() - lo).abs().max()) < 1e-4 and int(lb[0].argmax()) == int(lo.argmax())
+
+
+def test_14b_width_batch_of_32_after_64_token_prompts():
+    """The 14B configuration's batch decode at its real width (C=5120, F=20480, V=50277; 2 of the 40 layers): 32
+    independent sequences, each with its own seeded random prompt of 64 tokens (prefilled through the many-row
+    path; the 9..32-row product variant then serves the batch step at K = 5120 and 20480 inside the model), one
+    decode step of all 32 at once.  Every sequence of the batch must equal the same token fed on its own; four of
+    them are also checked, prompt and step, against the CPU oracle with exact accumulation (logits 1e-4, state
+    1e-4).  A 256-token prompt fed as one 256-token chunk is checked against the same oracle."""
+    from rwkvstic_amd.model import HipRWKV, wkv_state_to_reference
+    _, C, F, V = synth.SHAPES["14B"]
+    sd = synth.make_state_dict(2, C, F, V, seed=6, ln="random")
+    exact = O.OracleModel(sd, matmul_dtype=torch.float64)
+    hip = HipRWKV(sd)
+    B = 32
+    prompts = [synth.random_tokens(64, V=V, seed=100 + b).tolist() for b in range(B)]
+    states, last = [], []
+    for b in range(B):
+        lg, s = hip.forward(prompts[b], hip.emptyState.clone())
+        states.append(s)
+        last.append(int(lg.argmax()))
+    _say("batch step of 32")
+    lb, sb = hip.forward_batch(last, torch.stack(states).contiguous())
+    for b in range(B):
+        l1, s1 = hip.forward([last[b]], states[b].clone())
+        assert float((lb[b] - l1).abs().max()) < 1e-5 and int(lb[b].argmax()) == int(l1.argmax()), b
+        assert float((sb[b, :, :2] - s1[:, :2]).abs().max()) < 1e-6, b
+
+    def state_close(s_gpu, s_ref, tol=1e-4):
+        s = wkv_state_to_reference(s_gpu).cpu()
+        assert (s[:, :2] - s_ref[:, :2]).abs().max() < 10 * tol
+        assert ((s[:, 3] - s_ref[:, 3]).abs() <= tol * s_ref[:, 3].abs() + 1e-30).all()
+        assert ((s[:, 2] - s_ref[:, 2]).abs() <= tol * torch.maximum(s_ref[:, 2].abs(), s_ref[:, 3]) + 1e-30).all()
+
+    for b in (0, 7, 19, 31):
+        _say(f"oracle for sequence {b}")
+        le, se = exact.forward(prompts[b], exact.emptyState.clone())
+        assert int(le.argmax()) == last[b]
+        le, se = exact.forward([last[b]], se)
+        e64 = float((lb[b].cpu() - le).abs().max())
+        _say(f"  sequence {b}: |batch step - fp64 oracle| {e64:.2e}")
+        assert e64 < 1e-4 and int(lb[b].argmax()) == int(le.argmax())
+        state_close(sb[b], se)
+    _say("256-token chunk")
+    long_prompt = synth.random_tokens(256, V=V, seed=200).tolist()
+    lg, sg = hip.forward(long_prompt, hip.emptyState.clone())
+    le, se = exact.forward(long_prompt, exact.emptyState.clone())
+    assert float((lg.cpu() - le).abs().max()) < 1e-4 and int(lg.argmax()) == int(le.argmax())
+    state_close(sg, se)

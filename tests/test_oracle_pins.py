@@ -93,6 +93,35 @@ def test_mm8_naive_vs_fp64_dense(T):
     assert (got - x @ W.t().double()).abs().max() < 0.05
 
 
+def test_mm8_general_form_against_scalar_loops():
+    """The four-vector dequantisation dq[j,k] = code[j,k] r_row[j] r_col[k] + m_row[j] + m_col[k] written out
+    element by element on a 3 x 4 matrix, with and without the per-column vectors: pins the r_col / m_col branch
+    of the float64 dense product the GPU kernel of the isolated-matvec workload is checked against."""
+    g = torch.Generator().manual_seed(5)
+    n_in, n_out, B = 3, 4, 2
+    codes = torch.randint(0, 256, (n_in, n_out), generator=g, dtype=torch.uint8)
+    r_row = torch.rand(n_in, generator=g) * 1e-3 + 1e-4
+    m_row = (torch.randn(n_in, generator=g) * 0.01).double()
+    r_col = torch.rand(n_out, generator=g) * 1e-3 + 1e-4
+    m_col = torch.randn(n_out, generator=g) * 0.01
+    x = torch.randn(B, n_in, generator=g, dtype=torch.float64)
+    for rc, mc in ((r_col, m_col), (None, None), (r_col, None), (None, m_col)):
+        want = torch.zeros(B, n_out, dtype=torch.float64)
+        for b in range(B):
+            for k in range(n_out):
+                acc = 0.0
+                for j in range(n_in):
+                    dq = float(codes[j, k]) * float(r_row[j]) * (float(rc[k]) if rc is not None else 1.0) \
+                        + float(m_row[j]) + (float(mc[k]) if mc is not None else 0.0)
+                    acc += float(x[b, j]) * dq
+                want[b, k] = acc
+        got = O.mm8_general_f64(x, codes, r_row, m_row, rc, mc)
+        assert torch.allclose(got, want, rtol=1e-13, atol=1e-15)
+    # a transposed or swapped operand must not pass: the column vectors really act on columns
+    bad = O.mm8_general_f64(x, codes, r_row, m_row, r_col.flip(0), m_col)
+    assert not torch.allclose(bad, O.mm8_general_f64(x, codes, r_row, m_row, r_col, m_col), rtol=1e-6)
+
+
 # ---------------------------------------------------------------- layernorm
 def test_layernorm_matches_torch():
     x = torch.randn(7, 96, dtype=torch.float64) * 3 + 1
