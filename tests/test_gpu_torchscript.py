@@ -63,8 +63,14 @@ class MM8x3Like(torch.nn.Module):
 
 class WKVLike(torch.nn.Module):
     def forward(self, T: int, C: int, w, u, k, v, aa, bb, pp):
+        # the matrix modules hand over float32 rows (a float32 tensor plus a 0-dim float64 stays float32); the
+        # operator is float64, so the caller converts, as wkv.py:9-13 does
+        w = w.contiguous().to(torch.float64)
+        u = u.contiguous().to(torch.float64)
+        k = k.contiguous().to(torch.float64)
+        v = v.contiguous().to(torch.float64)
         y = torch.empty((T, C), device=w.device, dtype=torch.float64)
-        torch.ops.rwkv.wkv_forward(1, T, C, w.contiguous(), u.contiguous(), k.contiguous(), v.contiguous(), y, aa, bb, pp)
+        torch.ops.rwkv.wkv_forward(1, T, C, w, u, k, v, y, aa, bb, pp)
         return y, aa, bb, pp
 
 
@@ -101,8 +107,9 @@ def test_scripted_modules_call_the_operators_and_survive_an_archive(tmp_path):
     path = str(tmp_path / "timemix.rwkv")
     torch.jit.save(scripted, path)
     loaded = torch.jit.load(path, map_location="cuda")      # written two lines above by this test
-    for name in ("att.weight", "att.range1", "att.offset2", "attout.weight"):
-        assert name in loaded.state_dict()
+    # the tensors are plain module attributes, as in the reference's modules (matmul.py:12,67-68)
+    assert loaded.att.weight.dtype == torch.uint8 and loaded.att.range1.dtype == torch.float32
+    assert loaded.att.offset2.dtype == torch.float64 and torch.equal(loaded.attout.weight.cpu(), qs[3][0])
     x = torch.randn(1, C, generator=g, dtype=torch.float64)
     aa = torch.zeros(C, dtype=torch.float64); bb = torch.zeros(C, dtype=torch.float64)
     pp = torch.full((C,), -1e30, dtype=torch.float64)
@@ -118,7 +125,10 @@ def test_scripted_modules_call_the_operators_and_survive_an_archive(tmp_path):
             st = tuple(t.clone() for t in got_state)
             out, a3, b3, p3 = m(x.cuda(), *st)
             assert (out.cpu() - want).abs().max() < 1e-4
-            assert torch.allclose(a3.cpu(), a2, rtol=1e-4, atol=1e-12) and torch.allclose(b3.cpu(), b2, rtol=1e-4, atol=1e-12)
+            # (k and v reach the operator rounded to float32, as in the reference; aa is a signed sum, so it is
+            # measured against the size of the sums, not element by element)
+            assert ((b3.cpu() - b2).abs() <= 1e-4 * b2.abs() + 1e-30).all()
+            assert ((a3.cpu() - a2).abs() <= 1e-4 * torch.maximum(a2.abs(), b2) + 1e-30).all()
         got_state = (a3, b3, p3)
         x = x + want * 0.5
 
