@@ -346,6 +346,21 @@ def main() -> int:
                      "csrc_digest": digest,
                      "launch_us": round(step_us, 2), "decode_loop_us_per_token": round(dev_ms / args.steps * 1e3, 2)},
     }
+    # the kept API: RWKV(...).forward(number=n) with the built-in samplers (device-side loop) next to the raw loop
+    from rwkvstic_amd.master import RWKVMaster, greedy, typical
+    api = {}
+    n_api = min(256, max(args.steps, 8))
+    for name, smp in (("typical", typical), ("greedy", greedy)):
+        shell = RWKVMaster(model, model.emptyState, smp)
+        shell.myState = state.clone()
+        shell.lastToken = [int(toks[-1])]
+        shell.forward(number=4, stopTokens=[])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        shell.forward(number=n_api, stopTokens=[])
+        torch.cuda.synchronize()
+        api[name] = round(n_api / (time.perf_counter() - t0), 1)
+    out["api_forward_tokens_per_s"] = dict(api, tokens=n_api, note="RWKVMaster.forward(number=n): sampler, end_adj and stop test on the device")
     if not args.no_isolated:
         out["isolated_matvec"] = isolated_matvec()
         out["isolated_wkv"] = isolated_wkv()

@@ -294,6 +294,34 @@ int rwkv_model_decode_greedy(rwkv_model *m, rwkv_stream_t stream,
                              double *state, double *logits,
                              void *workspace, size_t workspace_bytes);
 
+/* The choice of the next token on the device (agnostic/samplers/typical.py:1-17 and the
+ * logit adjustment of rwkvMaster.py:37): logits[0] += end_adj (in place), then either
+ * the first maximum (greedy != 0) or locally typical sampling: softmax in float32,
+ * tokens ordered by |surprise - entropy|, the shortest prefix of that order whose mass
+ * reaches tau kept, kept p^(1/temp) sampled with the uniform number hash(seed, counter).
+ * V <= 53248.  out_token: device int64 [1]. */
+int rwkv_sample_token(rwkv_stream_t stream, double *logits, int64_t V, int greedy,
+                      float temp, float tau, double end_adj,
+                      uint64_t seed, uint64_t counter, int64_t *out_token);
+
+/* RWKVMaster.forward(number=n) (rwkvMaster.py:28-56) entirely on the device:
+ *   for i < n: logits, state = forward(tokens[i], state);
+ *              tokens[i+1] = rwkv_sample_token(logits, ..., counter = i);
+ *              stop if tokens[i+1] is one of stop_tokens[n_stop].
+ * stop_flag (device int32, zero on entry) is set when a stop token was chosen; the
+ * launches queued after that return without touching state or logits, so both are
+ * those of the stopping step.  n_done (device int64, zero on entry) counts the tokens
+ * chosen: tokens[1 .. n_done] are valid.  Only for handles with
+ * rwkv_model_has_fused_step; other shapes return RWKV_ERR_SIZE (sample from the logits
+ * of rwkv_model_forward instead). */
+int rwkv_model_decode_sample(rwkv_model *m, rwkv_stream_t stream,
+                             int64_t *tokens, int64_t n,
+                             double *state, double *logits,
+                             void *workspace, size_t workspace_bytes,
+                             int greedy, float temp, float tau, double end_adj,
+                             uint64_t seed, const int64_t *stop_tokens, int n_stop,
+                             int32_t *stop_flag, int64_t *n_done);
+
 /* out_token[0] = index of the first maximum of logits[V]. */
 int rwkv_argmax_f64(rwkv_stream_t stream, const double *logits, int64_t V,
                     int64_t *out_token);

@@ -331,6 +331,25 @@ class OracleModel:
         return toks, all_logits, state
 
 
+def typical_distribution(logits: Tensor, temp: float = 1.0, tau: float = 0.95) -> Tensor:
+    """The probability vector the reference's ``typical`` sampler hands to ``torch.multinomial``
+    (agnostic/samplers/typical.py:5-16; everything but the draw itself), normalised."""
+    probs = torch.nn.functional.softmax(logits.float(), dim=-1)          # typical.py:5
+    surprise = -torch.log(probs)                                         # :6
+    ent = torch.nansum(surprise * probs, dim=-1, keepdim=True)           # :7
+    shifted = torch.abs(surprise - ent)                                  # :8
+    sorted_ids = torch.argsort(shifted)                                  # :9
+    sorted_shifted = shifted[sorted_ids]                                 # :10
+    cumulative = torch.cumsum(probs[sorted_ids], dim=-1)                 # :11-12
+    cutoff = int((cumulative < tau).sum())                               # :13
+    cutoff = min(cutoff, probs.numel() - 1)
+    probs = probs.clone()
+    probs[shifted > sorted_shifted[cutoff]] = 0                          # :14
+    if temp != 1.0:
+        probs = probs ** (1.0 / temp)                                    # :15-16
+    return (probs / probs.sum()).double()
+
+
 def state_naive_from_stable(aa: Tensor, bb: Tensor, pp: Tensor):
     """Map a max-shifted triple to the reference's naive pair (float64)."""
     e = torch.exp(pp.double())

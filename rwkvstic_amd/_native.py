@@ -22,6 +22,7 @@ EXPORTS = (
     "rwkv_model_create", "rwkv_model_destroy", "rwkv_model_workspace_bytes",
     "rwkv_model_has_fused_step", "rwkv_model_check", "rwkv_model_set_trace",
     "rwkv_model_forward", "rwkv_model_decode_greedy", "rwkv_argmax_f64",
+    "rwkv_sample_token", "rwkv_model_decode_sample",
     "rwkv_gemm8_workspace_bytes", "rwkv_gemm8", "rwkv_gemm8_plan",
     "rwkv_model_batch_workspace_bytes", "rwkv_model_forward_batch",
 )
@@ -101,6 +102,9 @@ def lib() -> C.CDLL:
     L.rwkv_model_forward.argtypes = [vp, vp, vp, i64, vp, vp, vp, sz]
     L.rwkv_model_decode_greedy.argtypes = [vp, vp, vp, i64, vp, vp, vp, sz]
     L.rwkv_argmax_f64.argtypes = [vp, vp, i64, vp]
+    f32, f64, u64 = C.c_float, C.c_double, C.c_uint64
+    L.rwkv_sample_token.argtypes = [vp, vp, i64, ci, f32, f32, f64, u64, u64, vp]
+    L.rwkv_model_decode_sample.argtypes = [vp, vp, vp, i64, vp, vp, vp, sz, ci, f32, f32, f64, u64, vp, ci, vp, vp]
     L.rwkv_gemm8_workspace_bytes.restype = sz
     L.rwkv_gemm8_workspace_bytes.argtypes = [i64, i64, i64]
     L.rwkv_gemm8.argtypes = [vp, i64, i64, i64, vp, vp, vp, vp, vp, vp, sz]

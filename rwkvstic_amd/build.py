@@ -13,7 +13,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "librwkv_hip.so")
-SOURCES = ["rwkv_quant.hip", "rwkv_ops.hip", "rwkv_model.hip", "rwkv_decode.hip", "rwkv_rows.hip"]
+SOURCES = ["rwkv_quant.hip", "rwkv_ops.hip", "rwkv_model.hip", "rwkv_decode.hip", "rwkv_rows.hip", "rwkv_sample.hip"]
 
 FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "-shared",

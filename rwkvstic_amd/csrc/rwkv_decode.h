@@ -2,6 +2,7 @@
 #pragma once
 
 #include "rwkv_common.h"
+#include "rwkv_sample.h"
 
 namespace rwkv {
 
@@ -119,5 +120,11 @@ int decode_launch(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsig
 // n greedy steps: tokens[i + 1] = argmax(forward(tokens[i])); uses n * decode_epochs_per_token() epochs.
 int decode_launch_greedy(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsigned epoch0,
                          int64_t *tokens, int64_t n, double *state, double *logits);
+
+// n sampled steps: tokens[i + 1] = choice(forward(tokens[i])) by the sampler described in `sa` (its logits, V and
+// out_token are filled in here; sa.counter counts up per token).  A chosen stop token sets *sa.stop_flag, after
+// which the remaining launches return at once and leave state and logits as they are.
+int decode_launch_sampled(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsigned epoch0, int64_t *tokens, int64_t n,
+                          double *state, double *logits, SampleArgs sa);
 
 }  // namespace rwkv

@@ -96,6 +96,8 @@ struct DArgs {
     const int64_t *token;
     double *state;
     double *logits;
+    const int *stop;        // device word or null: when it reads non-zero the launch does nothing (a sampled stop token
+                            // ended the sequence; the remaining launches of a generation loop then leave the state alone)
 };
 
 // ---- the back (weight-streaming) waves ------------------------------------------
@@ -880,6 +882,7 @@ __global__ void __launch_bounds__((FW + kBW) * 64) decode_kernel(const DArgs a) 
     double *stat = reinterpret_cast<double *>(smem + Lds::DIG_BYTES + Lds::RED_BYTES);
     double *rf_lds = stat + 32;
     lds_flag_t *flags = (lds_flag_t *)(rf_lds + 32);
+    if (a.stop && gld(a.stop) != 0) return;          // written before this launch started: every workgroup reads the same value
     if (threadIdx.x < FLAG_COUNT) flags[threadIdx.x] = 0;
     __syncthreads();
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -1000,6 +1003,7 @@ __device__ __forceinline__ void prep_token(const DArgs &a, int64_t tok, unsigned
 // grid: L * (C / 512) layer parts, then one block for the token.
 __global__ void __launch_bounds__(kPrepThreads) prep_kernel(const DArgs a) {
     __shared__ double scr[8 * (kPrepThreads / 64)];
+    if (a.stop && gld(a.stop) != 0) return;
     const int parts = a.m.C / kPrepThreads;
     const int b = blockIdx.x;
     if (b < a.m.L * parts) prep_layer_part(a, b / parts, b % parts, scr);
@@ -1387,13 +1391,35 @@ int decode_launch(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsig
                   const int64_t *token, double *state, double *logits) {
     DArgs args;
     args.m = m; args.b = b; args.epoch0 = epoch0; args.token = token; args.state = state; args.logits = logits;
+    args.stop = nullptr;
     return launch_step(st, args, true);
+}
+
+int decode_launch_sampled(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsigned epoch0, int64_t *tokens, int64_t n,
+                          double *state, double *logits, SampleArgs sa) {
+    DArgs args;
+    args.m = m; args.b = b; args.state = state; args.logits = logits;
+    args.stop = sa.stop_flag;
+    sa.logits = logits; sa.V = m.V;
+    const unsigned ept = decode_epochs_per_token(m.L);
+    for (int64_t i = 0; i < n; ++i) {
+        args.epoch0 = epoch0 + (unsigned)i * ept;
+        args.token = tokens + i;
+        const int rc = launch_step(st, args, true);      // preparation (reads tokens[i]) + the token kernel
+        if (rc) return rc;
+        sa.out_token = tokens + i + 1;
+        const int rs = sample_launch(st, sa);
+        if (rs) return rs;
+        sa.counter += 1;
+    }
+    return RWKV_OK;
 }
 
 int decode_launch_greedy(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsigned epoch0,
                          int64_t *tokens, int64_t n, double *state, double *logits) {
     DArgs args;
     args.m = m; args.b = b; args.state = state; args.logits = logits;
+    args.stop = nullptr;
     const unsigned ept = decode_epochs_per_token(m.L);
     for (int64_t i = 0; i < n; ++i) {
         args.epoch0 = epoch0 + (unsigned)i * ept;

@@ -848,6 +848,38 @@ size_t rwkv_gemm8_workspace_bytes(int64_t T, int64_t n_in, int64_t n_out) {
     return round_up((size_t)T * 8, 256) * 3 + round_up(rows_dig_bytes(T, n_in), 256) + round_up(tot > qs ? tot : qs, 256);
 }
 
+int rwkv_sample_token(rwkv_stream_t stream, double *logits, int64_t V, int greedy, float temp, float tau, double end_adj,
+                      uint64_t seed, uint64_t counter, int64_t *out_token) {
+    RWKV_CHECK_ARG(logits && out_token, "rwkv_sample_token: null pointer");
+    RWKV_CHECK_ARG(V > 0 && V < (1ll << 31), "rwkv_sample_token: bad size");
+    RWKV_CHECK_ARG(greedy || (temp > 0.f && tau >= 0.f), "rwkv_sample_token: temp must be positive, tau non-negative");
+    SampleArgs sa{};
+    sa.logits = logits; sa.V = (int)V; sa.greedy = greedy ? 1 : 0; sa.temp = temp; sa.tau = tau; sa.end_adj = end_adj;
+    sa.seed = seed; sa.counter = counter; sa.out_token = out_token;
+    return sample_launch((hipStream_t)stream, sa);
+}
+
+int rwkv_model_decode_sample(rwkv_model *m, rwkv_stream_t stream, int64_t *tokens, int64_t n, double *state, double *logits,
+                             void *workspace, size_t workspace_bytes, int greedy, float temp, float tau, double end_adj,
+                             uint64_t seed, const int64_t *stop_tokens, int n_stop, int32_t *stop_flag, int64_t *n_done) {
+    int rc = check_forward_args(m, tokens, state, logits, workspace, workspace_bytes, 1, "rwkv_model_decode_sample");
+    if (rc) return rc;
+    RWKV_CHECK_ARG(n > 0, "rwkv_model_decode_sample: n must be positive");
+    RWKV_CHECK_ARG(stop_flag && n_done, "rwkv_model_decode_sample: stop_flag and n_done must point to device words");
+    RWKV_CHECK_ARG(n_stop >= 0 && (n_stop == 0 || stop_tokens), "rwkv_model_decode_sample: stop list");
+    RWKV_CHECK_ARG(greedy || (temp > 0.f && tau >= 0.f), "rwkv_model_decode_sample: temp must be positive, tau non-negative");
+    if (!m->fused)
+        return set_error(RWKV_ERR_SIZE, "rwkv_model_decode_sample: this shape does not run the persistent single-token "
+                                        "kernel; sample on the host from rwkv_model_forward's logits");
+    if ((rc = fused_epochs(m, (hipStream_t)stream, n))) return rc;
+    SampleArgs sa{};
+    sa.greedy = greedy ? 1 : 0; sa.temp = temp; sa.tau = tau; sa.end_adj = end_adj; sa.seed = seed; sa.counter = 0;
+    sa.stop_tokens = stop_tokens; sa.n_stop = n_stop; sa.stop_flag = stop_flag; sa.n_done = n_done;
+    rc = decode_launch_sampled((hipStream_t)stream, m->dm, m->db, m->epoch, tokens, n, state, logits, sa);
+    m->epoch += (unsigned)n * decode_epochs_per_token(m->d.n_layer);
+    return rc;
+}
+
 int rwkv_gemm8_plan(int64_t T, int64_t n_in, int64_t n_out, int n_products, int plan[4], size_t *tot_bytes_per_product) {
     RWKV_CHECK_ARG(plan && tot_bytes_per_product, "rwkv_gemm8_plan: null pointer");
     RWKV_CHECK_ARG(T > 0 && n_in > 0 && n_out > 0 && n_products >= 1 && n_products <= kRowsMaxProducts,

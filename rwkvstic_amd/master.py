@@ -6,7 +6,9 @@ Kept from the reference, because callers rely on it: ``forward`` adds ``end_adj`
 sampling and stops on ``stopTokens`` / ``stopStrings``; ``lastToken`` starts at ``[187]``; ``loadContext``
 sets ``lastToken`` to the last token of ``ctx`` (not of ``newctx``) and leaves the caller's state untouched;
 ``getState``/``setState`` exchange ``(state, lastToken)`` pairs.  Changed: prompts are fed in chunks of 1024
-tokens (the reference's default is 20) because they run as GEMMs here, and sampling stays on the GPU.
+tokens (the reference's default is 20) because they run as GEMMs here, and with the built-in samplers, no
+per-token callback and no stop strings that could match, ``forward(number=n)`` runs as one device-side loop
+(token kernel, sampler, stop-token test, next embedding) instead of n host round trips.
 """
 from __future__ import annotations
 
@@ -74,6 +76,10 @@ def load_tokenizer(spec):
     return spec
 
 
+def _no_progress(x):
+    return x
+
+
 class RWKVMaster:
     logging = False
 
@@ -86,10 +92,35 @@ class RWKVMaster:
         self.sampler = sampler
 
     # ------------------------------------------------------------------ generation (rwkvMaster.py:28-56)
+    def _device_loop(self, number, stopStrings, progressLambda, kwargs) -> bool:
+        """Whether the whole generation loop can run on the device (``HipRWKV.decode_sample``): the built-in
+        samplers, no per-token callback, and stop strings that cannot occur (no stop strings, or a tokenizer
+        that only ever yields token ids)."""
+        m = self.model
+        if not (callable(getattr(m, "decode_sample", None)) and getattr(m, "fused_step", False)):
+            return False
+        if self.sampler not in (typical, greedy) or progressLambda is not _no_progress or number < 1:
+            return False
+        if len(self.lastToken) != 1 or set(kwargs) - {"temp", "top_p_usual"}:
+            return False
+        return not stopStrings or isinstance(self.tokenizer, TokenIds)
+
     def forward(self, state=None, number: int = 1, stopStrings: Sequence[str] = ("<|endoftext|>",),
-                stopTokens: Sequence[int] = (0,), progressLambda: Callable[[Dict], None] = lambda x: x,
+                stopTokens: Sequence[int] = (0,), progressLambda: Callable[[Dict], None] = _no_progress,
                 end_adj: float = -990.0, **kwargs):
         ostate = self.myState if state is None else state
+        if self._device_loop(number, stopStrings, progressLambda, kwargs):
+            # one call: token kernel, sampler, stop test and the next embedding all stay on the GPU
+            self._draws = getattr(self, "_draws", 0) + 1
+            toks, logits, ostate = self.model.decode_sample(
+                self.lastToken[0], number, ostate, greedy=self.sampler is greedy, temp=kwargs.get("temp", 1.0),
+                tau=kwargs.get("top_p_usual", 0.8), end_adj=end_adj,
+                seed=(torch.initial_seed() * 1000003 + self._draws) & (2 ** 63 - 1), stop_tokens=list(stopTokens))
+            tokens = [int(t) for t in toks.tolist()]
+            self.myState = ostate
+            self.lastToken = [tokens[-1]]
+            self._raise_if_aborted()
+            return {"logits": logits, "state": ostate, "output": self.tokenizer.decode(tokens)}
         tokens: List[int] = []
         logits, text = None, ""
         for i in range(number):

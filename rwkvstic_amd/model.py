@@ -304,6 +304,33 @@ class HipRWKV:
         return toks[1:], logits, state
 
 
+    def decode_sample(self, token: int, n: int, state: torch.Tensor, *, greedy: bool = False, temp: float = 1.0,
+                      tau: float = 0.8, end_adj: float = 0.0, seed: int = 0, stop_tokens=()):
+        """``RWKVMaster.forward(number=n)`` (rwkvMaster.py:28-56) without a host round trip per token: feed
+        ``token``, then ``n`` times choose the next token on the device (locally typical sampling,
+        agnostic/samplers/typical.py:1-17, or argmax), with ``end_adj`` added to logit 0 before every choice
+        and the loop ending at the first chosen stop token (which is part of the output).  Returns
+        ``(tokens int64 on the device, logits, state)``; ``state`` and ``logits`` are those of the last step
+        that ran.  Needs the persistent single-token kernel (``fused_step``)."""
+        self._check_state(state)
+        if not self.fused_step:
+            raise RuntimeError("decode_sample needs the persistent single-token kernel (fused_step)")
+        toks = torch.empty(n + 1, dtype=torch.int64, device=self.device)
+        toks[0] = int(token)
+        stops = torch.as_tensor(list(stop_tokens), dtype=torch.int64, device=self.device)
+        flag = torch.zeros(1, dtype=torch.int32, device=self.device)
+        done = torch.zeros(1, dtype=torch.int64, device=self.device)
+        ws = self._workspace(1)
+        logits = torch.empty(self.vocab, dtype=torch.float64, device=self.device)
+        with torch.cuda.device(self.device):
+            N.check(N.lib().rwkv_model_decode_sample(
+                self._handle, torch.cuda.current_stream().cuda_stream, toks.data_ptr(), n, state.data_ptr(),
+                logits.data_ptr(), ws.data_ptr(), ws.numel(), 1 if greedy else 0, float(temp), float(tau), float(end_adj),
+                int(seed) & (2 ** 64 - 1), stops.data_ptr() if stops.numel() else None, int(stops.numel()),
+                flag.data_ptr(), done.data_ptr()))
+        return toks[1:1 + int(done)], logits, state
+
+
 def wkv_state_to_reference(state: torch.Tensor) -> torch.Tensor:
     """Rows 2-4 hold the max-shifted triple ``(aa', bb', pp')``; the reference's naive kernel keeps
     ``aa = aa' e^{pp'}``, ``bb = bb' e^{pp'}`` and never touches ``pp`` (cuda/operators.cu:21-36).

@@ -244,6 +244,17 @@ def wkv_f32(w, u, k, v, aa, bb, pp) -> torch.Tensor:
     return y
 
 
+def sample_token(logits: torch.Tensor, *, greedy: bool = False, temp: float = 1.0, tau: float = 0.8, end_adj: float = 0.0,
+                 seed: int = 0, counter: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One choice of the device-side sampler (typical.py:1-17; ``logits[0] += end_adj`` in place first,
+    rwkvMaster.py:37); the uniform number is a hash of ``(seed, counter)``."""
+    _req(logits, torch.float64, "logits"); _contig(logits, "logits")
+    out = out if out is not None else torch.empty(1, dtype=torch.int64, device=logits.device)
+    N.check(N.lib().rwkv_sample_token(_stream(), logits.data_ptr(), logits.numel(), 1 if greedy else 0, float(temp),
+                                      float(tau), float(end_adj), int(seed) & (2 ** 64 - 1), int(counter), out.data_ptr()))
+    return out
+
+
 def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     _req(logits, torch.float64, "logits"); _contig(logits, "logits")
     out = out if out is not None else torch.empty(1, dtype=torch.int64, device=logits.device)
