@@ -224,6 +224,46 @@ def phase_trace(model, L: int, C: int) -> int:
     return 0
 
 
+def batch_decode(model, args, shape) -> int:
+    """B independent sequences (own state, own seeded 64-token prompt), greedy decode by batch steps."""
+    import torch
+    from rwkvstic_amd import synth
+    L, C, F, V = shape
+    B = args.batch
+    states = []
+    toks = []
+    for b in range(B):
+        lg, s = model.forward(synth.random_tokens(64, V=V, seed=100 + b).cuda(), model.emptyState.clone())
+        states.append(s)
+        toks.append(lg.argmax())
+    st = torch.stack(states).contiguous()
+    tok = torch.stack(toks)
+    for _ in range(max(args.warmup, 1)):
+        lg, st = model.forward_batch(tok, st)
+        tok = lg.argmax(dim=1)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        lg, st = model.forward_batch(tok, st)
+        tok = lg.argmax(dim=1)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / args.steps
+    assert bool(torch.isfinite(lg).all())
+    wbytes = model.weight_bytes()
+    print(json.dumps({
+        "metric": f"decode tokens/s @ RWKV-4 {args.shape}-shape fp32i8 B={B}", "value": round(B / (ms / 1e3), 1),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "data": "synthetic",
+        "config": {"workload": f"RWKV-4 {args.shape}-shape (L={L}, C={C}, F={F}, V={V}) fp32i8, {B} independent states, "
+                               f"seeded 64-token prompts, greedy batch steps", "weight_bytes_per_step": wbytes},
+        "roofline": {"bound": "hbm", "achieved": round(wbytes / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(wbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "note": "one batch step streams the weights once for all sequences"}}), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -231,6 +271,12 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--shape", default="3B", choices=["169M", "3B", "14B"])
     ap.add_argument("--prefill", type=int, default=1024)
+    ap.add_argument("--prefill-chunk", type=int, default=0,
+                    help="feed the prompt in chunks of this many tokens (0 = one call); the 14B configuration uses 256")
+    ap.add_argument("--batch", type=int, default=1,
+                    help="instead of the batch-1 benchmark: this many independent sequences, each prefilled with its own "
+                         "64-token random prompt, decoded greedily one batch step at a time (the 14B configuration's "
+                         "batch-32 decode); prints its own JSON line")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-baseline-layers", type=int, default=8,
                     help="layers of the shape the CPU baseline times (0 = all of them; the rest is scaled)")
@@ -274,6 +320,8 @@ def main() -> int:
 
     if args.phase_trace:
         return phase_trace(model, L, C)
+    if args.batch > 1:
+        return batch_decode(model, args, shape)
 
     calibrate_copy(args.calibrate_copy_mib)
 
@@ -284,7 +332,9 @@ def main() -> int:
     e0, e1 = ev(), ev()
     torch.cuda.synchronize()
     e0.record(stream)
-    logits, state = model.forward(prompt, state)
+    chunk = args.prefill_chunk if args.prefill_chunk > 0 else args.prefill
+    for c0 in range(0, args.prefill, chunk):
+        logits, state = model.forward(prompt[c0:c0 + chunk], state)
     e1.record(stream)
     torch.cuda.synchronize()
     prefill_ms = e0.elapsed_time(e1)
@@ -336,6 +386,7 @@ def main() -> int:
                                f"{args.prefill}-token random prompt prefilled, then {args.steps} greedy tokens at batch 1",
                    "weight_bytes_per_token": wbytes, "load_seconds": round(load_s, 2)},
         "prefill_tokens_per_s": round(args.prefill / (prefill_ms / 1e3), 1),
+        "prefill_chunk": chunk,
         "roofline": {"bound": "hbm",
                      "kernel": "rwkv::decode_kernel (persistent, one launch per token; launch_us includes the prep_kernel in front of it)"
                                if model.fused_step

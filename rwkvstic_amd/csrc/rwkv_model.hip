@@ -592,12 +592,14 @@ int rows_layers(rwkv_model *m, hipStream_t st, const int64_t *tokens, int64_t R,
     for (int64_t l = 0; l < d.n_layer; ++l) {
         const rwkv_layer_desc &L = m->layers[l];
         double *sl = state + (size_t)l * 5 * C;
-        // TimeMix (block.py:58-80)
-        if (sequence) RWKV_CHECK_HIP(hipMemcpyAsync(w.prev0, sl, (size_t)C * 8, hipMemcpyDeviceToDevice, st));
+        // TimeMix (block.py:58-80).  Row 0 of a sequence reads the shift state while the last row replaces it,
+        // hence the copy; a single row is read and written by the same threads, in that order, and needs none.
+        const bool copy_prev = sequence && R > 1;
+        if (copy_prev) RWKV_CHECK_HIP(hipMemcpyAsync(w.prev0, sl, (size_t)C * 8, hipMemcpyDeviceToDevice, st));
         const rwkv_qmat *kvr[3] = {&L.att_k, &L.att_v, &L.att_r};
         const float *rg[3] = {kvr[0]->range, kvr[1]->range, kvr[2]->range};
         const double *of[3] = {kvr[0]->offset, kvr[1]->offset, kvr[2]->offset};
-        RWKV_TRY(rows_ln_mix_quant(st, 3, R, C, sequence, w.x, L.ln1_w, L.ln1_b, L.att_mix, sequence ? w.prev0 : sl, sl,
+        RWKV_TRY(rows_ln_mix_quant(st, 3, R, C, sequence, w.x, L.ln1_w, L.ln1_b, L.att_mix, copy_prev ? w.prev0 : sl, sl,
                                    state_stride, rg, of, w.q));
         RowsProduct pk[3];
         for (int i = 0; i < 3; ++i) { pk[i].a = w.q[i]; pk[i].w16 = kvr[i]->packed16; pk[i].out = w.kvr + i * RC; }
@@ -608,10 +610,10 @@ int rows_layers(rwkv_model *m, hipStream_t st, const int64_t *tokens, int64_t R,
         const RowsProduct po = {w.q[0], L.att_o.packed16, w.x};
         RWKV_TRY(rows_products(st, 1, &po, w.tot, R, C, C, ROW_ADD, nullptr));
         // ChannelMix (block.py:82-100)
-        if (sequence) RWKV_CHECK_HIP(hipMemcpyAsync(w.prev0, sl + C, (size_t)C * 8, hipMemcpyDeviceToDevice, st));
+        if (copy_prev) RWKV_CHECK_HIP(hipMemcpyAsync(w.prev0, sl + C, (size_t)C * 8, hipMemcpyDeviceToDevice, st));
         const float *rg2[2] = {L.ffn_k.range, L.ffn_r.range};
         const double *of2[2] = {L.ffn_k.offset, L.ffn_r.offset};
-        RWKV_TRY(rows_ln_mix_quant(st, 2, R, C, sequence, w.x, L.ln2_w, L.ln2_b, L.ffn_mix, sequence ? w.prev0 : sl + C,
+        RWKV_TRY(rows_ln_mix_quant(st, 2, R, C, sequence, w.x, L.ln2_w, L.ln2_b, L.ffn_mix, copy_prev ? w.prev0 : sl + C,
                                    sl + C, state_stride, rg2, of2, w.q + 1));
         const RowsProduct pfk = {w.q[1], L.ffn_k.packed16, w.h}, pfr = {w.q[2], L.ffn_r.packed16, w.kvr};
         RWKV_TRY(rows_products(st, 1, &pfk, w.tot, R, C, F, ROW_RELU2, nullptr));
