@@ -27,23 +27,39 @@ class QuantMatrix:
         self.packed16 = packed16
 
     @classmethod
-    def from_weight(cls, weight: torch.Tensor, device, m16: bool = True) -> "QuantMatrix":
+    def from_weight(cls, weight: torch.Tensor, device, m16: bool = True, stream: bool = False) -> "QuantMatrix":
         """``weight[out, in]`` in any float dtype, on any device."""
         w = weight.to(device=device, dtype=torch.float32).contiguous()
         codes, rng, off = ops.quantize(w)
         n_in, n_out = codes.shape
-        return cls(ops.pack(codes), rng, off, n_in, n_out, ops.pack_m16(codes) if m16 else None)
+        return cls(ops.pack(codes), rng, off, n_in, n_out, ops.pack_m16(codes) if m16 else None)._placed(stream)
 
     @classmethod
-    def from_codes(cls, codes: torch.Tensor, rng: torch.Tensor, off: torch.Tensor, device) -> "QuantMatrix":
+    def from_codes(cls, codes: torch.Tensor, rng: torch.Tensor, off: torch.Tensor, device, stream: bool = False) -> "QuantMatrix":
         """From the reference/.rwkv layout: ``codes[in, out]`` uint8, ``range[in]``, ``offset[in]``."""
         codes = codes.to(device)
         n_in, n_out = codes.shape
         return cls(ops.pack(codes), rng.to(device=device, dtype=torch.float32).contiguous(),
-                   off.to(device=device, dtype=torch.float64).contiguous(), n_in, n_out, ops.pack_m16(codes))
+                   off.to(device=device, dtype=torch.float64).contiguous(), n_in, n_out, ops.pack_m16(codes))._placed(stream)
+
+    def _placed(self, stream: bool) -> "QuantMatrix":
+        """``stream=True`` (the reference's per-device ``stream`` option, matmul.py:21,186: codes stay in host
+        memory, range and offset on the device): the packed codes move to pinned host memory, which the GPU
+        reads in place over the host link while the kernels run; nothing else changes."""
+        if stream:
+            def pinned(t):
+                h = torch.empty(t.shape, dtype=t.dtype, pin_memory=True)
+                h.copy_(t)
+                return h
+            self.packed = pinned(self.packed)
+            if self.packed16 is not None:
+                self.packed16 = pinned(self.packed16)
+        self.stream = stream
+        return self
 
     def codes(self) -> torch.Tensor:
-        return ops.unpack(self.packed, self.n_in, self.n_out)
+        packed = self.packed.to(self.range.device) if not self.packed.is_cuda else self.packed
+        return ops.unpack(packed, self.n_in, self.n_out)
 
     def desc(self) -> N.QMat:
         return N.QMat(self.packed.data_ptr(), self.packed16.data_ptr() if self.packed16 is not None else None,
@@ -55,9 +71,11 @@ class QuantMatrix:
 
 class HipRWKV:
     def __init__(self, weights: Union[Dict[str, torch.Tensor], Iterable[Tuple[str, torch.Tensor]]],
-                 device: str = "cuda", fused: bool = True):
+                 device: str = "cuda", fused: bool = True, stream: bool = False):
         """``fused=False`` skips the second weight layout, so single-token steps run as one launch per
-        phase (the path every shape supports) instead of the persistent kernel."""
+        phase (the path every shape supports) instead of the persistent kernel.  ``stream=True`` keeps the
+        quantised codes of every matrix in pinned host memory (models larger than the GPU's memory; the
+        reference's ``stream`` option, matmul.py:21,186) - the same kernels then read them over the host link."""
         if not torch.cuda.is_available():
             raise RuntimeError("HipRWKV needs a ROCm GPU (gfx950); there is no CPU path in this backend")
         N.lib()
@@ -71,7 +89,7 @@ class HipRWKV:
             if key == "emb.weight":
                 self.emb = t.to(device=self.device, dtype=torch.float32).contiguous()
             elif key.endswith(".weight") and t.dim() == 2:
-                mats[key] = QuantMatrix.from_weight(t, self.device, m16=fused)
+                mats[key] = QuantMatrix.from_weight(t, self.device, m16=fused, stream=stream)
             else:
                 vec[key] = t
         if self.emb is None:

@@ -420,3 +420,27 @@ def test_quantized_tree_round_trip_and_oracle_layout(tmp_path, tiny):
         bad = dict(tree)
         bad["head.weights.0.weight"] = bad["head.weights.0.weight"].float()
         HipRWKV.from_quantized(bad)
+
+
+def test_host_resident_weights_give_identical_results():
+    """stream=True (matmul.py:21,186: the codes stay in host memory): the kernels read the pinned host copies in
+    place; logits and state are bit-identical to the device-resident model, on the prompt path, the persistent
+    single-token kernel and the per-phase kernels."""
+    from rwkvstic_amd.model import HipRWKV
+    sd = synth.make_state_dict(2, 1024, 4096, 1999, seed=31, ln="random")
+    dev, host = HipRWKV(sd), HipRWKV(sd, stream=True)
+    assert host.fused_step and not host.blocks[0]["att_k"].packed16.is_cuda and host.blocks[0]["att_k"].packed16.is_pinned()
+    toks = synth.random_tokens(9, V=1999, seed=4).tolist()
+    l1, s1 = dev.forward(toks, dev.emptyState.clone())
+    l2, s2 = host.forward(toks, host.emptyState.clone())
+    assert torch.equal(l1, l2) and torch.equal(s1, s2)
+    for t in (5, 77):
+        l1, s1 = dev.forward([t], s1)
+        l2, s2 = host.forward([t], s2)
+        host.check()
+        assert torch.equal(l1, l2) and torch.equal(s1, s2)
+    tiny_sd = synth.make_state_dict(layers=2, C=72, F=200, V=301, seed=8, ln="random")
+    a, b = HipRWKV(tiny_sd), HipRWKV(tiny_sd, stream=True)
+    la, sa = a.forward([3, 4], a.emptyState.clone())
+    lb, sb = b.forward([3, 4], b.emptyState.clone())
+    assert torch.equal(la, lb) and torch.equal(sa, sb)

@@ -103,3 +103,50 @@ def test_rwkv_rejects_unknown_modes_and_files():
         RWKV("model.onnx")
     with pytest.raises(TypeError):
         RWKV({}, strategy="cuda fp16")
+
+
+def test_post_contract_and_state_json_round_trip():
+    """server.py:56-86: state in and out as nested float lists, "input" loaded as context, the rest passed to forward."""
+    import json
+    from rwkvstic_amd import serving
+    m, r = _master()
+    r.emptyState = torch.zeros(2, 3, dtype=torch.float64)
+    r.resetState()
+    reply = serving.post(r, {"input": "4 5 6", "number": 2, "stopTokens": [], "end_adj": 0.0})
+    assert m.calls[0] == [4, 5, 6] and len(m.calls) == 3            # the prompt, then two single-token steps
+    assert reply["output"] == "188 189" or len(reply["output"].split()) == 2
+    assert isinstance(reply["logits"], list) and len(reply["logits"]) == StubModel.V
+    assert isinstance(reply["state"], list) and len(reply["state"]) == 2 and len(reply["state"][0]) == 3
+    wire = json.loads(json.dumps(reply))                             # survives the wire format
+    # the returned state fed back continues where the first request stopped
+    before = len(m.calls)
+    reply2 = serving.post(r, {"state": wire["state"], "number": 1, "stopTokens": [], "end_adj": 0.0})
+    assert len(m.calls) == before + 1
+    assert float(torch.tensor(reply2["state"]).flatten()[0]) == float(torch.tensor(wire["state"]).flatten()[0]) + 1
+    # a state of the wrong shape is refused
+    import pytest as _pytest
+    with _pytest.raises(ValueError):
+        serving.post(r, {"state": [[0.0]], "number": 1})
+    # float32 on the wire: the empty WKV row's -1e30 survives, finer digits do not
+    st = torch.tensor([[-1e30, 1.0 + 2 ** -30, 0.5]], dtype=torch.float64)
+    back = serving.state_from_json(serving.state_to_json(st), st)
+    assert back.dtype == torch.float64 and float(back[0, 0]) == float(torch.tensor(-1e30, dtype=torch.float32))
+    assert float(back[0, 1]) == 1.0 and float(back[0, 2]) == 0.5
+
+
+def test_http_handler_speaks_the_wire_format():
+    import json
+    import threading
+    import urllib.request
+    import socketserver
+    from rwkvstic_amd import serving
+    m, r = _master()
+    with socketserver.TCPServer(("127.0.0.1", 0), serving.make_handler(r)) as httpd:
+        port = httpd.server_address[1]
+        t = threading.Thread(target=httpd.handle_request)
+        t.start()
+        req = urllib.request.Request(f"http://127.0.0.1:{port}/", data=json.dumps({"number": 1, "stopTokens": []}).encode(),
+                                     headers={"Content-Type": "application/json"})
+        reply = json.loads(urllib.request.urlopen(req, timeout=10).read())
+        t.join()
+    assert set(reply) >= {"logits", "state", "output"}
