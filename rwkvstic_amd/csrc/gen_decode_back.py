@@ -41,6 +41,13 @@ DEFER = int(os.environ.get("RWKV_BACK_DEFER", "1"))
 WINDOWS = [int(x) for x in os.environ.get("RWKV_BACK_WINDOWS", ",".join([str(WINDOW)] * 4)).split(",")]
 BURST = int(os.environ.get("RWKV_BACK_BURST", "0"))      # the first BURST reloads after a phase's barrier go out back to back
 PACE = int(os.environ.get("RWKV_BACK_PACE", "0"))        # s_sleep units (64 cycles) in front of every deferred reload: the reloads of a phase go out at a steady rate instead of as fast as the window allows
+# RWKV_BACK_GATE="a,b,c,d": after the barrier of the att k/v/r, att output, ffn key and ffn value phases only the first
+# a / b / c / d deferred reloads go out at once; the rest wait until the front waves have seen every workgroup's
+# results of the NEXT exchange arrive (LDS word FLAG_GO), so that those polls and gathers do not queue behind a
+# burst of weight loads.  Empty: no gate.
+GATE = [int(x) for x in os.environ.get("RWKV_BACK_GATE", "8,5,12,12").split(",")] if os.environ.get("RWKV_BACK_GATE", "8,5,12,12") else None
+GATE_SPINS = 1 << 16     # the gate gives way after this many looks (a few milliseconds): it only orders loads, it must never hold a wave
+S_SEQ = 98        # phases finished by this wave (the front waves' exchange sequence number runs one ahead)
 SLEEP = int(os.environ.get("RWKV_BACK_SLEEP", "0"))      # s_sleep units (64 cycles) between a phase's barrier and its reloads   # weight loads a wave keeps in flight while it reloads slots
 
 
@@ -151,6 +158,7 @@ def gen(KW, R, NV, NSH):
         e(f"v_add_u32 v{V_OFF + b}, {8192 * b}, v{V_OFF}")
     e(f"s_mov_b64 s[{S_JT}:{S_JT + 1}], %[jt]")
     e(f"s_mov_b32 s{S_L}, %[L]")
+    e(f"s_mov_b32 s{S_SEQ}, 0")
     for base, off in ((S_CUR, 0), (S_NXT, 128)):
         e(f"s_load_dwordx16 s[{base}:{base + 15}], s[{S_JT}:{S_JT + 1}], {off}")
         e(f"s_load_dwordx8 s[{base + 16}:{base + 23}], s[{S_JT}:{S_JT + 1}], {off + 64}")
@@ -225,8 +233,28 @@ def gen(KW, R, NV, NSH):
             deferred += list(range(NREAL, PP))     # padding positions: nothing to compute, only their turn to load
         if SLEEP and deferred:
             e(f"s_sleep {SLEEP}")
+        e(f"s_add_u32 s{S_SEQ}, s{S_SEQ}, 1")
         for i, p in enumerate(deferred):
             assert issued_loads == p + R
+            if GATE is not None and i == GATE[ph]:
+                # wait for FLAG_GO >= phases finished + 1 (or the abort flag: then the next barrier check leaves)
+                e(f"s_add_u32 s{S_T}, s{S_SEQ}, 1")
+                e(f"s_mov_b32 s{S_TILE}, {GATE_SPINS}")       # (free until the head)
+                e(f"7{ph}:")
+                e(f"ds_read_b64 v[{V_A}:{V_A + 1}], v{V_FLAG}")
+                e("s_waitcnt lgkmcnt(0)")
+                e(f"v_readfirstlane_b32 vcc_lo, v{V_A}")
+                e(f"v_readfirstlane_b32 vcc_hi, v{V_A + 1}")
+                e("s_cmp_lg_u32 vcc_lo, 0")
+                e(f"s_cbranch_scc1 6{ph}f")
+                e(f"s_cmp_ge_i32 vcc_hi, s{S_T}")
+                e(f"s_cbranch_scc1 6{ph}f")
+                e(f"s_sub_u32 s{S_TILE}, s{S_TILE}, 1")
+                e(f"s_cmp_eq_u32 s{S_TILE}, 0")
+                e(f"s_cbranch_scc1 6{ph}f")
+                e("s_sleep 1")
+                e(f"s_branch 7{ph}b")
+                e(f"6{ph}:")
             if PACE and i >= BURST:
                 e(f"s_sleep {PACE}")
             layer_reload(p, max(BURST, WINDOWS[ph]) if i < BURST else WINDOWS[ph])

@@ -69,7 +69,7 @@ constexpr int kEarlyDiv = RWKV_EARLY_DIV;           // gathers start when all bu
 constexpr int kHeadCsPerThread = 4;    // head column sums a front thread fetches: 16 per head tile of the workgroup
 
 // LDS flag words
-enum { FLAG_ARRIVED = 0, FLAG_SCALE = 1, FLAG_ABORT = 2, FLAG_ALL = 3, FLAG_COUNT = 4 };
+enum { FLAG_ARRIVED = 0, FLAG_SCALE = 1, FLAG_ABORT = 2, FLAG_GO = 3, FLAG_COUNT = 4 };   // FLAG_GO: see the reload gate of the generated back-wave program
 
 // Pointers that were themselves loaded from memory are "flat" to the compiler, and a flat load
 // counts against the LDS counter as well as the vector-memory counter: every wait for an LDS read
@@ -550,6 +550,7 @@ __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, co
     if (fx.wave == 0) {
         RowPoll<kStatRows, G> r;
         r.poll(fx, a.b.XR, epoch, seq, kStatRows * (G / kEarlyDiv), [&] { issue_quads<FT, NQT>(xt, fx.tid, 0, NQ, w); });
+        if (fx.lane == 0) fx.flags[FLAG_GO] = seq;                // every workgroup's publish has been seen: opens the reload gate
         if (tp && fx.tid == 0) tp[0] = wall_clock64();
         // groups of 16 channels combined: mean of the group sums, variance from the groups' own squared
         // deviations plus the spread of the group means
@@ -621,6 +622,7 @@ __device__ __forceinline__ void vec_front(Front &fx, int &seq, const u64 *src, c
     if (fx.wave == 0) {
         RowPoll<3, G> r;
         r.poll(fx, rec, epoch, seq, 3 * (G / kEarlyDiv), [&] { issue_quads<FT, CH>(st, fx.tid, 0, nq, w[0]); });
+        if (fx.lane == 0) fx.flags[FLAG_GO] = seq;
         if (tp && fx.tid == 0) tp[0] = wall_clock64();
         const float mx = wave_max_dpp(r.lane_max(fx, 0));
         const double so = wave_sum_dpp(r.lane_sum(fx, 1) + r.lane_sum(fx, 2));
