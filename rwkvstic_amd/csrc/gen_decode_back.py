@@ -42,10 +42,13 @@ WINDOWS = [int(x) for x in os.environ.get("RWKV_BACK_WINDOWS", ",".join([str(WIN
 BURST = int(os.environ.get("RWKV_BACK_BURST", "0"))      # the first BURST reloads after a phase's barrier go out back to back
 PACE = int(os.environ.get("RWKV_BACK_PACE", "0"))        # s_sleep units (64 cycles) in front of every deferred reload: the reloads of a phase go out at a steady rate instead of as fast as the window allows
 # RWKV_BACK_GATE="a,b,c,d": after the barrier of the att k/v/r, att output, ffn key and ffn value phases only the first
-# a / b / c / d deferred reloads go out at once; the rest wait until the front waves have seen every workgroup's
-# results of the NEXT exchange arrive (LDS word FLAG_GO), so that those polls and gathers do not queue behind a
-# burst of weight loads.  Empty: no gate.
-GATE = [int(x) for x in os.environ.get("RWKV_BACK_GATE", "8,5,12,12").split(",")] if os.environ.get("RWKV_BACK_GATE", "8,5,12,12") else None
+# a / b / c / d deferred reloads go out at once, so that the front waves' polls and gathers of the NEXT exchange do
+# not queue behind a burst of weight loads.  The rest follow once every workgroup's results of that exchange have
+# arrived: for the att k/v/r and ffn key phases a bounded spin on the LDS word FLAG_GO, for the att output and ffn
+# value phases (BARGATE) simply after the first barrier of the LayerNorm phase that follows, which the front waves
+# only reach with the statistics of all workgroups in hand.  Empty: no gate.
+GATE = [int(x) for x in os.environ.get("RWKV_BACK_GATE", "8,2,12,6").split(",")] if os.environ.get("RWKV_BACK_GATE", "8,2,12,6") else None
+BARGATE = int(os.environ.get("RWKV_BACK_BARGATE", "1"))   # reloads deferred past the att output and ffn value phases follow the next phase's first barrier
 GATE_SPINS = 1 << 16     # the gate gives way after this many looks (a few milliseconds): it only orders loads, it must never hold a wave
 S_SEQ = 98        # phases finished by this wave (the front waves' exchange sequence number runs one ahead)
 SLEEP = int(os.environ.get("RWKV_BACK_SLEEP", "0"))      # s_sleep units (64 cycles) between a phase's barrier and its reloads   # weight loads a wave keeps in flight while it reloads slots
@@ -164,7 +167,23 @@ def gen(KW, R, NV, NSH):
         e(f"s_load_dwordx8 s[{base + 16}:{base + 23}], s[{S_JT}:{S_JT + 1}], {off + 64}")
         e(f"s_load_dwordx2 s[{base + 24}:{base + 25}], s[{S_JT}:{S_JT + 1}], {off + 96}")
     e("s_waitcnt lgkmcnt(0)")
+    # Which reloads follow a barrier instead of a spin gate: those deferred past a phase whose successor starts with
+    # the statistics barrier (att output -> ffn key/receptance; ffn value -> next layer / head).  What the ffn value
+    # phase carries over is issued at the top of the next layer, after that layer's first barrier - also in the
+    # first layer, which is why the prologue leaves those positions out.
+    phases = [(0, 3 * KW, 2), (3 * KW, 4 * KW, 1), (4 * KW, 9 * KW, 2), (9 * KW, 13 * KW, 1)]   # start, end, barriers before
+    def deferred_of(ph):
+        ps, pe, _ = phases[ph]
+        d = [p for p in range(ps, pe) if not (p + R < pe and DEFER) and DEFER]
+        if pe == NREAL:
+            d += list(range(NREAL, PP))
+        return d
+    carry_d = deferred_of(3)[GATE[3]:] if (GATE is not None and BARGATE) else []
+    assert all(p + R >= PP for p in carry_d)
+    skip = set(p + R - PP for p in carry_d)
     for p in range(R):
+        if p in skip:
+            continue
         j, b = divmod(p, KW)
         e(f"global_load_dwordx4 {ring(p)}, v{V_OFF + b}, s[{S_CUR + 2 * j}:{S_CUR + 2 * j + 1}]")
 
@@ -173,23 +192,24 @@ def gen(KW, R, NV, NSH):
     # is reloaded right away only when its next position still belongs to the current phase;
     # otherwise the reload waits until the phase's tiles are parked and the barrier is passed, so
     # that pushing requests into a busy memory system never delays the phase's results.
-    phases = [(0, 3 * KW, 2), (3 * KW, 4 * KW, 1), (4 * KW, 9 * KW, 2), (9 * KW, 13 * KW, 1)]   # start, end, barriers before
-
     def throttle(window=WINDOW):
         # A burst of reloads would sit in the compute unit's memory pipeline in front of the front
         # waves' polls and stores; keeping a window in flight paces the requests to what HBM delivers.
         if window - 1 < R - 1:
             e(f"s_waitcnt vmcnt({window - 1})")
 
-    def layer_reload(p, window=WINDOW):
-        """Reload the slot of layer position p (0 <= p < PP) with position p + R."""
+    def layer_reload(p, window=WINDOW, top=False):
+        """Reload the slot of layer position p (0 <= p < PP) with position p + R.  top: issued at the top of the
+        NEXT layer (or of the head), where that layer's addresses have already become the current ones."""
         throttle(window)
         slot = p % R
         q = p + R
         sset = S_CUR
         if q >= PP:
             q -= PP
-            sset = S_NXT
+            sset = S_CUR if top else S_NXT
+        else:
+            assert not top
         if q >= NREAL:
             e(f"global_load_dwordx4 {ring(slot)}, v{V_OFF}, %[wh]")
         else:
@@ -197,9 +217,15 @@ def gen(KW, R, NV, NSH):
             e(f"global_load_dwordx4 {ring(slot)}, v{V_OFF + bq}, s[{sset + 2 * jq}:{sset + 2 * jq + 1}]")
 
     e("1:")
+    carry = []
     for ph, (ps, pe, nbar) in enumerate(phases):
-        for _ in range(nbar):
+        for k in range(nbar):
             bar_check()
+            if k == 0 and nbar == 2:
+                # behind the statistics barrier: every exchange word of this phase has been fetched
+                for p in (carry_d if ph == 0 else carry):
+                    layer_reload(p, WINDOWS[ph], top=(ph == 0))
+                carry = []
         for q in range(ps, min(ps + PF, pe)):
             aread(q)
         issued_loads = ps + R          # loads issued so far: positions < ps + R
@@ -234,6 +260,10 @@ def gen(KW, R, NV, NSH):
         if SLEEP and deferred:
             e(f"s_sleep {SLEEP}")
         e(f"s_add_u32 s{S_SEQ}, s{S_SEQ}, 1")
+        assert deferred == deferred_of(ph)
+        if GATE is not None and BARGATE and ph in (1, 3):
+            carry = deferred[GATE[ph]:]
+            deferred = deferred[:GATE[ph]]
         for i, p in enumerate(deferred):
             assert issued_loads == p + R
             if GATE is not None and i == GATE[ph]:
@@ -299,6 +329,8 @@ def gen(KW, R, NV, NSH):
     assert tiles_per_body % NSH == 0
     e("2:")
     bar_check()
+    for p in carry_d:
+        layer_reload(p, WINDOW, top=True)
     bar_check()
     e(f"s_mov_b32 s{S_TILE}, 0")
     e(f"s_mov_b32 s{S_PAR}, 0")
