@@ -26,7 +26,7 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E vendor peak
 # both scaled by a 1 GiB device copy in the same run; profiles/decode_kernel_3B_b1_hbm_traffic.md): a measured
 # constant per shape, not something this script can read live.  It is tied to the kernel sources it was measured on
 # by their digest (csrc_digest() below): with any other sources the bench reports null instead of a stale figure.
-PMC_TRAFFIC = {"3B": {"bytes": 2_964_600_000, "csrc_digest": "unmeasured"}}
+PMC_TRAFFIC = {"3B": {"bytes": 2_965_400_000, "csrc_digest": "557184e2139ce3f3"}}
 
 
 def csrc_digest() -> str:
@@ -290,7 +290,13 @@ def main() -> int:
                     help="instead of the benchmark: one token step of the persistent kernel with its 100 MHz phase "
                          "stamps switched on (rwkv_model_set_trace), printed as a table of min / median / max over "
                          "the workgroups per phase boundary, for three layers")
+    ap.add_argument("--lib", default=None,
+                    help="load this build of the library instead of the in-tree one (a diagnostic build made with "
+                         "`python -m rwkvstic_amd.build --define NAME --output FILE`)")
     args = ap.parse_args()
+    if args.lib:
+        from rwkvstic_amd import _native
+        _native.LIB_PATH = os.path.abspath(args.lib)
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (batch-1 decode of one model replica); "
               "--gpus must be 1", file=sys.stderr)

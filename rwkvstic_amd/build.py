@@ -31,17 +31,25 @@ def hipcc() -> str:
     return exe
 
 
-def build(verbose: bool = True, extra_flags=()) -> str:
+def build(verbose: bool = True, extra_flags=(), output: str | None = None) -> str:
+    """output: write the library there instead of next to this file (diagnostic builds, e.g. with
+    ``-DRWKV_DIAG_HOT_WEIGHTS``; ``bench.py --lib`` loads such a file)."""
     srcs = [os.path.join(CSRC, s) for s in SOURCES]
-    tmp = LIB + ".tmp"
+    out = os.path.abspath(output) if output else LIB
+    tmp = out + ".tmp"
     cmd = [hipcc(), *FLAGS, *extra_flags, "-o", tmp, *srcs]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
-    os.replace(tmp, LIB)
-    return LIB
+    os.replace(tmp, out)
+    return out
 
 
 if __name__ == "__main__":
-    build()
-    print(LIB)
+    import argparse
+
+    ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("--define", action="append", default=[], metavar="NAME[=VALUE]", help="preprocessor definition (repeatable)")
+    ap.add_argument("--output", default=None, help="library file to write (default: in-tree librwkv_hip.so)")
+    ns = ap.parse_args()
+    print(build(extra_flags=[f"-D{d}" for d in ns.define], output=ns.output))

@@ -49,6 +49,8 @@ PACE = int(os.environ.get("RWKV_BACK_PACE", "0"))        # s_sleep units (64 cyc
 # only reach with the statistics of all workgroups in hand.  Empty: no gate.
 GATE = [int(x) for x in os.environ.get("RWKV_BACK_GATE", "8,2,12,6").split(",")] if os.environ.get("RWKV_BACK_GATE", "8,2,12,6") else None
 BARGATE = int(os.environ.get("RWKV_BACK_BARGATE", "1"))   # reloads deferred past the att output and ffn value phases follow the next phase's first barrier
+CARRYK = int(os.environ.get("RWKV_BACK_CARRYK", "0"))     # the carried reloads follow this barrier of the LayerNorm phase (0: statistics, 1: digits ready)
+CARRYW = int(os.environ.get("RWKV_BACK_CARRYW", "0"))     # window of the carried reloads (0: the phase's)
 GATE_SPINS = 1 << 16     # the gate gives way after this many looks (a few milliseconds): it only orders loads, it must never hold a wave
 S_SEQ = 98        # phases finished by this wave (the front waves' exchange sequence number runs one ahead)
 SLEEP = int(os.environ.get("RWKV_BACK_SLEEP", "0"))      # s_sleep units (64 cycles) between a phase's barrier and its reloads   # weight loads a wave keeps in flight while it reloads slots
@@ -221,10 +223,10 @@ def gen(KW, R, NV, NSH):
     for ph, (ps, pe, nbar) in enumerate(phases):
         for k in range(nbar):
             bar_check()
-            if k == 0 and nbar == 2:
+            if k == CARRYK and nbar == 2:
                 # behind the statistics barrier: every exchange word of this phase has been fetched
                 for p in (carry_d if ph == 0 else carry):
-                    layer_reload(p, WINDOWS[ph], top=(ph == 0))
+                    layer_reload(p, CARRYW or WINDOWS[ph], top=(ph == 0))
                 carry = []
         for q in range(ps, min(ps + PF, pe)):
             aread(q)
@@ -329,9 +331,13 @@ def gen(KW, R, NV, NSH):
     assert tiles_per_body % NSH == 0
     e("2:")
     bar_check()
-    for p in carry_d:
-        layer_reload(p, WINDOW, top=True)
+    if CARRYK == 0:
+        for p in carry_d:
+            layer_reload(p, CARRYW or WINDOW, top=True)
     bar_check()
+    if CARRYK == 1:
+        for p in carry_d:
+            layer_reload(p, CARRYW or WINDOW, top=True)
     e(f"s_mov_b32 s{S_TILE}, 0")
     e(f"s_mov_b32 s{S_PAR}, 0")
     e(f"s_mov_b32 s{S_RT}, {R // KW - (1 if R % KW == 0 else 0)}")
