@@ -20,10 +20,16 @@ the checks live in ``tests/test_oracle_*.py``):
   matrices.  The reference holds no golden vectors for it.
 * ``mm8_naive``        – equals a float64 dense product on the canonically
   dequantised matrix to float32 accumulation error.
+* ``mm8_general_f64``  – the four-vector form (row and column ranges and
+  offsets) equals three nested scalar loops on a 3 x 4 matrix, with each of the
+  per-column vectors present or absent.
 * ``layernorm``        – equals ``torch.nn.functional.layer_norm`` in float64.
 * ``wkv_naive``        – equals the O(T^2) direct sum of textbook RWKV-4, the
   max-shifted recurrence ``wkv_stable``, the geometric-series closed form for
   constant input, and is split-invariant in T.
+* ``typical_distribution`` – hand-worked kept sets and probabilities for the
+  distribution (1/2, 1/4, 1/8, 1/8) at four values of tau and with a
+  temperature; uniform logits keep every token.
 * ``block_forward`` / ``model_forward`` – composition of the above; token
   shift and state rows pinned by chunk-size invariance (T tokens at once ==
   T single-token calls) and by ``state[0]/state[1]`` equalling the last

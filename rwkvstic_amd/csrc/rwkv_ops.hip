@@ -38,18 +38,34 @@ mm8_packed_kernel(int n_in, int n_out, int n_kb, int kc_blocks,
     for (int kb0 = 0; kb0 < n_kb; kb0 += kc_blocks) {
         const int kb1 = min(kb0 + kc_blocks, n_kb);
         const int j0 = kb0 * kBlockRows;
-        for (int i = threadIdx.x; i < (kb1 - kb0) * kBlockRows; i += kThreads) {
-            const int j = j0 + i;
+        // kStageAhead rows per thread at a time, every load of the group issued before the first use: the loop is
+        // otherwise a chain of dependent memory latencies (NB loads of x per row, one row after the other)
+        constexpr int kStageAhead = NB >= 4 ? 4 : 8;
+        const int rows_here = (kb1 - kb0) * kBlockRows;
+        for (int i0 = threadIdx.x; i0 < rows_here; i0 += kStageAhead * kThreads) {
+            float xv[kStageAhead][NB], rr[kStageAhead];
+            double mr[kStageAhead];
 #pragma unroll
-            for (int b = 0; b < NB; ++b) {
-                float v = 0.f;
-                if (j < n_in) {
-                    const double xv = (double)x[(size_t)b * n_in + j];
-                    v = (float)(xv * (double)r_row[j]);
-                    zsum[b] += xv * m_row[j];
-                    zsum[NB + b] += xv;
+            for (int u = 0; u < kStageAhead; ++u) {
+                const int i = i0 + u * kThreads, j = j0 + i;
+                const bool in = i < rows_here && j < n_in;
+                rr[u] = in ? r_row[j] : 0.f;
+                mr[u] = in ? m_row[j] : 0.0;
+#pragma unroll
+                for (int b = 0; b < NB; ++b) xv[u][b] = in ? x[(size_t)b * n_in + j] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < kStageAhead; ++u) {
+                const int i = i0 + u * kThreads;
+                if (i < rows_here) {
+#pragma unroll
+                    for (int b = 0; b < NB; ++b) {
+                        const double xd = (double)xv[u][b];
+                        xs[(size_t)b * kc_rows + i] = (float)(xd * (double)rr[u]);      // matmul.py:131
+                        zsum[b] += xd * mr[u];
+                        zsum[NB + b] += xd;
+                    }
                 }
-                xs[(size_t)b * kc_rows + i] = v;
             }
         }
         __syncthreads();

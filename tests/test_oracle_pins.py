@@ -262,3 +262,31 @@ def test_model_matches_unquantised_float64_network(tiny):
     # 8-bit weights: agreement to quantisation noise, far below the logit scale (~0.16)
     assert (got - want).abs().max() < 0.02
     assert torch.corrcoef(torch.stack([got, want]))[0, 1] > 0.995
+
+
+# ---------------------------------------------------------------- sampler
+def test_typical_distribution_hand_worked_cases():
+    """Probabilities (1/2, 1/4, 1/8, 1/8): surprises (1, 2, 3, 3) ln 2, entropy 1.75 ln 2, distances to the entropy
+    (0.75, 0.25, 1.25, 1.25) ln 2.  In order of distance the tokens are 1, 0, then 2 and 3 tied, with cumulative mass
+    0.25, 0.75, 0.875, 1.  The kept set is everything not farther than the token at position #(cumulative < tau):
+    worked by hand for four values of tau, and with a temperature (kept probabilities to the power 1 / temp)."""
+    logits = torch.log(torch.tensor([0.5, 0.25, 0.125, 0.125])) + 3.0       # softmax is shift invariant
+    cases = {
+        0.2: [0.0, 1.0, 0.0, 0.0],                 # only the token closest to the entropy - not the most probable one
+        0.5: [2 / 3, 1 / 3, 0.0, 0.0],
+        0.8: [0.5, 0.25, 0.125, 0.125],            # position 2 is one of the tied pair: both stay
+        0.99: [0.5, 0.25, 0.125, 0.125],
+    }
+    for tau, want in cases.items():
+        got = O.typical_distribution(logits, temp=1.0, tau=tau)
+        assert torch.allclose(got, torch.tensor(want, dtype=torch.float64), atol=1e-6), (tau, got)
+    got = O.typical_distribution(logits, temp=2.0, tau=0.5)
+    a, b = math.sqrt(0.5), math.sqrt(0.25)
+    assert torch.allclose(got, torch.tensor([a / (a + b), b / (a + b), 0.0, 0.0], dtype=torch.float64), atol=1e-6)
+
+
+def test_typical_distribution_uniform_logits_keep_everything():
+    """All surprises equal the entropy: every distance is zero, nothing can be cut, whatever tau."""
+    for tau in (0.01, 0.5, 0.95):
+        got = O.typical_distribution(torch.full((37,), -1.25), temp=0.7, tau=tau)
+        assert torch.allclose(got, torch.full((37,), 1 / 37, dtype=torch.float64), atol=1e-7)
