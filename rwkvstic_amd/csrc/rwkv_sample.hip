@@ -7,16 +7,23 @@
 // that one, are kept (everything with d greater than its d is zeroed);  kept p^(1/temp) is sampled.
 // The order itself is never needed: the cut is the smallest d* among the tokens with mass{d <= d*} >= tau,
 // found by a radix search over the bit pattern of d (non-negative floats order like their bits), two bits
-// per round.  One workgroup of 1024 threads; thread t owns the contiguous tokens [t * CH, (t + 1) * CH).
+// per round.  One workgroup of 1024 threads; thread t owns the tokens t, t + 1024, ... (coalesced reads of the
+// logits).  The probabilities stay in registers; of the keys the first kSKeysLds per thread live in LDS and the
+// rest in registers: both arrays in registers would not fit the 128 registers a wave of a 1024-thread workgroup has.
 #include "rwkv_common.h"
 #include "rwkv_sample.h"
+
+#include <mutex>
 
 namespace rwkv {
 
 namespace {
 
 constexpr int kST = 1024;            // threads
-constexpr int kSMaxPer = 52;         // tokens per thread kept in registers (probability and key): vocabularies up to 53248
+constexpr int kSMaxPer = 52;         // tokens per thread: vocabularies up to 53248
+constexpr int kSFirstBit = 16;       // full passes settle the key's bits down to this one before the first attempt to list the undecided tokens
+constexpr int kSList = 2048;         // tokens that share the upper half of the cut's key: finished by one wave
+constexpr int kSKeysLds = 32;        // keys per thread kept in LDS ([k][thread]: conflict-free), 128 KiB
 
 __device__ __forceinline__ float block_sum_f(float v, float *scr) {
     v = wave_sum(v);
@@ -52,28 +59,29 @@ __device__ __forceinline__ float uniform01(unsigned long long seed, unsigned lon
 template <int PER>
 __global__ void __launch_bounds__(kST)
 sample_kernel(SampleArgs a) {
+    constexpr int KL = PER < kSKeysLds ? PER : kSKeysLds, KR = PER - KL > 0 ? PER - KL : 1;
+    extern __shared__ unsigned key_lds[];            // [KL][kST]
     __shared__ float scr[3 * (kST / 64)];
     __shared__ float wsum[kST / 64];
-    __shared__ int s_tok;
+    __shared__ int s_tok, s_cnt;
+    __shared__ unsigned s_prefix;
+    __shared__ unsigned list_key[kSList];
+    __shared__ float list_p[kSList];
     if (a.stop_flag && *a.stop_flag) return;         // a stop token ended the sequence: the rest of the loop is skipped
     const int V = a.V, tid = threadIdx.x;
-    const int CH = (V + kST - 1) / kST, i0 = tid * CH;
     if (a.end_adj != 0.0 && tid == 0) a.logits[0] += a.end_adj;       // rwkvMaster.py:37, kept in the returned logits
     __syncthreads();
     float p[PER];                                    // first the float32 logits, then the probabilities
     float mx = -INFINITY;
-#pragma unroll
-    for (int k = 0; k < PER; ++k) {
-        const int i = i0 + k;
-        p[k] = (k < CH && i < V) ? (float)a.logits[i] : -INFINITY;
-        mx = fmaxf(mx, p[k]);
-    }
-    mx = block_max_f(mx, scr);
     int token = 0;
     if (a.greedy) {
         // first maximum (float64 comparison on the stored logits, as the greedy loop does)
         double best = -INFINITY; int bi = 0x7fffffff;
-        for (int k = 0; k < CH; ++k) { const int i = i0 + k; if (i < V) { const double x = a.logits[i]; if (x > best) { best = x; bi = i; } } }
+#pragma unroll 13
+        for (int k = 0; k < PER; ++k) {
+            const int i = tid + kST * k;
+            if (i < V) { const double x = a.logits[i]; if (x > best) { best = x; bi = i; } }      // i grows with k: the first of equals stays
+        }
 #pragma unroll
         for (int off = 32; off >= 1; off >>= 1) {
             const double ob = __shfl_xor(best, off, 64); const int oi = __shfl_xor(bi, off, 64);
@@ -89,56 +97,120 @@ sample_kernel(SampleArgs a) {
         __syncthreads();
         token = s_tok;
     } else {
-        // softmax in float32 (typical.py:5)
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+            const int i = tid + kST * k;
+            p[k] = i < V ? (float)a.logits[i] : -INFINITY;
+            mx = fmaxf(mx, p[k]);
+            if (k % 13 == 12) __builtin_amdgcn_sched_barrier(0);      // at most 13 float64 loads in flight: all 52 at once would not fit the registers
+        }
+        mx = block_max_f(mx, scr);
+        // softmax in float32 (typical.py:5); the hardware exponential (about one ulp) is enough here: only a tie at
+        // the edge of the kept set could fall the other way.  p[k] holds t = logit - max until the last pass.
         float z = 0.f;
 #pragma unroll
-        for (int k = 0; k < PER; ++k) { p[k] = expf(p[k] - mx); z += p[k]; }       // exp(-inf) = 0 past the end
+        for (int k = 0; k < PER; ++k) { p[k] -= mx; z += __expf(p[k]); }          // exp(-inf) = 0 past the end
         z = block_sum_f(z, scr);
-        const float rz = 1.0f / z;
-        // surprise, entropy (nansum: terms with p == 0 are skipped), distance from the entropy
+        const float rz = 1.0f / z, logz = logf(z);
+        // surprise s = -log p = log z - t (no logarithm per token), entropy (nansum: terms with p == 0 are skipped)
         float h = 0.f;
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
-            p[k] *= rz;
-            if (p[k] > 0.f) h -= logf(p[k]) * p[k];
+            const float pk = __expf(p[k]) * rz;
+            if (pk > 0.f) h += (logz - p[k]) * pk;
         }
         h = block_sum_f(h, scr);
-        unsigned key[PER];
+        // distance from the entropy as the search key
+        unsigned kreg[KR];
+#define RWKV_KEY(k) ((k) < KL ? key_lds[(k) * kST + tid] : kreg[(k) - KL < KR ? (k) - KL : 0])
 #pragma unroll
-        for (int k = 0; k < PER; ++k) key[k] = p[k] > 0.f ? __float_as_uint(fabsf(-logf(p[k]) - h)) : 0x7f800000u;   // p == 0: d = inf
-        // radix search, most significant bits first: the largest prefix P with mass{key < P} < tau
+        for (int k = 0; k < PER; ++k) {
+            const float pk = __expf(p[k]) * rz;
+            const unsigned key = pk > 0.f ? __float_as_uint(fabsf(logz - p[k] - h)) : 0x7f800000u;   // p == 0: d = inf
+            if (k < KL) key_lds[k * kST + tid] = key; else kreg[k - KL < KR ? k - KL : 0] = key;      // (each thread reads back only its own)
+            p[k] = pk;
+        }
+        // Radix search, most significant bits first, two bits per round: the largest prefix P with mass{key < P} < tau.
+        // `below` = mass{key < prefix}.
         unsigned prefix = 0;
-        for (int shift = 30; shift >= 0; shift -= 2) {
-            float m1 = 0.f, m2 = 0.f, m3 = 0.f;
-            const unsigned c1 = prefix | (1u << shift), c2 = prefix | (2u << shift), c3 = prefix | (3u << shift);
+        float below = 0.f;
+#define RWKV_FULL_ROUND(shift)                                                                                           \
+        {                                                                                                                \
+            float m1 = 0.f, m2 = 0.f, m3 = 0.f;                                                                          \
+            const unsigned c1 = prefix | (1u << (shift)), c2 = prefix | (2u << (shift)), c3 = prefix | (3u << (shift));  \
+            _Pragma("unroll") for (int k = 0; k < PER; ++k) {                                                            \
+                const unsigned key = RWKV_KEY(k);                                                                        \
+                m1 += key < c1 ? p[k] : 0.f;                                                                             \
+                m2 += key < c2 ? p[k] : 0.f;                                                                             \
+                m3 += key < c3 ? p[k] : 0.f;                                                                             \
+            }                                                                                                            \
+            m1 = wave_sum(m1); m2 = wave_sum(m2); m3 = wave_sum(m3);       /* three sums with one pair of barriers */     \
+            __syncthreads();                                                                                             \
+            if ((tid & 63) == 0) { scr[tid >> 6] = m1; scr[kST / 64 + (tid >> 6)] = m2; scr[2 * (kST / 64) + (tid >> 6)] = m3; } \
+            __syncthreads();                                                                                             \
+            float t1 = 0.f, t2 = 0.f, t3 = 0.f;                                                                          \
+            _Pragma("unroll") for (int w = 0; w < kST / 64; ++w) { t1 += scr[w]; t2 += scr[kST / 64 + w]; t3 += scr[2 * (kST / 64) + w]; } \
+            if (t3 < a.tau) { prefix = c3; below = t3; } else if (t2 < a.tau) { prefix = c2; below = t2; }               \
+            else if (t1 < a.tau) { prefix = c1; below = t1; }                                                            \
+        }
+        // After 16 (or 20, 24, 28) bits only the tokens that share those bits with the cut can still decide the rest.
+        // As soon as they fit a list of kSList entries, one wave finishes alone: no pass over all tokens, no barriers.
+        int shift = 30;
+        for (; shift >= kSFirstBit; shift -= 2) RWKV_FULL_ROUND(shift)
+        bool listed = false;
+        while (shift >= 0) {                           // (uniform) shift = next undecided bit pair
+            if (tid == 0) s_cnt = 0;
+            __syncthreads();
 #pragma unroll
             for (int k = 0; k < PER; ++k) {
-                m1 += key[k] < c1 ? p[k] : 0.f;
-                m2 += key[k] < c2 ? p[k] : 0.f;
-                m3 += key[k] < c3 ? p[k] : 0.f;
+                const unsigned key = RWKV_KEY(k);
+                if (((key ^ prefix) >> (shift + 2)) == 0u) {
+                    const int at = atomicAdd(&s_cnt, 1);
+                    if (at < kSList) { list_key[at] = key; list_p[at] = p[k]; }
+                }
             }
-            // three sums with one pair of barriers
-            m1 = wave_sum(m1); m2 = wave_sum(m2); m3 = wave_sum(m3);
             __syncthreads();
-            if ((tid & 63) == 0) { scr[tid >> 6] = m1; scr[kST / 64 + (tid >> 6)] = m2; scr[2 * (kST / 64) + (tid >> 6)] = m3; }
-            __syncthreads();
-            float t1 = 0.f, t2 = 0.f, t3 = 0.f;
-#pragma unroll
-            for (int w = 0; w < kST / 64; ++w) { t1 += scr[w]; t2 += scr[kST / 64 + w]; t3 += scr[2 * (kST / 64) + w]; }
-            if (t3 < a.tau) prefix = c3; else if (t2 < a.tau) prefix = c2; else if (t1 < a.tau) prefix = c1;
+            if (s_cnt <= kSList) { listed = true; break; }
+            __syncthreads();                           // everybody has read the count before it is cleared again
+            RWKV_FULL_ROUND(shift)
+            shift -= 2;
+            if (shift >= 0) { RWKV_FULL_ROUND(shift) shift -= 2; }
         }
+        if (listed) {
+            const int n_list = s_cnt;
+            if (tid < 64) {
+                for (; shift >= 0; shift -= 2) {
+                    float m1 = 0.f, m2 = 0.f, m3 = 0.f;
+                    const unsigned c1 = prefix | (1u << shift), c2 = prefix | (2u << shift), c3 = prefix | (3u << shift);
+                    for (int i = tid; i < n_list; i += 64) {
+                        const unsigned key = list_key[i];
+                        const float pi = list_p[i];
+                        m1 += key < c1 ? pi : 0.f;
+                        m2 += key < c2 ? pi : 0.f;
+                        m3 += key < c3 ? pi : 0.f;
+                    }
+                    const float t1 = below + wave_sum(m1), t2 = below + wave_sum(m2), t3 = below + wave_sum(m3);
+                    if (t3 < a.tau) prefix = c3; else if (t2 < a.tau) prefix = c2; else if (t1 < a.tau) prefix = c1;
+                }
+                if (tid == 0) s_prefix = prefix;
+            }
+            __syncthreads();
+            prefix = s_prefix;
+        }
+#undef RWKV_FULL_ROUND
         // prefix = d* as bits (mass{key < d*} < tau <= mass{key <= d*}); if the whole mass stays below tau every
         // finite key passes.  Kept tokens, temperature, total.
         const float inv_t = a.temp != 1.0f ? 1.0f / a.temp : 1.0f;
         float q = 0.f;
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
-            float w = (key[k] <= prefix && p[k] > 0.f) ? p[k] : 0.f;
-            if (a.temp != 1.0f && w > 0.f) w = powf(w, inv_t);
+            float w = (RWKV_KEY(k) <= prefix && p[k] > 0.f) ? p[k] : 0.f;
+            if (a.temp != 1.0f && w > 0.f) w = __powf(w, inv_t);      // hardware log2 / exp2: a few ulp, immaterial for a sampling weight
             p[k] = w;
             q += w;
         }
-        // inverse CDF in token order: scan of the per-thread sums, then a walk inside one thread's tokens
+#undef RWKV_KEY
+        // inverse CDF in the order (thread, k): scan of the per-thread sums, then a walk inside one thread's tokens
         float own = q;
         float incl = own;
 #pragma unroll
@@ -158,11 +230,11 @@ sample_kernel(SampleArgs a) {
             int pick = -1;
 #pragma unroll
             for (int k = 0; k < PER; ++k) {
-                if (pick < 0 && p[k] > 0.f) { acc += p[k]; if (target < acc) pick = i0 + k; }
+                if (pick < 0 && p[k] > 0.f) { acc += p[k]; if (target < acc) pick = tid + kST * k; }
             }
             if (pick < 0) {                            // rounding at the upper edge: the thread's last kept token
 #pragma unroll
-                for (int k = 0; k < PER; ++k) if (p[k] > 0.f) pick = i0 + k;
+                for (int k = 0; k < PER; ++k) if (p[k] > 0.f) pick = tid + kST * k;
             }
             atomicMax(&s_tok, pick);
         }
@@ -171,7 +243,7 @@ sample_kernel(SampleArgs a) {
             // argmax over float32 logits kept in key order is gone; fall back on the first maximum of p
             float bp = -1.f; int bi = 0;
 #pragma unroll
-            for (int k = 0; k < PER; ++k) if (p[k] > bp) { bp = p[k]; bi = i0 + k; }
+            for (int k = 0; k < PER; ++k) if (p[k] > bp) { bp = p[k]; bi = tid + kST * k; }
 #pragma unroll
             for (int off = 32; off >= 1; off >>= 1) {
                 const float ob = __shfl_xor(bp, off, 64); const int oi = __shfl_xor(bi, off, 64);
@@ -201,8 +273,22 @@ sample_kernel(SampleArgs a) {
 
 int sample_launch(hipStream_t st, const SampleArgs &a) {
     if (a.V <= 0 || a.V > kST * kSMaxPer) return set_error(RWKV_ERR_SIZE, "sampler: vocabulary %d exceeds %d", a.V, kST * kSMaxPer);
-    if (a.V <= kST * 8) hipLaunchKernelGGL(sample_kernel<8>, dim3(1), dim3(kST), 0, st, a);
-    else hipLaunchKernelGGL(sample_kernel<kSMaxPer>, dim3(1), dim3(kST), 0, st, a);
+    constexpr size_t kSmall = (size_t)8 * kST * 4, kLarge = (size_t)kSKeysLds * kST * 4;
+    {   // the large variant's dynamic LDS exceeds the default limit: raised once per device
+        static std::mutex mu;
+        static bool configured[64] = {};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return set_error(RWKV_ERR_DEVICE, "sampler: no current device");
+        std::lock_guard<std::mutex> lock(mu);
+        if (!configured[dev]) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&sample_kernel<kSMaxPer>),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLarge);
+            if (e != hipSuccess) return set_error(RWKV_ERR_HIP, "sampler: %s", hipGetErrorString(e));
+            configured[dev] = true;
+        }
+    }
+    if (a.V <= kST * 8) hipLaunchKernelGGL(sample_kernel<8>, dim3(1), dim3(kST), kSmall, st, a);
+    else hipLaunchKernelGGL(sample_kernel<kSMaxPer>, dim3(1), dim3(kST), kLarge, st, a);
     RWKV_CHECK_LAUNCH("sample_kernel");
     return RWKV_OK;
 }

@@ -46,6 +46,34 @@ def test_typical_draws_follow_the_reference_distribution(V, temp, tau):
     assert chi < dof + 5.0 * (2 * dof) ** 0.5 + 10       # about five standard deviations
 
 
+@pytest.mark.parametrize("spread,tau", [(0.02, 0.5), (0.3, 0.8)])
+def test_typical_cut_on_a_nearly_flat_distribution(spread, tau):
+    """Logits of a random-init model: 50277 tokens of almost equal probability, so tens of thousands of distances
+    from the entropy share their leading bits (the search's list of undecided tokens overflows and it falls back to
+    more passes over all tokens).  Tokens are grouped by their rank in distance; the draws per group must follow
+    the oracle's kept mass per group - a cut too tight empties groups, one too wide fills groups that must stay empty."""
+    from rwkvstic_amd import ops
+    V, n, groups = 50277, 20000, 40
+    g = torch.Generator().manual_seed(int(spread * 1000))
+    logits = torch.randn(V, generator=g, dtype=torch.float64) * spread
+    want = O.typical_distribution(logits, 1.0, tau)
+    probs = torch.softmax(logits.float(), dim=-1)
+    s = -torch.log(probs)
+    d = (s - (s * probs).sum()).abs()
+    rank = torch.argsort(torch.argsort(d))
+    grp = (rank * groups // V).long()
+    got = _draws(ops, logits, n, temp=1.0, tau=tau, seed=99)
+    assert int((want[got] == 0).sum()) <= n * 2e-3
+    exp = torch.zeros(groups, dtype=torch.float64).index_add_(0, grp, want) * n
+    cnt = torch.bincount(grp[got], minlength=groups).double()
+    big = exp >= 5
+    chi = float((((cnt - exp) ** 2) / exp)[big].sum())
+    dof = int(big.sum()) - 1
+    print(f"spread={spread} tau={tau}: kept {int((want > 0).sum())} tokens, chi2 {chi:.1f} on {dof} dof", flush=True)
+    assert float(cnt[~big].sum()) <= n * 2e-3 + float(exp[~big].sum()) * 3 + 5
+    assert chi < dof + 5.0 * (2 * dof) ** 0.5 + 10
+
+
 def test_greedy_mode_end_adj_and_determinism():
     from rwkvstic_amd import ops
     g = torch.Generator().manual_seed(3)
