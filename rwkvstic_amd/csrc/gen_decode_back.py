@@ -69,12 +69,19 @@ class Emit:
         self.issued = 0
 
 
+S_TMP = 62        # scratch pair for a block's address where block offsets are added on the scalar side
+
+
 def gen(KW, R, NV, NSH):
     C = 512 * KW
     F = 4 * C
     PS, PSF = C + 64, F + 64
-    G = 32 * KW
-    NREAL = 13 * KW
+    NT = 2 if KW > 8 else 1          # groups of 16 channels (and their tiles) per workgroup
+    SPG = 5                          # parked-tile slots per group
+    NWG = 32 * KW // NT              # workgroups
+    SADDR = KW > 8                   # no room for one offset register per block of a job: the block offset joins the base address in a scalar pair
+    NJ = 13 * NT                     # jobs per layer
+    NREAL = NJ * KW
     PP = (NREAL + R - 1) // R * R
     RB = NV - 4 * R
     assert RB >= V_A + 4 * NA, "ring does not fit"
@@ -82,8 +89,45 @@ def gen(KW, R, NV, NSH):
     TB = 8 * KW * 1024
     DIG = max(12 * PS, 4 * PSF)
     RED = DIG                                 # byte offset of the parked tiles from the start of LDS
-    RED_SLOTS = max(5, 2 * NSH)
-    FLAG = RED + RED_SLOTS * 2048 + 32 * 8 + 32 * 8 + 2 * 4   # FLAG_ABORT word
+    RED_SLOTS = max(SPG * NT, 2 * NSH)
+    FLAG = RED + RED_SLOTS * 2048 + 32 * 8 + NT * 32 * 8 + 2 * 4   # FLAG_ABORT word
+
+    # Jobs of a layer in stream order.  ptr: index of the job's base address in the workgroup's table row (that of
+    # its first group; the same tile of the next group lies `stride` bytes further), aset/aoff: digit planes the
+    # A operand comes from, chain: jobs that add into one accumulator (the four quarters of an ffn value tile),
+    # slot: where the finished tile is parked.
+    jobs = []
+    for gi in range(NT):
+        for m in range(3):
+            jobs.append(dict(ph=0, gi=gi, ptr=m, stride=TB, aset="C", aoff=m * 4 * PS, first=True, park=gi * SPG + m))
+    for gi in range(NT):
+        jobs.append(dict(ph=1, gi=gi, ptr=3, stride=TB, aset="C", aoff=0, first=True, park=gi * SPG))
+    for gi in range(NT):
+        jobs.append(dict(ph=2, gi=gi, ptr=4, stride=TB, aset="C", aoff=4 * PS, first=True, park=gi * SPG))
+        for r in range(4):
+            jobs.append(dict(ph=2, gi=gi, ptr=5 + r, stride=TB, aset="C", aoff=0, first=True, park=gi * SPG + 1 + r))
+    for gi in range(NT):
+        for q in range(4):
+            jobs.append(dict(ph=3, gi=gi, ptr=9 + q, stride=4 * TB, aset="F", aoff=q * C, first=q == 0, park=gi * SPG if q == 3 else None))
+    assert len(jobs) == NJ
+    # accumulators alternate from one chain to the next, so that a parked tile is still being written while the next one starts
+    acc_of, chain = [], -1
+    for jb in jobs:
+        if jb["first"]:
+            chain += 1
+        acc_of.append(chain % 2)
+
+    def block_load(dst, sbase, extra, b, wh=False):
+        """16-byte-per-lane load of block b of a job whose base address is in s[sbase:sbase+1] (+ extra bytes)."""
+        if wh:
+            e(f"global_load_dwordx4 {dst}, v{V_OFF}, %[wh]")
+        elif SADDR:
+            e(f"s_add_u32 s{S_TMP}, s{sbase}, {extra + 8192 * b}")
+            e(f"s_addc_u32 s{S_TMP + 1}, s{sbase + 1}, 0")
+            e(f"global_load_dwordx4 {dst}, v{V_OFF}, s[{S_TMP}:{S_TMP + 1}]")
+        else:
+            assert extra == 0
+            e(f"global_load_dwordx4 {dst}, v{V_OFF + b}, s[{sbase}:{sbase + 1}]")
     LH = R * KW // math.gcd(R, KW)
     e = Emit()
 
@@ -101,16 +145,7 @@ def gen(KW, R, NV, NSH):
         else:
             q = q_layer_pos
             j, b = divmod(q, KW)
-            if j <= 2:
-                base, off = V_APC, j * 4 * PS + 512 * b
-            elif j == 3:
-                base, off = V_APC, 512 * b
-            elif j == 4:
-                base, off = V_APC, 4 * PS + 512 * b
-            elif j <= 8:
-                base, off = V_APC, 512 * b
-            else:
-                base, off = V_APF, (j - 9) * C + 512 * b
+            base, off = (V_APC if jobs[j]["aset"] == "C" else V_APF), jobs[j]["aoff"] + 512 * b
             k = q % NA
         assert off < 65536
         e(f"ds_read_b128 v[{V_A + 4 * k}:{V_A + 4 * k + 3}], v{base} offset:{off}")
@@ -159,8 +194,9 @@ def gen(KW, R, NV, NSH):
     e(f"s_lshl_b32 s{S_T}, %[wb], 10")
     e(f"v_lshlrev_b32 v{V_OFF}, 4, v{V_A}")
     e(f"v_add_u32 v{V_OFF}, s{S_T}, v{V_OFF}")
-    for b in range(1, KW):
-        e(f"v_add_u32 v{V_OFF + b}, {8192 * b}, v{V_OFF}")
+    if not SADDR:
+        for b in range(1, KW):
+            e(f"v_add_u32 v{V_OFF + b}, {8192 * b}, v{V_OFF}")
     e(f"s_mov_b64 s[{S_JT}:{S_JT + 1}], %[jt]")
     e(f"s_mov_b32 s{S_L}, %[L]")
     e(f"s_mov_b32 s{S_SEQ}, 0")
@@ -173,7 +209,8 @@ def gen(KW, R, NV, NSH):
     # the statistics barrier (att output -> ffn key/receptance; ffn value -> next layer / head).  What the ffn value
     # phase carries over is issued at the top of the next layer, after that layer's first barrier - also in the
     # first layer, which is why the prologue leaves those positions out.
-    phases = [(0, 3 * KW, 2), (3 * KW, 4 * KW, 1), (4 * KW, 9 * KW, 2), (9 * KW, 13 * KW, 1)]   # start, end, barriers before
+    NB = NT * KW
+    phases = [(0, 3 * NB, 2), (3 * NB, 4 * NB, 1), (4 * NB, 9 * NB, 2), (9 * NB, 13 * NB, 1)]   # start, end, barriers before
     def deferred_of(ph):
         ps, pe, _ = phases[ph]
         d = [p for p in range(ps, pe) if not (p + R < pe and DEFER) and DEFER]
@@ -187,7 +224,7 @@ def gen(KW, R, NV, NSH):
         if p in skip:
             continue
         j, b = divmod(p, KW)
-        e(f"global_load_dwordx4 {ring(p)}, v{V_OFF + b}, s[{S_CUR + 2 * j}:{S_CUR + 2 * j + 1}]")
+        block_load(ring(p), S_CUR + 2 * jobs[j]["ptr"], jobs[j]["gi"] * jobs[j]["stride"], b)
 
     # ------------------------------------------------------------------ layers
     # Loads are issued in position order; position q's load is the q-th load of the wave.  A slot
@@ -213,10 +250,10 @@ def gen(KW, R, NV, NSH):
         else:
             assert not top
         if q >= NREAL:
-            e(f"global_load_dwordx4 {ring(slot)}, v{V_OFF}, %[wh]")
+            block_load(ring(slot), 0, 0, 0, wh=True)
         else:
             jq, bq = divmod(q, KW)
-            e(f"global_load_dwordx4 {ring(slot)}, v{V_OFF + bq}, s[{sset + 2 * jq}:{sset + 2 * jq + 1}]")
+            block_load(ring(slot), sset + 2 * jobs[jq]["ptr"], jobs[jq]["gi"] * jobs[jq]["stride"], bq)
 
     e("1:")
     carry = []
@@ -241,8 +278,8 @@ def gen(KW, R, NV, NSH):
             nvm = issued_loads - 1 - p
             assert 0 <= nvm <= 63, (KW, R, p, nvm)
             e(f"s_waitcnt vmcnt({nvm}) lgkmcnt({allow})")
-            dreg = V_D + 4 * (1 if j >= 9 else j % 2)
-            first = (b == 0) and not (j > 9)
+            dreg = V_D + 4 * acc_of[j]
+            first = (b == 0) and jobs[j]["first"]
             acc = "0" if first else f"v[{dreg}:{dreg + 3}]"
             e(f"v_mfma_i32_16x16x64_i8 v[{dreg}:{dreg + 3}], {abuf(p)}, {ring(p % R)}, {acc}")
             if p + R < pe or not DEFER:
@@ -251,9 +288,8 @@ def gen(KW, R, NV, NSH):
                 issued_loads += 1
             else:
                 deferred.append(p)
-            if b == KW - 1 and (j < 9 or j == 12):
-                pslot = j if j <= 2 else (0 if j == 3 else (j - 4 if j <= 8 else 0))
-                park_static(dreg, pslot)
+            if b == KW - 1 and jobs[j]["park"] is not None:
+                park_static(dreg, jobs[j]["park"])
         e("s_waitcnt lgkmcnt(0)")
         e("s_barrier")
         e.drain_state()
@@ -309,7 +345,7 @@ def gen(KW, R, NV, NSH):
     # LH = lcm(R, KW) positions (a whole number of rounds), after which slots and blocks line up again.
     def head_ptr():
         """s[S_RP] = address of head tile g + G * s[S_RT], or of tile 0 when that is past the end."""
-        e(f"s_mul_i32 vcc_lo, s{S_RT}, {G}")
+        e(f"s_mul_i32 vcc_lo, s{S_RT}, {NWG}")
         e(f"s_add_u32 vcc_lo, vcc_lo, %[g]")
         e(f"s_cmp_ge_u32 vcc_lo, %[vt]")
         e(f"s_cselect_b32 vcc_lo, 0, vcc_lo")
@@ -325,7 +361,7 @@ def gen(KW, R, NV, NSH):
         if rb == 0:
             e(f"s_add_u32 s{S_RT}, s{S_RT}, 1")
             head_ptr()
-        e(f"global_load_dwordx4 {ring(q % R)}, v{V_OFF + rb}, s[{S_RP}:{S_RP + 1}]")
+        block_load(ring(q % R), S_RP, 0, rb)
 
     tiles_per_body = LH // KW
     assert tiles_per_body % NSH == 0
@@ -401,7 +437,7 @@ def gen(KW, R, NV, NSH):
 # (KW, front waves, ring size): 4 front waves -> 12 waves per workgroup, 168 VGPRs each;
 # 8 front waves -> 16 waves, 128 VGPRs each.
 CONFIGS = [(2, 4, 26), (4, 4, 26), (5, 4, 33), (8, 4, 26),
-           (2, 8, 13), (4, 8, 13), (5, 8, 22), (8, 8, 13)]
+           (2, 8, 13), (4, 8, 13), (5, 8, 22), (8, 8, 13), (10, 8, 20)]
 
 
 def main():

@@ -46,7 +46,8 @@ struct DScal {
 static_assert(sizeof(DScal) == 128, "DScal is read as a 128-byte record");
 
 struct DModel {
-    int L, C, F, V, G;
+    int L, C, F, V, G;           // G = C / 16 groups of 16 channels
+    int NWG;                     // workgroups of the single-token kernel: G, or G / 2 where a workgroup owns two groups (C = 5120)
     const float *emb;
     const double *ln0_w, *ln0_b;
     const uint8_t *w_head;
@@ -56,7 +57,7 @@ struct DModel {
     // the order att k, v, r, o, ffn r [C each], ffn k [F], ffn v [C]; cs_head [round_up(V, 16)].
     const int *cs;
     const int *cs_head;
-    const u64 *jt;               // [G][L+1][16] job base addresses per workgroup (row L: first head tiles)
+    const u64 *jt;               // [NWG][L+1][16] job base addresses per workgroup, of its first group (row L: first head tiles)
     const u64 *ownrec;           // [L][G][512] per-layer constants of each workgroup's own channels
     // With xy = ln(x), mixed = xy mu + shift (1 - mu) and t = (x - mean) rsd:
     //   fp32(mixed range)          = fp32(t P + Q),  P = ln_w mu range,  Q = (ln_b mu + shift (1 - mu)) range
@@ -66,7 +67,7 @@ struct DModel {
     double *PO;                  // [L+1][5][C]
     DScal *sc;                   // [L+1]
     DScal *scp;                  // [L][C/512] per-token scalars (sumQO, maxQ) of each 512-channel part of a layer
-    double *amax_val;            // [G] device-side argmax: first maximum of the logits each workgroup wrote, and its index
+    double *amax_val;            // [NWG] device-side argmax: first maximum of the logits each workgroup wrote, and its index
     int *amax_idx;
     double *X0;                  // [C] ln0(emb[token]) of the launch in flight
 };
@@ -75,13 +76,13 @@ struct DModel {
 // the first launch; they belong to one model handle (one token step in flight at a time).
 struct DecodeBuffers {
     u64 *X;                 // [C]       residual stream
-    u64 *XR;                // [13][G]   per workgroup: sum x (hi, lo), sum x^2 (hi, lo), then per matrix max |x P|, sum x PO (hi, lo)
+    u64 *XR;                // [11][G]   per group of 16 channels: sum x, squared deviations from the group's mean, then per matrix max |x P|, sum x PO (hi, lo)
     u64 *A;                 // [C]       fp32(wkv * sigmoid(r) * range_o)
     u64 *AR;                // [3][G]    per workgroup: max |A|, zero-point share (hi, lo)
     u64 *H;                 // [F]       fp32(relu(k)^2 * range_v)
     u64 *HR;                // [3][G]
     unsigned *abort_flag;   // set to 1 by any workgroup whose wait ran out
-    long long *trace;       // optional: [G][L][24] 100 MHz timestamps of every workgroup's phase boundaries (null = off)
+    long long *trace;       // optional: [NWG][L][24] 100 MHz timestamps of every workgroup's phase boundaries (null = off)
 };
 
 // Host-side description from which the tables are built.
@@ -98,6 +99,7 @@ struct DSetup {
 };
 
 bool decode_supported(int64_t L, int64_t C, int64_t F, int64_t V);
+int64_t decode_workgroups(int64_t C);          // grid of the single-token kernel (C / 16, or C / 32 where a workgroup owns two groups)
 unsigned decode_epochs_per_token(int64_t L);
 constexpr int kTraceStampsPerLayer = 24;
 

@@ -66,6 +66,7 @@ constexpr int kLnRows = kStatRows + 3 * 3;     // rows of the XR record table
 #define RWKV_EARLY_DIV 4
 #endif
 constexpr int kEarlyDiv = RWKV_EARLY_DIV;           // gathers start when all but G / kEarlyDiv workgroups have published (measured flat from G/20 to G)
+constexpr int kSlotsPerGroup = 5;      // parked-tile slots a group of 16 channels needs at once (ffn receptance + 4 ffn key tiles)
 constexpr int kHeadCsPerThread = 4;    // head column sums a front thread fetches: 16 per head tile of the workgroup
 
 // LDS flag words
@@ -88,6 +89,13 @@ __device__ __forceinline__ void gst(T *p, T v) { *(RWKV_GLOBAL T *)p = v; }
 #define ASTORE(p, v) __hip_atomic_store((RWKV_GLOBAL u64 *)(p), (u64)(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
 #define ALOAD32(p) __hip_atomic_load((RWKV_GLOBAL unsigned *)(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
 #define ASTORE32(p, v) __hip_atomic_store((RWKV_GLOBAL unsigned *)(p), (unsigned)(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+
+// A workgroup owns NT groups of 16 channels (and their tiles): one up to C = 4096, two at C = 5120, whose 320
+// groups would not all be resident on 256 compute units.  Wave gi < NT of the front waves finishes group NT w + gi.
+template <int KW>
+struct GroupShape {
+    static constexpr int NT = KW > 8 ? 2 : 1, G = 32 * KW, NWG = G / NT;
+};
 
 struct DArgs {
     DModel m;
@@ -463,8 +471,7 @@ __device__ __forceinline__ float or_maxQ(const u64 *rec, int m) { return reinter
 
 // l == L stages the head's scalars only.
 template <int FT, int PARTS>
-__device__ __forceinline__ void stage_owner_record(const DArgs &a, int l, int g, int G, int C, u64 *own_lds, int tid) {
-    u64 *dst = own_lds + (l & 1) * kOrSlots;
+__device__ __forceinline__ void stage_owner_record(const DArgs &a, int l, int g, int G, int C, u64 *dst, int tid) {
     const bool layer = l < a.m.L;
 #pragma unroll
     for (int i = 0; i < kOrSlots / FT; ++i) {
@@ -660,14 +667,19 @@ __device__ __forceinline__ void vec_front(Front &fx, int &seq, const u64 *src, c
 template <int KW, int FW, bool TRACE>
 __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, const v4i *red, double *stat, double *rf_lds,
                                            lds_flag_t *flags, u64 *own_lds, double *st_lds, long long *trace_lds) {
-    constexpr int C = 512 * KW, F = 4 * C, G = 32 * KW, FT = 64 * FW;
+    constexpr int C = 512 * KW, F = 4 * C, G = GroupShape<KW>::G, NT = GroupShape<KW>::NT, NWG = GroupShape<KW>::NWG, FT = 64 * FW;
     constexpr int PS = C + 64, PSF = F + 64;
     constexpr int NQH = F / 4, NQTH = (NQH + FT - 1) / FT, NQC = C / 4, NQTC = (NQC + FT - 1) / FT;
+    static_assert(FW >= NT, "one finishing wave per group");
     Front fx;
     fx.abort_flag = a.b.abort_flag; fx.flags = flags; fx.ok = true;
     fx.refresh();
-    const int g = blockIdx.x, L = a.m.L, V = a.m.V;
-    const bool fin = fx.wave == 0;                       // wave 0 owns the workgroup's 16 channels
+    const int wg = blockIdx.x, L = a.m.L, V = a.m.V;
+    const bool fin = fx.wave < NT;                       // wave gi finishes the workgroup's group gi of 16 channels
+    const int gi = fin ? fx.wave : 0;
+    const int g = NT * wg + gi;
+    red += gi * kSlotsPerGroup * kBW * 16;               // the group's parked tiles
+    rf_lds += gi * 32;
     // stamps are collected in LDS and copied out after the head: a store to memory here would queue behind the weight stream
     long long *trace = TRACE ? trace_lds : nullptr;     // uniform; thread 0 stamps
     int seq = 0;
@@ -675,17 +687,22 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
 #define RWKV_IDS() do { fx.refresh(); lane = fx.lane; n = lane & 15; row = lane >> 4; c_own = 16 * g + n; } while (0)
     RWKV_IDS();
 
-    stage_owner_record<FT, KW>(a, 0, g, G, C, own_lds, fx.tid);   // read after the first barriers below
+#pragma unroll
+    for (int t = 0; t < NT; ++t) stage_owner_record<FT, KW>(a, 0, NT * wg + t, G, C, own_lds + (2 * t) * kOrSlots, fx.tid);   // read after the first barriers below
     // the residual value of the own channels lives in LDS between the epilogues (rf_lds[16 + n])
     double *x_lds = rf_lds + 16;
     if (fin && row == 0) x_lds[n] = a.m.X0[c_own];
 
     for (int l = 0; l < L && fx.ok; ++l) {
-        const u64 *rec = own_lds + (l & 1) * kOrSlots;
+        const u64 *rec = own_lds + (2 * gi + (l & 1)) * kOrSlots;     // (waves that finish nothing read the layer's scalars from group 0's)
         // New state rows of the own channels are collected in LDS and written out once, after the
         // head: nobody else reads them during this token, and a store issued here would queue in
         // the compute unit's memory pipeline behind the weight stream, in front of the exchange.
-        double *sl = st_lds + (size_t)l * 5 * 16;
+        // With two groups per workgroup LDS has no room for that: the rows go straight to memory.
+        auto put_state = [&](int r, int nn, double v) {
+            if constexpr (NT == 1) st_lds[((size_t)l * 5 + r) * 16 + nn] = v;
+            else gst(a.state + ((size_t)l * 5 + r) * C + 16 * g + nn, v);
+        };
         const unsigned e = a.epoch0 + 4u * (unsigned)l;
         long long *tr = trace ? trace + (size_t)l * kTraceStampsPerLayer : nullptr;
         const float *P32 = a.m.P32 + (size_t)l * kLnMats * C, *Q32 = a.m.Q32 + (size_t)l * kLnMats * C;
@@ -696,7 +713,7 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
         if (!fx.ok) break;
         RWKV_IDS();
         // while the matrix cores run: the LayerNorm output of the own channel is the new att shift state (block.py:58,63-64)
-        if (fin && row == 0) sl[n] = or_d(rec, OR_LN1W * 16 + n) * ((x_lds[n] - stat[0]) * stat[1]) + or_d(rec, OR_LN1B * 16 + n);
+        if (fin && row == 0) put_state(0, n, or_d(rec, OR_LN1W * 16 + n) * ((x_lds[n] - stat[0]) * stat[1]) + or_d(rec, OR_LN1B * 16 + n));
         __syncthreads();                                                         // tile sums parked
         if (tr && fx.tid == 0) tr[3] = wall_clock64();
         if (fin) {
@@ -721,9 +738,9 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
                 if (row == 1) { dst = a.b.AR + (size_t)n * G + g; val = n == 0 ? mx : (n == 1 ? hi : lo); }
                 if (row == 0 || (row == 1 && n < 3)) put_word(dst, e + 1u, val);
                 if (row == 0) {
-                    sl[2 * 16 + n] = (double)aa;
-                    sl[3 * 16 + n] = (double)bb;
-                    sl[4 * 16 + n] = pp;
+                    put_state(2, n, (double)aa);
+                    put_state(3, n, (double)bb);
+                    put_state(4, n, pp);
                 }
             }
         }
@@ -733,7 +750,9 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
         // The next layer's owner record (l + 1 == L: the head's scalars) is fetched here, where every wave
         // is about to wait for the other workgroups anyway: the copy to LDS has to wait for the loads.
         RWKV_IDS();
-        stage_owner_record<FT, KW>(a, l + 1, g, G, C, own_lds, fx.tid);
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+            stage_owner_record<FT, KW>(a, l + 1, NT * wg + t, G, C, own_lds + (2 * t + ((l + 1) & 1)) * kOrSlots, fx.tid);
         vec_front<KW, FW, NQTC>(fx, seq, a.b.A, a.b.AR, NQC, e + 1u, dig, PS, stat, tr ? tr + 5 : nullptr, tr ? tr + 17 : nullptr);
         if (!fx.ok) break;
         __syncthreads();
@@ -756,7 +775,7 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
         if (!fx.ok) break;
         RWKV_IDS();
         // the LayerNorm output of the own channel is the new ffn shift state (block.py:82,87-88)
-        if (fin && row == 0) sl[16 + n] = or_d(rec, OR_LN2W * 16 + n) * ((x_lds[n] - stat[0]) * stat[1]) + or_d(rec, OR_LN2B * 16 + n);
+        if (fin && row == 0) put_state(1, n, or_d(rec, OR_LN2W * 16 + n) * ((x_lds[n] - stat[0]) * stat[1]) + or_d(rec, OR_LN2B * 16 + n));
         __syncthreads();
         if (tr && fx.tid == 0) tr[11] = wall_clock64();
         if (fin) {
@@ -799,7 +818,8 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
     }
 
     // ========================= head (opt.py:71-73) ==============================
-    const int v_tiles = (V + 15) / 16, head_rounds = (v_tiles + G - 1) / G;
+    const int v_tiles = (V + 15) / 16, head_rounds = (v_tiles + NWG - 1) / NWG;
+    red -= gi * kSlotsPerGroup * kBW * 16;                 // the head's parked tiles belong to the workgroup
     const u64 *rec_h = own_lds + (L & 1) * kOrSlots;
     // column sums of the workgroup's head tiles: requested now, parked in the LDS half that held the
     // last layer's record once the wait for x is over (a load inside the loop below would cost a
@@ -808,7 +828,7 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
     int csv[kHeadCsPerThread];
 #pragma unroll
     for (int k = 0; k < kHeadCsPerThread; ++k) {
-        const int i = fx.tid + FT * k, v = 16 * (g + G * (i >> 4)) + (i & 15);
+        const int i = fx.tid + FT * k, v = 16 * (wg + NWG * (i >> 4)) + (i & 15);
         csv[k] = (i < head_rounds * 16 && v < V) ? a.m.cs_head[v] : 0;
     }
     if (fx.ok)
@@ -832,7 +852,7 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
         __syncthreads();                                   // (the first one also orders the csh writes above)
         const int s = fx.tid >> 4;                         // parked tile of this round
         if (s < NS && h0 + s < head_rounds) {
-            const int v = 16 * (g + G * (h0 + s)) + n;
+            const int v = 16 * (wg + NWG * (h0 + s)) + n;
             if (v < V) {
                 const double y = finish_col(red + par * (NS * kBW * 16), s, n, Sh, csh[16 * (h0 + s) + n], zph);
                 a.logits[v] = y;
@@ -848,31 +868,33 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
             const int oi = __shfl_xor(best_i, off, 64);
             if (ob > best || (ob == best && oi < best_i)) { best = ob; best_i = oi; }
         }
-        if (fx.lane == 0) { a.m.amax_val[g] = best; a.m.amax_idx[g] = best_i; }
+        if (fx.lane == 0) { a.m.amax_val[wg] = best; a.m.amax_idx[wg] = best_i; }
     }
     // the state rows of the own channels: st_lds[l][row][n] -> state[l][row][16 g + n]
-    for (int i = fx.tid; i < L * 5 * 16; i += FT) a.state[(size_t)(i >> 4) * C + 16 * g + (i & 15)] = st_lds[i];
+    if constexpr (NT == 1)
+        for (int i = fx.tid; i < L * 5 * 16; i += FT) a.state[(size_t)(i >> 4) * C + 16 * wg + (i & 15)] = st_lds[i];
     if (TRACE)
-        for (int i = fx.tid; i < L * kTraceStampsPerLayer; i += FT) a.b.trace[(size_t)g * L * kTraceStampsPerLayer + i] = trace_lds[i];
+        for (int i = fx.tid; i < L * kTraceStampsPerLayer; i += FT) a.b.trace[(size_t)wg * L * kTraceStampsPerLayer + i] = trace_lds[i];
 }
 
 template <int KW, int FW>
 struct DecodeLds {
-    static constexpr int C = 512 * KW, F = 4 * C;
+    static constexpr int C = 512 * KW, F = 4 * C, NT = GroupShape<KW>::NT;
     static constexpr int PS = C + 64, PSF = F + 64;
     static constexpr int DIG_BYTES = (3 * 4 * PS > 4 * PSF) ? 3 * 4 * PS : 4 * PSF;
     static constexpr int RED_SLOTS = BackCfg<KW, FW>::RED_SLOTS;
     static constexpr int RED_BYTES = RED_SLOTS * kBW * 16 * 16;
-    static constexpr int STAT_BYTES = 32 * 8, RF_BYTES = 32 * 8, FLAG_BYTES = FLAG_COUNT * 4;   // RF: gate and residual of the own channels
+    static constexpr int STAT_BYTES = 32 * 8, RF_BYTES = NT * 32 * 8, FLAG_BYTES = FLAG_COUNT * 4;   // RF: gate and residual of the own channels
     static constexpr int OWN_OFFSET = DIG_BYTES + RED_BYTES + STAT_BYTES + RF_BYTES + FLAG_BYTES;
-    static constexpr int STATE_OFFSET = OWN_OFFSET + 2 * kOrSlots * 8;
-    static __host__ __device__ int total(int L, bool trace = false) {                           // + the new state rows of the own channels (+ the stamps)
-        return STATE_OFFSET + L * 5 * 16 * 8 + (trace ? L * kTraceStampsPerLayer * 8 : 0);
+    static constexpr int STATE_OFFSET = OWN_OFFSET + NT * 2 * kOrSlots * 8;
+    static __host__ __device__ int state_bytes(int L) { return NT == 1 ? L * 5 * 16 * 8 : 0; }  // the new state rows of the own channels
+    static __host__ __device__ int total(int L, bool trace = false) {                           // (+ the stamps)
+        return STATE_OFFSET + state_bytes(L) + (trace ? L * kTraceStampsPerLayer * 8 : 0);
     }
     // the generated back-wave program addresses LDS by these offsets
     static_assert(BackCfg<KW, FW>::RED == DIG_BYTES, "parked tiles follow the digit planes");
     static_assert(BackCfg<KW, FW>::FLAG == DIG_BYTES + RED_BYTES + STAT_BYTES + RF_BYTES + FLAG_ABORT * 4, "abort flag offset");
-    static_assert(RED_SLOTS >= 5 && RED_SLOTS >= 2 * BackCfg<KW, FW>::NS, "park slots");
+    static_assert(RED_SLOTS >= kSlotsPerGroup * NT && RED_SLOTS >= 2 * BackCfg<KW, FW>::NS, "park slots");
 };
 
 template <int KW, int FW, bool TRACE>
@@ -883,7 +905,7 @@ __global__ void __launch_bounds__((FW + kBW) * 64) decode_kernel(const DArgs a) 
     v4i *red = reinterpret_cast<v4i *>(smem + Lds::DIG_BYTES);
     double *stat = reinterpret_cast<double *>(smem + Lds::DIG_BYTES + Lds::RED_BYTES);
     double *rf_lds = stat + 32;
-    lds_flag_t *flags = (lds_flag_t *)(rf_lds + 32);
+    lds_flag_t *flags = (lds_flag_t *)(rf_lds + 32 * Lds::NT);
     if (a.stop && gld(a.stop) != 0) return;          // written before this launch started: every workgroup reads the same value
     if (threadIdx.x < FLAG_COUNT) flags[threadIdx.x] = 0;
     __syncthreads();
@@ -891,10 +913,10 @@ __global__ void __launch_bounds__((FW + kBW) * 64) decode_kernel(const DArgs a) 
     if (wave < FW) {
         front_path<KW, FW, TRACE>(a, dig, red, stat, rf_lds, flags, reinterpret_cast<u64 *>(smem + Lds::OWN_OFFSET),
                                   reinterpret_cast<double *>(smem + Lds::STATE_OFFSET),
-                                  reinterpret_cast<long long *>(smem + Lds::total(a.m.L)));
+                                  reinterpret_cast<long long *>(smem + Lds::total(a.m.L)));       // (total without the stamps = where they start)
     } else {
-        constexpr int G = 32 * KW;
-        const int v_tiles = (a.m.V + 15) / 16, head_rounds = (v_tiles + G - 1) / G;
+        constexpr int NWG = GroupShape<KW>::NWG;
+        const int v_tiles = (a.m.V + 15) / 16, head_rounds = (v_tiles + NWG - 1) / NWG;
         const unsigned lds = (unsigned)(uintptr_t)(RWKV_LDS unsigned char *)smem;
         BackCfg<KW, FW>::run(a.m.jt + (size_t)blockIdx.x * (a.m.L + 1) * 16, a.m.w_head, a.m.L, head_rounds, v_tiles,
                          (int)blockIdx.x, wave - FW, lds);
@@ -1027,7 +1049,7 @@ __global__ void __launch_bounds__(kPrepThreads) next_token_kernel(const DArgs a,
     auto better = [](double v, int i, double bv, int bi) { return v > bv || (v == bv && i < bi); };
     double best = -INFINITY;
     int bi = 0x7fffffff;
-    if ((int)threadIdx.x < a.m.G) { best = a.m.amax_val[threadIdx.x]; bi = a.m.amax_idx[threadIdx.x]; }   // G <= 256
+    if ((int)threadIdx.x < a.m.NWG) { best = a.m.amax_val[threadIdx.x]; bi = a.m.amax_idx[threadIdx.x]; }   // NWG <= 256
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) {
         const double ob = __shfl_xor(best, off, 64);
@@ -1116,9 +1138,9 @@ __global__ void __launch_bounds__(kOrSlots) build_ownrec_kernel(const DPrep *__r
 // jt[g][l][16]: base address of job j of layer l for workgroup g (13 used); row L: the first head
 // tiles of the workgroup (tiles past the end of the vocabulary point at tile 0, whose blocks stay
 // hot in L2 and whose products are never used).  grid (G), any block size.
-__global__ void build_jobtab_kernel(const DLayer *__restrict__ layers, const uint8_t *w_head, int L, int G, int n_kb,
+__global__ void build_jobtab_kernel(const DLayer *__restrict__ layers, const uint8_t *w_head, int L, int G, int NWG, int n_kb,
                                     int v_tiles, u64 *__restrict__ jt) {
-    const int g = blockIdx.x;
+    const int wg = blockIdx.x, g = (G / NWG) * wg;     // the workgroup's first group; the tiles of its next group follow at fixed strides
     const size_t TB = (size_t)n_kb * 1024;
     for (int i = threadIdx.x; i < (L + 1) * 16; i += blockDim.x) {
         const int l = i >> 4, j = i & 15;
@@ -1131,7 +1153,7 @@ __global__ void build_jobtab_kernel(const DLayer *__restrict__ layers, const uin
             else if (j <= 8) p = Ly.w[MAT_FFN_K] + (size_t)(g + G * (j - 5)) * TB;
             else p = Ly.w[MAT_FFN_V] + ((size_t)g * 4 + (j - 9)) * TB;
         } else if (l == L) {
-            const int tile = g + G * j;
+            const int tile = wg + NWG * j;
             p = w_head + (size_t)(tile < v_tiles ? tile : 0) * TB;
         }
 #ifdef RWKV_DIAG_HOT_WEIGHTS
@@ -1139,7 +1161,7 @@ __global__ void build_jobtab_kernel(const DLayer *__restrict__ layers, const uin
         // takes HBM out of the picture and leaves the time of the dependency chain between the workgroups.
         p = w_head;
 #endif
-        jt[(size_t)g * (L + 1) * 16 + i] = (u64) reinterpret_cast<uintptr_t>(p);
+        jt[(size_t)wg * (L + 1) * 16 + i] = (u64) reinterpret_cast<uintptr_t>(p);
     }
 }
 
@@ -1207,11 +1229,13 @@ __global__ void __launch_bounds__(kPrepThreads) build_consts_kernel(const ConstA
 bool decode_supported(int64_t L, int64_t C, int64_t F, int64_t V) {
     if (L <= 0 || V <= 0 || F != 4 * C) return false;
     // one 16-column tile per workgroup, all workgroups resident: C/16 <= 256 CUs
-    if (!(C == 1024 || C == 2048 || C == 2560 || C == 4096)) return false;
+    if (!(C == 1024 || C == 2048 || C == 2560 || C == 4096 || C == 5120)) return false;
     // the column sums of a workgroup's head tiles are staged by its front threads into half an owner record
-    const int64_t G = C / 16, head_rounds = ((V + 15) / 16 + G - 1) / G, front_threads = C == 2560 ? 512 : 256;
+    const int64_t NWG = decode_workgroups(C), head_rounds = ((V + 15) / 16 + NWG - 1) / NWG, front_threads = (C == 2560 || C == 5120) ? 512 : 256;
     return head_rounds * 16 <= kHeadCsPerThread * front_threads && head_rounds * 16 * (int64_t)sizeof(int) <= kOrSlots * 8;
 }
+
+int64_t decode_workgroups(int64_t C) { return C > 4096 ? C / 32 : C / 16; }
 
 unsigned decode_epochs_per_token(int64_t L) { return (unsigned)(4 * L + 1); }
 
@@ -1292,7 +1316,7 @@ int decode_setup(void *block, void *exchange, const DSetup &s, DModel *dm, Decod
     RWKV_CHECK_HIP(hipMemcpy(base + p.layers, tab.data(), (size_t)L * sizeof(DLayer), hipMemcpyHostToDevice));
     RWKV_CHECK_HIP(hipMemcpy(base + p.prep, prep.data(), (size_t)L * sizeof(DPrep), hipMemcpyHostToDevice));
 
-    dm->L = (int)L; dm->C = (int)C; dm->F = (int)F; dm->V = (int)V; dm->G = (int)G;
+    dm->L = (int)L; dm->C = (int)C; dm->F = (int)F; dm->V = (int)V; dm->G = (int)G; dm->NWG = (int)decode_workgroups(C);
     dm->emb = s.emb; dm->ln0_w = s.ln0_w; dm->ln0_b = s.ln0_b;
     dm->w_head = s.head.w16; dm->cs = cs; dm->cs_head = cs_head;
     dm->ownrec = reinterpret_cast<const u64 *>(base + p.ownrec);
@@ -1309,8 +1333,8 @@ int decode_setup(void *block, void *exchange, const DSetup &s, DModel *dm, Decod
 
     ConstArgs ca;
     dm->jt = reinterpret_cast<const u64 *>(base + p.jt);
-    hipLaunchKernelGGL(build_jobtab_kernel, dim3((unsigned)G), dim3(256), 0, nullptr, dm->layers, s.head.w16, (int)L,
-                       (int)G, c_kb, (int)ceil_div(V, 16), reinterpret_cast<u64 *>(base + p.jt));
+    hipLaunchKernelGGL(build_jobtab_kernel, dim3((unsigned)dm->NWG), dim3(256), 0, nullptr, dm->layers, s.head.w16, (int)L,
+                       (int)G, dm->NWG, c_kb, (int)ceil_div(V, 16), reinterpret_cast<u64 *>(base + p.jt));
     RWKV_CHECK_LAUNCH("build_jobtab_kernel");
     ca.L = (int)L; ca.C = (int)C; ca.prep = dm->prep;
     ca.lnout_w = s.lnout_w; ca.lnout_b = s.lnout_b; ca.range_h = s.head.range; ca.offset_h = s.head.offset;
@@ -1372,9 +1396,9 @@ static int launch_one(hipStream_t st, const DArgs &args, bool with_prep) {
         RWKV_CHECK_LAUNCH("prep_kernel");
     }
     if (trace)
-        hipLaunchKernelGGL((decode_kernel<KW, FW, true>), dim3((unsigned)args.m.G), dim3((FW + kBW) * 64), lds, st, args);
+        hipLaunchKernelGGL((decode_kernel<KW, FW, true>), dim3((unsigned)args.m.NWG), dim3((FW + kBW) * 64), lds, st, args);
     else
-        hipLaunchKernelGGL((decode_kernel<KW, FW, false>), dim3((unsigned)args.m.G), dim3((FW + kBW) * 64), lds, st, args);
+        hipLaunchKernelGGL((decode_kernel<KW, FW, false>), dim3((unsigned)args.m.NWG), dim3((FW + kBW) * 64), lds, st, args);
     RWKV_CHECK_LAUNCH("decode_kernel");
     return RWKV_OK;
 }
@@ -1385,6 +1409,7 @@ static int launch_step(hipStream_t st, const DArgs &args, bool with_prep) {
         case 2048: return launch_one<4, 4>(st, args, with_prep);
         case 2560: return launch_one<5, 8>(st, args, with_prep);
         case 4096: return launch_one<8, 4>(st, args, with_prep);
+        case 5120: return launch_one<10, 8>(st, args, with_prep);
         default: return set_error(RWKV_ERR_SIZE, "decode kernel: n_embd %d not supported", args.m.C);
     }
 }

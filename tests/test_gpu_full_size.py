@@ -130,16 +130,16 @@ def test_3b_width_two_layers_against_oracle():
 
 
 def test_14b_width_two_layers_prompt_chunks_batch_and_oracle():
-    """The 14B shape's width (C=5120, F=20480, V=50277; the persistent single-token kernel does not serve it:
-    320 tiles for 256 compute units), 2 layers: a prompt in chunks of 16 and single tokens through the many-row
-    kernels (their few-row product variant), one step of a batch of independent states, all against the CPU oracle."""
+    """The 14B shape's width (C=5120, F=20480, V=50277), 2 layers: a prompt in chunks of 16 through the many-row
+    kernels, single tokens through the persistent kernel (two groups of 16 channels per workgroup at this width:
+    320 tiles for 256 compute units), one step of a batch of independent states, all against the CPU oracle."""
     from rwkvstic_amd.model import HipRWKV
     _, C, F, V = synth.SHAPES["14B"]
     sd = synth.make_state_dict(2, C, F, V, seed=4, ln="random")
     ref = O.OracleModel(sd)
     exact = O.OracleModel(sd, matmul_dtype=torch.float64)
     hip = HipRWKV(sd)
-    assert not hip.fused_step
+    assert hip.fused_step
     prompt = synth.random_tokens(40, V=V, seed=15).tolist()
     _say("oracle prompt")
     lr, sr = ref.forward(prompt, ref.emptyState.clone())
@@ -178,7 +178,7 @@ def test_14b_width_batch_of_32_after_64_token_prompts():
     """The 14B configuration's batch decode at its real width (C=5120, F=20480, V=50277; 2 of the 40 layers): 32
     independent sequences, each with its own seeded random prompt of 64 tokens (prefilled through the many-row
     path; the 9..32-row product variant then serves the batch step at K = 5120 and 20480 inside the model), one
-    decode step of all 32 at once.  Every sequence of the batch must equal the same token fed on its own; four of
+    decode step of all 32 at once.  Every sequence of the batch must agree with the same token fed on its own; four of
     them are also checked, prompt and step, against the CPU oracle with exact accumulation (logits 1e-4, state
     1e-4).  A 256-token prompt fed as one 256-token chunk is checked against the same oracle."""
     from rwkvstic_amd.model import HipRWKV, wkv_state_to_reference
@@ -198,7 +198,9 @@ def test_14b_width_batch_of_32_after_64_token_prompts():
     for b in range(B):
         l1, s1 = hip.forward([last[b]], states[b].clone())
         assert float((lb[b] - l1).abs().max()) < 1e-5 and int(lb[b].argmax()) == int(l1.argmax()), b
-        assert float((sb[b, :, :2] - s1[:, :2]).abs().max()) < 1e-6, b
+        # (the lone token runs through the persistent kernel, whose LayerNorm statistics travel as float32 words;
+        # the batch step through the many-row kernels)
+        assert float((sb[b, :, :2] - s1[:, :2]).abs().max()) < 1e-5, b
 
     def state_close(s_gpu, s_ref, tol=1e-4):
         s = wkv_state_to_reference(s_gpu).cpu()

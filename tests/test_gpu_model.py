@@ -144,7 +144,7 @@ def test_169m_shape_greedy_128_tokens():
 
 
 # ------------------------------------------------------------------ persistent single-token kernel
-@pytest.mark.parametrize("C,L,V", [(1024, 2, 1999), (2560, 2, 5003), (2048, 1, 1600), (4096, 1, 1777)])
+@pytest.mark.parametrize("C,L,V", [(1024, 2, 1999), (2560, 2, 5003), (2048, 1, 1600), (4096, 1, 1777), (5120, 2, 1777)])
 def test_fused_step_matches_oracle_and_phase_kernels(C, L, V):
     from rwkvstic_amd.model import HipRWKV
     _say(f"fused step C={C} L={L} V={V}")
