@@ -182,7 +182,7 @@ def phase_trace(model, L: int, C: int) -> int:
     if not model.fused_step:
         print("phase trace: this shape does not run the persistent kernel", file=sys.stderr)
         return 2
-    G, per = C // 16, 24
+    G, per = (C // 32 if C > 4096 else C // 16), 24          # workgroups of the persistent kernel
     st = model.emptyState.clone()
     for t in range(5):
         _, st = model.forward([t + 3], st)

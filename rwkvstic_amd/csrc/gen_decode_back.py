@@ -48,6 +48,7 @@ PACE = int(os.environ.get("RWKV_BACK_PACE", "0"))        # s_sleep units (64 cyc
 # value phases (BARGATE) simply after the first barrier of the LayerNorm phase that follows, which the front waves
 # only reach with the statistics of all workgroups in hand.  Empty: no gate.
 GATE = [int(x) for x in os.environ.get("RWKV_BACK_GATE", "8,2,12,6").split(",")] if os.environ.get("RWKV_BACK_GATE", "8,2,12,6") else None
+GATE_WIDE = [int(x) for x in os.environ.get("RWKV_BACK_GATE_WIDE", "8,2,12,6").split(",")]     # the same for two groups per workgroup (C = 5120)
 BARGATE = int(os.environ.get("RWKV_BACK_BARGATE", "1"))   # reloads deferred past the att output and ffn value phases follow the next phase's first barrier
 CARRYK = int(os.environ.get("RWKV_BACK_CARRYK", "0"))     # the carried reloads follow this barrier of the LayerNorm phase (0: statistics, 1: digits ready)
 CARRYW = int(os.environ.get("RWKV_BACK_CARRYW", "0"))     # window of the carried reloads (0: the phase's)
@@ -81,6 +82,7 @@ def gen(KW, R, NV, NSH):
     NWG = 32 * KW // NT              # workgroups
     SADDR = KW > 8                   # no room for one offset register per block of a job: the block offset joins the base address in a scalar pair
     NJ = 13 * NT                     # jobs per layer
+    GATE = globals()["GATE"] if NT == 1 else GATE_WIDE
     NREAL = NJ * KW
     PP = (NREAL + R - 1) // R * R
     RB = NV - 4 * R
@@ -437,7 +439,7 @@ def gen(KW, R, NV, NSH):
 # (KW, front waves, ring size): 4 front waves -> 12 waves per workgroup, 168 VGPRs each;
 # 8 front waves -> 16 waves, 128 VGPRs each.
 CONFIGS = [(2, 4, 26), (4, 4, 26), (5, 4, 33), (8, 4, 26),
-           (2, 8, 13), (4, 8, 13), (5, 8, 22), (8, 8, 13), (10, 8, 20)]
+           (2, 8, 13), (4, 8, 13), (5, 8, 22), (8, 8, 13), (10, 8, int(os.environ.get("RWKV_BACK_R_WIDE", "20")))]
 
 
 def main():
