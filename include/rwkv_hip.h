@@ -235,6 +235,16 @@ int rwkv_model_set_trace(rwkv_model *m, int64_t *device_buffer);
  * incomplete), else RWKV_OK.  For tests and diagnostics. */
 int rwkv_model_check(rwkv_model *m);
 
+/* Self-test of the single-token kernel's failure path (no counterpart in the
+ * reference): launches one token step whose input is never published and whose
+ * waits give up after a few hundred polls instead of the usual million, so
+ * that every workgroup runs into its bounded wait, raises the abort flag and
+ * leaves - the launch ends normally within a millisecond.  state and logits
+ * are left untouched.  The next rwkv_model_check reports the aborted step
+ * (and clears the flag); token steps after that run as usual.  Only models
+ * with rwkv_model_has_fused_step. */
+int rwkv_model_selftest_timeout(rwkv_model *m, rwkv_stream_t stream, double *state, double *logits);
+
 /* Scratch needed by rwkv_model_forward for chunks of up to max_tokens tokens. */
 size_t rwkv_model_workspace_bytes(const rwkv_model *m, int64_t max_tokens);
 

@@ -119,6 +119,11 @@ int decode_clear_exchange(hipStream_t st, const DModel &m, const DecodeBuffers &
 // decode_epochs_per_token() between launches on the same buffers and never be 0.
 int decode_launch(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsigned epoch0,
                   const int64_t *token, double *state, double *logits);
+// One token step whose input never arrives, with waits that give up after spin_limit polls (self-test of the
+// failure path: the launch ends normally with the abort flag set; logits and state are left as they were).
+int decode_launch_unfed(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsigned epoch0, double *state, double *logits,
+                        unsigned spin_limit);
+
 // n greedy steps: tokens[i + 1] = argmax(forward(tokens[i])); uses n * decode_epochs_per_token() epochs.
 int decode_launch_greedy(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsigned epoch0,
                          int64_t *tokens, int64_t n, double *state, double *logits);

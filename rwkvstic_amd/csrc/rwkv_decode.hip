@@ -59,7 +59,7 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 
 constexpr int kBW = 8;                 // back (streaming) waves per workgroup
 constexpr int kRealJobs = 13;          // tile jobs per layer: k v r | o | ffn_r, 4 x ffn_k | 4 quarters of ffn_v
-constexpr unsigned kSpinLimit = 1u << 20;
+constexpr unsigned kSpinLimit = 1u << 20;        // polls before a wait gives up (DArgs::spin_limit; a self-test passes a small one)
 constexpr int kStatRows = 2;           // XR rows 0-1: sum x of a workgroup's 16 channels, and their squared deviations from the workgroup's own mean
 constexpr int kLnRows = kStatRows + 3 * 3;     // rows of the XR record table
 #ifndef RWKV_EARLY_DIV
@@ -104,6 +104,7 @@ struct DArgs {
     const int64_t *token;
     double *state;
     double *logits;
+    unsigned spin_limit;    // polls before a wait gives up
     const int *stop;        // device word or null: when it reads non-zero the launch does nothing (a sampled stop token
                             // ended the sequence; the remaining launches of a generation loop then leave the state alone)
 };
@@ -201,6 +202,7 @@ struct Front {
     int tid, wave, lane;
     unsigned *abort_flag;
     lds_flag_t *flags;
+    unsigned spin_limit;
     bool ok;
     __device__ __forceinline__ void refresh() {
         tid = opaque((int)threadIdx.x);
@@ -261,7 +263,7 @@ struct RowPoll {
             }
             if (missing == 0) break;
             __builtin_amdgcn_s_sleep(2);
-            if ((++spins & 63u) == 0u && (spins > kSpinLimit || ALOAD32(fx.abort_flag) != 0u || fx.flags[FLAG_ABORT])) fx.fail();
+            if ((++spins & 63u) == 0u && (spins > fx.spin_limit || ALOAD32(fx.abort_flag) != 0u || fx.flags[FLAG_ABORT])) fx.fail();
         }
 #pragma unroll
         for (int k = 0; k < K; ++k) {
@@ -309,7 +311,7 @@ __device__ __forceinline__ void wait_flag(Front &fx, int which, int seq) {
     unsigned spins = 0;
     while (fx.ok && fx.flags[which] < seq) {
         __builtin_amdgcn_s_sleep(1);
-        if ((++spins & 255u) == 0u && (spins > (kSpinLimit << 4) || fx.flags[FLAG_ABORT])) fx.fail();
+        if ((++spins & 255u) == 0u && (spins > (fx.spin_limit << 4) || fx.flags[FLAG_ABORT])) fx.fail();
     }
 }
 
@@ -350,7 +352,7 @@ __device__ __forceinline__ void settle_quads(Front &fx, xtab_t src, int first, i
         }
         if (all) break;
         __builtin_amdgcn_s_sleep(4);
-        if ((++spins & 63u) == 0u && (spins > kSpinLimit || ALOAD32(fx.abort_flag) != 0u)) { fx.fail(); break; }
+        if ((++spins & 63u) == 0u && (spins > fx.spin_limit || ALOAD32(fx.abort_flag) != 0u)) { fx.fail(); break; }
     }
 }
 
@@ -672,7 +674,7 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
     constexpr int NQH = F / 4, NQTH = (NQH + FT - 1) / FT, NQC = C / 4, NQTC = (NQC + FT - 1) / FT;
     static_assert(FW >= NT, "one finishing wave per group");
     Front fx;
-    fx.abort_flag = a.b.abort_flag; fx.flags = flags; fx.ok = true;
+    fx.abort_flag = a.b.abort_flag; fx.flags = flags; fx.spin_limit = a.spin_limit; fx.ok = true;
     fx.refresh();
     const int wg = blockIdx.x, L = a.m.L, V = a.m.V;
     const bool fin = fx.wave < NT;                       // wave gi finishes the workgroup's group gi of 16 channels
@@ -1418,15 +1420,26 @@ int decode_launch(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsig
                   const int64_t *token, double *state, double *logits) {
     DArgs args;
     args.m = m; args.b = b; args.epoch0 = epoch0; args.token = token; args.state = state; args.logits = logits;
-    args.stop = nullptr;
+    args.stop = nullptr; args.spin_limit = kSpinLimit;
     return launch_step(st, args, true);
+}
+
+// A token step whose input is never published (no preparation launch under this epoch) and whose waits give up
+// after spin_limit polls: every workgroup runs into its bounded wait, raises the abort flag and leaves.  Exercises
+// the failure path without anything that could hang: the limit is a few hundred polls.
+int decode_launch_unfed(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsigned epoch0, double *state, double *logits,
+                        unsigned spin_limit) {
+    DArgs args;
+    args.m = m; args.b = b; args.epoch0 = epoch0; args.token = nullptr; args.state = state; args.logits = logits;
+    args.stop = nullptr; args.spin_limit = spin_limit;
+    return launch_step(st, args, false);
 }
 
 int decode_launch_sampled(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsigned epoch0, int64_t *tokens, int64_t n,
                           double *state, double *logits, SampleArgs sa) {
     DArgs args;
     args.m = m; args.b = b; args.state = state; args.logits = logits;
-    args.stop = sa.stop_flag;
+    args.stop = sa.stop_flag; args.spin_limit = kSpinLimit;
     sa.logits = logits; sa.V = m.V;
     const unsigned ept = decode_epochs_per_token(m.L);
     for (int64_t i = 0; i < n; ++i) {
@@ -1446,7 +1459,7 @@ int decode_launch_greedy(hipStream_t st, const DModel &m, const DecodeBuffers &b
                          int64_t *tokens, int64_t n, double *state, double *logits) {
     DArgs args;
     args.m = m; args.b = b; args.state = state; args.logits = logits;
-    args.stop = nullptr;
+    args.stop = nullptr; args.spin_limit = kSpinLimit;
     const unsigned ept = decode_epochs_per_token(m.L);
     for (int64_t i = 0; i < n; ++i) {
         args.epoch0 = epoch0 + (unsigned)i * ept;

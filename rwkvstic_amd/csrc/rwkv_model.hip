@@ -756,6 +756,15 @@ int rwkv_model_check(rwkv_model *m) {
     return RWKV_OK;
 }
 
+int rwkv_model_selftest_timeout(rwkv_model *m, rwkv_stream_t stream, double *state, double *logits) {
+    RWKV_CHECK_ARG(m && state && logits, "rwkv_model_selftest_timeout: null pointer");
+    if (!m->fused) return set_error(RWKV_ERR_SIZE, "rwkv_model_selftest_timeout: this model does not run the persistent kernel");
+    RWKV_TRY(fused_epochs(m, (hipStream_t)stream, 1));
+    const int rc = decode_launch_unfed((hipStream_t)stream, m->dm, m->db, m->epoch, state, logits, 256u);
+    m->epoch += decode_epochs_per_token(m->d.n_layer);
+    return rc;
+}
+
 size_t rwkv_model_workspace_bytes(const rwkv_model *m, int64_t max_tokens) {
     if (!m || max_tokens <= 0) return 0;
     size_t n = round_up(ws_doubles(m->d.n_embd, m->d.n_ffn) * sizeof(double), 256);

@@ -254,6 +254,15 @@ class HipRWKV:
         """Synchronise and raise if a single-token launch gave up waiting (diagnostics)."""
         N.check(N.lib().rwkv_model_check(self._handle))
 
+    def selftest_timeout(self, state: torch.Tensor) -> None:
+        """Launch one token step whose input never arrives and whose waits give up after a few hundred polls: the
+        launch ends normally, ``state`` is untouched, and the next ``check()`` raises (self-test of the failure path)."""
+        self._check_state(state)
+        logits = torch.empty(self.vocab, dtype=torch.float64, device=self.device)
+        with torch.cuda.device(self.device):
+            N.check(N.lib().rwkv_model_selftest_timeout(self._handle, torch.cuda.current_stream().cuda_stream,
+                                                        state.data_ptr(), logits.data_ptr()))
+
     def weight_bytes(self) -> int:
         """uint8 weight bytes streamed per decoded token: L*13*C^2 + V*C."""
         n = self.head.nbytes()

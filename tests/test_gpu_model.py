@@ -444,3 +444,33 @@ def test_host_resident_weights_give_identical_results():
     la, sa = a.forward([3, 4], a.emptyState.clone())
     lb, sb = b.forward([3, 4], b.emptyState.clone())
     assert torch.equal(la, lb) and torch.equal(sa, sb)
+
+
+@pytest.mark.parametrize("C,L", [(1024, 2), (2560, 1), (5120, 1)])
+def test_a_token_step_that_never_gets_its_input_drains_and_is_reported(C, L):
+    """The failure path of the persistent kernel, forced from the host without anything that could hang: a token
+    step is launched whose input is never published and whose waits give up after a few hundred polls.  Every
+    workgroup must leave (the launch ends), the state must be untouched, check() must report the step once, and
+    the steps after it must give exactly what a model that never saw the failure gives."""
+    from rwkvstic_amd.model import HipRWKV
+    V = 1500
+    sd = synth.make_state_dict(L, C, 4 * C, V, seed=77 + C, ln="random")
+    hip, clean = HipRWKV(sd), HipRWKV(sd)
+    assert hip.fused_step
+    toks = synth.random_tokens(4, V=V, seed=3).tolist()
+    s, sc = hip.emptyState.clone(), clean.emptyState.clone()
+    for t in toks[:2]:
+        _, s = hip.forward([t], s)
+        _, sc = clean.forward([t], sc)
+    before = s.clone()
+    _say(f"unfed token step, C={C}")
+    hip.selftest_timeout(s)
+    with pytest.raises(RuntimeError, match="gave up waiting"):
+        hip.check()
+    assert torch.equal(s, before)
+    hip.check()                                        # reported once, then clear
+    for t in toks[2:]:
+        lg, s = hip.forward([t], s)
+        lc, sc = clean.forward([t], sc)
+    hip.check()
+    assert torch.equal(lg, lc) and torch.equal(s, sc)
