@@ -48,7 +48,8 @@ PACE = int(os.environ.get("RWKV_BACK_PACE", "0"))        # s_sleep units (64 cyc
 # value phases (BARGATE) simply after the first barrier of the LayerNorm phase that follows, which the front waves
 # only reach with the statistics of all workgroups in hand.  Empty: no gate.
 GATE = [int(x) for x in os.environ.get("RWKV_BACK_GATE", "8,2,12,6").split(",")] if os.environ.get("RWKV_BACK_GATE", "8,2,12,6") else None
-GATE_WIDE = [int(x) for x in os.environ.get("RWKV_BACK_GATE_WIDE", "8,2,12,6").split(",")]     # the same for two groups per workgroup (C = 5120)
+WINDOW_WIDE = int(os.environ.get("RWKV_BACK_WINDOW_WIDE", "12"))
+GATE_WIDE = [int(x) for x in os.environ.get("RWKV_BACK_GATE_WIDE", "16,8,16,12").split(",")]     # the same for two groups per workgroup (C = 5120)
 BARGATE = int(os.environ.get("RWKV_BACK_BARGATE", "1"))   # reloads deferred past the att output and ffn value phases follow the next phase's first barrier
 CARRYK = int(os.environ.get("RWKV_BACK_CARRYK", "0"))     # the carried reloads follow this barrier of the LayerNorm phase (0: statistics, 1: digits ready)
 CARRYW = int(os.environ.get("RWKV_BACK_CARRYW", "0"))     # window of the carried reloads (0: the phase's)
@@ -57,11 +58,14 @@ S_SEQ = 98        # phases finished by this wave (the front waves' exchange sequ
 SLEEP = int(os.environ.get("RWKV_BACK_SLEEP", "0"))      # s_sleep units (64 cycles) between a phase's barrier and its reloads   # weight loads a wave keeps in flight while it reloads slots
 
 
+S_FLAG = 100      # LDS address of the abort / go flag pair, where no register holds it (compact register map)
+
+
 class Emit:
-    def __init__(self):
+    def __init__(self, na=NA):
         self.lines = []
         self.issued = 0          # LDS operations issued since the last full drain
-        self.ridx = [0] * NA      # issue index of the read into A buffer k
+        self.ridx = [0] * na      # issue index of the read into A buffer k
 
     def __call__(self, s):
         self.lines.append(s)
@@ -81,8 +85,14 @@ def gen(KW, R, NV, NSH):
     SPG = 5                          # parked-tile slots per group
     NWG = 32 * KW // NT              # workgroups
     SADDR = KW > 8                   # no room for one offset register per block of a job: the block offset joins the base address in a scalar pair
+    # Compact register map where block offsets travel on the scalar side: one offset register, two A-operand buffers
+    # and no register for the flag address leave room for a ring of 26 blocks in 128 registers.
+    V_OFF, V_D, V_A, NA = (7, 8, 16, 2) if SADDR else (globals()["V_OFF"], globals()["V_D"], globals()["V_A"], globals()["NA"])
+    PF = NA - 1
     NJ = 13 * NT                     # jobs per layer
     GATE = globals()["GATE"] if NT == 1 else GATE_WIDE
+    WINDOW = globals()["WINDOW"] if NT == 1 else WINDOW_WIDE
+    WINDOWS = globals()["WINDOWS"] if NT == 1 else [WINDOW_WIDE] * 4
     NREAL = NJ * KW
     PP = (NREAL + R - 1) // R * R
     RB = NV - 4 * R
@@ -131,7 +141,14 @@ def gen(KW, R, NV, NSH):
             assert extra == 0
             e(f"global_load_dwordx4 {dst}, v{V_OFF + b}, s[{sbase}:{sbase + 1}]")
     LH = R * KW // math.gcd(R, KW)
-    e = Emit()
+    e = Emit(NA)
+
+    def flag_addr():
+        """Register that holds the LDS address of the flag pair (valid where no A-operand read is in flight)."""
+        if not SADDR:
+            return f"v{V_FLAG}"
+        e(f"v_mov_b32 v{V_A + 2}, s{S_FLAG}")
+        return f"v{V_A + 2}"
 
     def ring(slot):
         return f"v[{RB + 4 * slot}:{RB + 4 * slot + 3}]"
@@ -157,7 +174,7 @@ def gen(KW, R, NV, NSH):
     def bar_check():
         e("s_waitcnt lgkmcnt(0)")
         e("s_barrier")
-        e(f"ds_read_b32 v{V_A}, v{V_FLAG}")
+        e(f"ds_read_b32 v{V_A}, {flag_addr()}")
         e("s_waitcnt lgkmcnt(0)")
         e(f"v_readfirstlane_b32 s{S_T}, v{V_A}")
         e(f"s_cmp_lg_u32 s{S_T}, 0")
@@ -192,7 +209,7 @@ def gen(KW, R, NV, NSH):
     e(f"v_lshlrev_b32 v{V_PARK}, 4, v{V_A}")
     e(f"v_add_u32 v{V_PARK}, s{S_T}, v{V_PARK}")
     e(f"s_add_u32 s{S_T}, %[lds], {FLAG}")
-    e(f"v_mov_b32 v{V_FLAG}, s{S_T}")
+    e(f"s_mov_b32 s{S_FLAG}, s{S_T}" if SADDR else f"v_mov_b32 v{V_FLAG}, s{S_T}")
     e(f"s_lshl_b32 s{S_T}, %[wb], 10")
     e(f"v_lshlrev_b32 v{V_OFF}, 4, v{V_A}")
     e(f"v_add_u32 v{V_OFF}, s{S_T}, v{V_OFF}")
@@ -311,7 +328,7 @@ def gen(KW, R, NV, NSH):
                 e(f"s_add_u32 s{S_T}, s{S_SEQ}, 1")
                 e(f"s_mov_b32 s{S_TILE}, {GATE_SPINS}")       # (free until the head)
                 e(f"7{ph}:")
-                e(f"ds_read_b64 v[{V_A}:{V_A + 1}], v{V_FLAG}")
+                e(f"ds_read_b64 v[{V_A}:{V_A + 1}], {flag_addr()}")
                 e("s_waitcnt lgkmcnt(0)")
                 e(f"v_readfirstlane_b32 vcc_lo, v{V_A}")
                 e(f"v_readfirstlane_b32 vcc_hi, v{V_A + 1}")
@@ -439,7 +456,7 @@ def gen(KW, R, NV, NSH):
 # (KW, front waves, ring size): 4 front waves -> 12 waves per workgroup, 168 VGPRs each;
 # 8 front waves -> 16 waves, 128 VGPRs each.
 CONFIGS = [(2, 4, 26), (4, 4, 26), (5, 4, 33), (8, 4, 26),
-           (2, 8, 13), (4, 8, 13), (5, 8, 22), (8, 8, 13), (10, 8, int(os.environ.get("RWKV_BACK_R_WIDE", "20")))]
+           (2, 8, 13), (4, 8, 13), (5, 8, 22), (8, 8, 13), (10, 8, int(os.environ.get("RWKV_BACK_R_WIDE", "26")))]
 
 
 def main():
@@ -450,7 +467,7 @@ def main():
     w("template <int KW, int FW> struct BackCfg;")
     for KW, FW, R in CONFIGS:
         NV = 168 if FW == 4 else 128
-        clob = ", ".join(f'"v{i}"' for i in range(V_APC, NV)) + ", " + ", ".join(f'"s{i}"' for i in range(S_CUR, 100))
+        clob = ", ".join(f'"v{i}"' for i in range(V_APC, NV)) + ", " + ", ".join(f'"s{i}"' for i in range(S_CUR, 102 if KW > 8 else 100))
         tiles_per_body = R // math.gcd(R, KW)
         NSH = max(d for d in range(1, 5) if tiles_per_body % d == 0)     # head tiles per barrier round
         lines, info = gen(KW, R, NV, NSH)
