@@ -235,6 +235,16 @@ int rwkv_model_set_trace(rwkv_model *m, int64_t *device_buffer);
  * incomplete), else RWKV_OK.  For tests and diagnostics. */
 int rwkv_model_check(rwkv_model *m);
 
+/* Measurement aid (no counterpart in the reference): feeds the token at *token
+ * n times (the state advances n steps) with HIP events recorded on the stream
+ * immediately before and after each launch of the persistent single-token
+ * kernel - the per-token preparation launch stays outside the pair - then
+ * synchronises the stream and returns the kernel's average duration in
+ * microseconds.  Creates and destroys 2 n events.  Only models with
+ * rwkv_model_has_fused_step. */
+int rwkv_model_time_token_kernel(rwkv_model *m, rwkv_stream_t stream, const int64_t *token, double *state,
+                                 double *logits, int n, float *avg_us);
+
 /* Self-test of the single-token kernel's failure path (no counterpart in the
  * reference): launches one token step whose input is never published and whose
  * waits give up after a few hundred polls instead of the usual million, so

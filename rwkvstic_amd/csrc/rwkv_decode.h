@@ -119,6 +119,10 @@ int decode_clear_exchange(hipStream_t st, const DModel &m, const DecodeBuffers &
 // decode_epochs_per_token() between launches on the same buffers and never be 0.
 int decode_launch(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsigned epoch0,
                   const int64_t *token, double *state, double *logits);
+// decode_launch with events recorded on the stream around the token kernel alone (after the preparation launch).
+int decode_launch_bracketed(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsigned epoch0, const int64_t *token,
+                            double *state, double *logits, hipEvent_t before, hipEvent_t after);
+
 // One token step whose input never arrives, with waits that give up after spin_limit polls (self-test of the
 // failure path: the launch ends normally with the abort flag set; logits and state are left as they were).
 int decode_launch_unfed(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsigned epoch0, double *state, double *logits,

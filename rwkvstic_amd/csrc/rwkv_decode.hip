@@ -1001,28 +1001,40 @@ __device__ __forceinline__ void prep_layer_part(const DArgs &a, int l, int part,
 // x0 = ln0(emb[tok]) (emb.py:9, opt.py:63-64), published with its LayerNorm records as the input
 // of layer 0 under `epoch`.  C is a multiple of 512 and thread t takes channels t, t + 512, ...
 __device__ __forceinline__ void prep_token(const DArgs &a, int64_t tok, unsigned epoch, double *scr) {
-    const int C = a.m.C, G = a.m.G;
+    constexpr int kMaxParts = 10;                               // C <= 5120
+    const int C = a.m.C, G = a.m.G, parts = C / kPrepThreads;
     if (tok < 0) tok = 0;
     if (tok >= a.m.V) tok = a.m.V - 1;
-    double s[2] = {0.0, 0.0};
-    for (int c = threadIdx.x; c < C; c += kPrepThreads) {
-        const double v = (double)a.m.emb[(size_t)tok * C + c];
-        s[0] += v; s[1] += v * v;
+    // everything this thread needs is requested before the first use: the block is one chain of memory latencies otherwise
+    double v[kMaxParts], lw[kMaxParts], lb[kMaxParts], PO[kMaxParts][3];
+    float P[kMaxParts][3];
+#pragma unroll
+    for (int k = 0; k < kMaxParts; ++k) {
+        const int c = threadIdx.x + k * kPrepThreads;
+        if (k < parts) {
+            v[k] = (double)a.m.emb[(size_t)tok * C + c];
+            lw[k] = a.m.ln0_w[c]; lb[k] = a.m.ln0_b[c];
+#pragma unroll
+            for (int m = 0; m < 3; ++m) { P[k][m] = a.m.P32[(size_t)m * C + c]; PO[k][m] = a.m.PO[(size_t)m * C + c]; }
+        }
     }
+    double s[2] = {0.0, 0.0};
+#pragma unroll
+    for (int k = 0; k < kMaxParts; ++k)
+        if (k < parts) { s[0] += v[k]; s[1] += v[k] * v[k]; }
     prep_block_sum<2>(s, scr);
     const double mean = s[0] / (double)C;
     double var = s[1] / (double)C - mean * mean;
     if (var < 0.0) var = 0.0;
     const double rsd = 1.0 / sqrt(var + 1e-5);
-    for (int c = threadIdx.x; c < C; c += kPrepThreads) {     // whole waves are in or out: C % 64 == 0
-        const double v = (double)a.m.emb[(size_t)tok * C + c];
-        const double x0 = a.m.ln0_w[c] * ((v - mean) * rsd) + a.m.ln0_b[c];
-        a.m.X0[c] = x0;
-        float P[3];
-        double PO[3];
 #pragma unroll
-        for (int m = 0; m < 3; ++m) { P[m] = a.m.P32[(size_t)m * C + c]; PO[m] = a.m.PO[(size_t)m * C + c]; }
-        publish_ln_input<3>(a.b.X, a.b.XR, G, c >> 4, c & 15, epoch, x0, P, PO);
+    for (int k = 0; k < kMaxParts; ++k) {                       // whole waves are in or out: C % 512 == 0
+        if (k < parts) {
+            const int c = threadIdx.x + k * kPrepThreads;
+            const double x0 = lw[k] * ((v[k] - mean) * rsd) + lb[k];
+            a.m.X0[c] = x0;
+            publish_ln_input<3>(a.b.X, a.b.XR, G, c >> 4, c & 15, epoch, x0, P[k], PO[k]);
+        }
     }
 }
 
@@ -1422,6 +1434,22 @@ int decode_launch(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsig
     args.m = m; args.b = b; args.epoch0 = epoch0; args.token = token; args.state = state; args.logits = logits;
     args.stop = nullptr; args.spin_limit = kSpinLimit;
     return launch_step(st, args, true);
+}
+
+// One token step with events recorded on the stream right before and right after the token kernel itself (the
+// preparation launch stays outside the pair): the kernel's own duration, for measurements.
+int decode_launch_bracketed(hipStream_t st, const DModel &m, const DecodeBuffers &b, unsigned epoch0, const int64_t *token,
+                            double *state, double *logits, hipEvent_t before, hipEvent_t after) {
+    DArgs args;
+    args.m = m; args.b = b; args.epoch0 = epoch0; args.token = token; args.state = state; args.logits = logits;
+    args.stop = nullptr; args.spin_limit = kSpinLimit;
+    hipLaunchKernelGGL(prep_kernel, dim3((unsigned)(m.L * (m.C / kPrepThreads) + 1)), dim3(kPrepThreads), 0, st, args);
+    RWKV_CHECK_LAUNCH("prep_kernel");
+    RWKV_CHECK_HIP(hipEventRecord(before, st));
+    const int rc = launch_step(st, args, false);
+    if (rc) return rc;
+    RWKV_CHECK_HIP(hipEventRecord(after, st));
+    return RWKV_OK;
 }
 
 // A token step whose input is never published (no preparation launch under this epoch) and whose waits give up

@@ -756,6 +756,34 @@ int rwkv_model_check(rwkv_model *m) {
     return RWKV_OK;
 }
 
+int rwkv_model_time_token_kernel(rwkv_model *m, rwkv_stream_t stream, const int64_t *token, double *state, double *logits,
+                                 int n, float *avg_us) {
+    RWKV_CHECK_ARG(m && token && state && logits && avg_us, "rwkv_model_time_token_kernel: null pointer");
+    RWKV_CHECK_ARG(n > 0 && n <= 4096, "rwkv_model_time_token_kernel: n must be in 1..4096");
+    if (!m->fused) return set_error(RWKV_ERR_SIZE, "rwkv_model_time_token_kernel: this model does not run the persistent kernel");
+    const hipStream_t st = (hipStream_t)stream;
+    std::vector<hipEvent_t> ev((size_t)2 * n, nullptr);
+    int rc = RWKV_OK;
+    for (auto &e : ev)
+        if (rc == RWKV_OK && hipEventCreate(&e) != hipSuccess) rc = set_error(RWKV_ERR_HIP, "rwkv_model_time_token_kernel: hipEventCreate failed");
+    for (int i = 0; i < n && rc == RWKV_OK; ++i) {
+        rc = fused_epochs(m, st, 1);
+        if (rc == RWKV_OK) rc = decode_launch_bracketed(st, m->dm, m->db, m->epoch, token, state, logits, ev[2 * i], ev[2 * i + 1]);
+        m->epoch += decode_epochs_per_token(m->d.n_layer);
+    }
+    if (rc == RWKV_OK && hipStreamSynchronize(st) != hipSuccess) rc = set_error(RWKV_ERR_HIP, "rwkv_model_time_token_kernel: synchronize failed");
+    double total_ms = 0.0;
+    for (int i = 0; i < n && rc == RWKV_OK; ++i) {
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, ev[2 * i], ev[2 * i + 1]) != hipSuccess) rc = set_error(RWKV_ERR_HIP, "rwkv_model_time_token_kernel: hipEventElapsedTime failed");
+        total_ms += (double)ms;
+    }
+    for (auto &e : ev)
+        if (e) (void)hipEventDestroy(e);
+    if (rc == RWKV_OK) *avg_us = (float)(total_ms * 1e3 / n);
+    return rc;
+}
+
 int rwkv_model_selftest_timeout(rwkv_model *m, rwkv_stream_t stream, double *state, double *logits) {
     RWKV_CHECK_ARG(m && state && logits, "rwkv_model_selftest_timeout: null pointer");
     if (!m->fused) return set_error(RWKV_ERR_SIZE, "rwkv_model_selftest_timeout: this model does not run the persistent kernel");

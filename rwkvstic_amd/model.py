@@ -263,6 +263,19 @@ class HipRWKV:
             N.check(N.lib().rwkv_model_selftest_timeout(self._handle, torch.cuda.current_stream().cuda_stream,
                                                         state.data_ptr(), logits.data_ptr()))
 
+    def time_token_kernel(self, token: int, n: int, state: torch.Tensor) -> float:
+        """Feed ``token`` ``n`` times (``state`` advances) and return the persistent kernel's own average duration
+        in microseconds, from events recorded on the stream around each of its launches (measurement aid)."""
+        import ctypes
+        self._check_state(state)
+        tok = torch.tensor([int(token)], dtype=torch.int64, device=self.device)
+        logits = torch.empty(self.vocab, dtype=torch.float64, device=self.device)
+        us = ctypes.c_float(0.0)
+        with torch.cuda.device(self.device):
+            N.check(N.lib().rwkv_model_time_token_kernel(self._handle, torch.cuda.current_stream().cuda_stream, tok.data_ptr(),
+                                                         state.data_ptr(), logits.data_ptr(), int(n), ctypes.byref(us)))
+        return float(us.value)
+
     def weight_bytes(self) -> int:
         """uint8 weight bytes streamed per decoded token: L*13*C^2 + V*C."""
         n = self.head.nbytes()

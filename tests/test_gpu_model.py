@@ -474,3 +474,20 @@ def test_a_token_step_that_never_gets_its_input_drains_and_is_reported(C, L):
         lc, sc = clean.forward([t], sc)
     hip.check()
     assert torch.equal(lg, lc) and torch.equal(s, sc)
+
+
+def test_timed_token_steps_advance_the_state_like_forward():
+    """rwkv_model_time_token_kernel: n steps with events around the persistent kernel only; the state it leaves is
+    the one n forward() calls leave, and the duration is a plausible positive number."""
+    from rwkvstic_amd.model import HipRWKV
+    L, C, V = 2, 1024, 1200
+    sd = synth.make_state_dict(L, C, 4 * C, V, seed=12, ln="random")
+    hip = HipRWKV(sd)
+    assert hip.fused_step
+    s1, s2 = hip.emptyState.clone(), hip.emptyState.clone()
+    us = hip.time_token_kernel(17, 5, s1)
+    for _ in range(5):
+        _, s2 = hip.forward([17], s2)
+    hip.check()
+    assert torch.equal(s1, s2)
+    assert 1.0 < us < 5000.0
