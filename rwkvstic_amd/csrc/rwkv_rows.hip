@@ -229,6 +229,12 @@ __global__ void __launch_bounds__(kLT) rows_ln_mix_quant_kernel(const LnQuantArg
         const int c0 = 4 * (tid + g * kLT);
         if (c0 < C) {
             double xy[4], prev[4];
+            if (kLT < 512 && NM > 0) {
+                // many rows: the previous row's values are read again here (a cache hit) instead of staying in
+                // registers through the two reductions above: 48 registers less, one more row per compute unit
+                const double2 p0 = *reinterpret_cast<const double2 *>(pr + c0), p1 = *reinterpret_cast<const double2 *>(pr + c0 + 2);
+                pv[g][0] = p0.x; pv[g][1] = p0.y; pv[g][2] = p1.x; pv[g][3] = p1.y;
+            }
             if (kLT < 512) {
                 const double2 w0 = *reinterpret_cast<const double2 *>(a.ln_w + c0), w1 = *reinterpret_cast<const double2 *>(a.ln_w + c0 + 2);
                 const double2 b0 = *reinterpret_cast<const double2 *>(a.ln_b + c0), b1 = *reinterpret_cast<const double2 *>(a.ln_b + c0 + 2);
