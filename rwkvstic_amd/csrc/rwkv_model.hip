@@ -601,10 +601,12 @@ int rows_layers(rwkv_model *m, hipStream_t st, const int64_t *tokens, int64_t R,
         const double *of[3] = {kvr[0]->offset, kvr[1]->offset, kvr[2]->offset};
         RWKV_TRY(rows_ln_mix_quant(st, 3, R, C, sequence, w.x, L.ln1_w, L.ln1_b, L.att_mix, copy_prev ? w.prev0 : sl, sl,
                                    state_stride, rg, of, w.q));
+        // k, v, r (and the ffn receptance below) are kept as float32 arrays in the kvr slab
+        float *kvr32 = reinterpret_cast<float *>(w.kvr);
         RowsProduct pk[3];
-        for (int i = 0; i < 3; ++i) { pk[i].a = w.q[i]; pk[i].w16 = kvr[i]->packed16; pk[i].out = w.kvr + i * RC; }
-        RWKV_TRY(rows_products(st, 3, pk, w.tot, R, C, C, ROW_STORE, nullptr));
-        RWKV_TRY(rows_wkv(st, R, C, sequence, w.kvr, w.kvr + RC, w.kvr + 2 * RC, L.time_decay, L.time_first,
+        for (int i = 0; i < 3; ++i) { pk[i].a = w.q[i]; pk[i].w16 = kvr[i]->packed16; pk[i].out = reinterpret_cast<double *>(kvr32 + i * RC); }
+        RWKV_TRY(rows_products(st, 3, pk, w.tot, R, C, C, ROW_STORE_F32, nullptr));
+        RWKV_TRY(rows_wkv(st, R, C, sequence, kvr32, kvr32 + RC, kvr32 + 2 * RC, L.time_decay, L.time_first,
                           sl + 2 * (size_t)C, state_stride, w.att, w.wkv_scr));
         RWKV_TRY(rows_quant(st, R, C, w.att, L.att_o.range, L.att_o.offset, w.q[0], (double *)w.tot));
         const RowsProduct po = {w.q[0], L.att_o.packed16, w.x};
@@ -617,10 +619,10 @@ int rows_layers(rwkv_model *m, hipStream_t st, const int64_t *tokens, int64_t R,
                                    sl + C, state_stride, rg2, of2, w.q + 1));
         const RowsProduct pfk = {w.q[1], L.ffn_k.packed16, w.h}, pfr = {w.q[2], L.ffn_r.packed16, w.kvr};
         RWKV_TRY(rows_products(st, 1, &pfk, w.tot, R, C, F, ROW_RELU2, nullptr));
-        RWKV_TRY(rows_products(st, 1, &pfr, w.tot, R, C, C, ROW_STORE, nullptr));
+        RWKV_TRY(rows_products(st, 1, &pfr, w.tot, R, C, C, ROW_STORE_F32, nullptr));
         RWKV_TRY(rows_quant(st, R, F, w.h, L.ffn_v.range, L.ffn_v.offset, w.q[0], (double *)w.tot));
         const RowsProduct pfv = {w.q[0], L.ffn_v.packed16, w.x};
-        RWKV_TRY(rows_products(st, 1, &pfv, w.tot, R, F, C, ROW_GATE_ADD, w.kvr));
+        RWKV_TRY(rows_products(st, 1, &pfv, w.tot, R, F, C, ROW_GATE_ADD, kvr32));
     }
     return RWKV_OK;
 }

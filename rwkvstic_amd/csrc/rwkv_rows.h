@@ -5,7 +5,9 @@
 
 namespace rwkv {
 
-enum RowTail { ROW_STORE = 0, ROW_RELU2 = 1, ROW_ADD = 2, ROW_GATE_ADD = 3 };
+// ROW_STORE_F32: the product's `out` points at a float32 [R, N] array (k, v, r and the ffn receptance: their consumers
+// round them to float32 anyway, as the single-token kernel does, and the arrays are read several times)
+enum RowTail { ROW_STORE = 0, ROW_RELU2 = 1, ROW_ADD = 2, ROW_GATE_ADD = 3, ROW_STORE_F32 = 4 };
 
 // One quantised left operand of a product: R rows rewritten as fixed-point digit fragments plus the
 // per-row constants of the tail (scale, sum of the fixed-point values, zero-point sum).
@@ -43,8 +45,8 @@ int rows_quant(hipStream_t st, int64_t R, int64_t K, const double *in, const flo
 // n (<= kRowsMaxProducts) products of the same shape [R, K] x [K, N] and tail in one launch;
 // tot: n * rows_tot_bytes(R, N) bytes of scratch.
 int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, int64_t R, int64_t K, int64_t N, int op,
-                  const double *gate);
-int rows_wkv(hipStream_t st, int64_t R, int C, bool sequence, const double *k, const double *v, const double *r,
+                  const float *gate);
+int rows_wkv(hipStream_t st, int64_t R, int C, bool sequence, const float *k, const float *v, const float *r,
              const double *w, const double *u, double *state, int64_t state_stride, double *out,
              double *scratch /* rows_wkv_scratch_bytes(R, C), or null: serial over the rows */);
 

@@ -554,7 +554,7 @@ struct GemmArgs {
     int gx, gy, gz, per_xcd, by_rows;   // logical grid (column blocks, row blocks, splits x products) behind the 1-D launch
     // when the contraction is not split the tail of the product is applied here (see rows_finish_kernel)
     int tail, R, N;                 // tail < 0: totals only
-    const double *gate;
+    const float *gate;
 };
 
 constexpr int kGemmNT = 8, kGemmWideNT = 10;     // N-tiles per workgroup (two wavefronts side by side)
@@ -601,9 +601,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs &a, const v4i (&acc
                     const double y = S * (double)tot + add;
                     double *o = outv + (size_t)t * a.N + col;
                     if (a.tail == ROW_STORE) *o = y;
+                    else if (a.tail == ROW_STORE_F32) reinterpret_cast<float *>(outv)[(size_t)t * a.N + col] = (float)y;
                     else if (a.tail == ROW_RELU2) { const double r = y > 0.0 ? y : 0.0; *o = r * r; }              // block.py:97
                     else if (a.tail == ROW_ADD) *o += y;                                                            // block.py:80
-                    else *o += y * (1.0 / (1.0 + exp(-a.gate[(size_t)t * a.N + col])));                             // block.py:95-100
+                    else *o += y * (1.0 / (1.0 + exp(-(double)a.gate[(size_t)t * a.N + col])));                     // block.py:95-100
                 }
                 continue;
             }
@@ -914,7 +915,7 @@ struct FinishArgs {
     const long long *tot;       // [products][slices][...]
     const double *S[kRowsMaxProducts], *qs[kRowsMaxProducts], *zp[kRowsMaxProducts];
     double *out[kRowsMaxProducts];      // [R, N] each
-    const double *gate;         // ROW_GATE_ADD: raw receptance [R, N]
+    const float *gate;          // ROW_GATE_ADD: raw receptance [R, N]
 };
 
 template <int OP>
@@ -933,9 +934,10 @@ __global__ void __launch_bounds__(256) rows_finish_kernel(const FinishArgs a) {
     const double y = S * (double)tot + 128.0 * (S * qsv[t]) + zpv[t];
     double *o = outv + (size_t)t * a.N + j;
     if (OP == ROW_STORE) *o = y;
+    else if (OP == ROW_STORE_F32) reinterpret_cast<float *>(outv)[(size_t)t * a.N + j] = (float)y;
     else if (OP == ROW_RELU2) { const double r = y > 0.0 ? y : 0.0; *o = r * r; }            // block.py:97
     else if (OP == ROW_ADD) *o += y;                                                          // block.py:80
-    else if (OP == ROW_GATE_ADD) *o += y * (1.0 / (1.0 + exp(-a.gate[(size_t)t * a.N + j]))); // block.py:95-100
+    else if (OP == ROW_GATE_ADD) *o += y * (1.0 / (1.0 + exp(-(double)a.gate[(size_t)t * a.N + j]))); // block.py:95-100
 }
 
 // ---------------------------------------------------------------------------
@@ -944,7 +946,7 @@ __global__ void __launch_bounds__(256) rows_finish_kernel(const FinishArgs a) {
 // ---------------------------------------------------------------------------
 struct WkvRowsArgs {
     int C, R, sequence;
-    const double *k, *v, *r;    // [R, C]
+    const float *k, *v, *r;     // [R, C]  float32: what the single-token kernel rounds them to as well
     const double *w, *u;        // [C]  (w = -exp(time_decay))
     double *state;              // rows aa, bb, pp of the layer: state + 2C; batch: + row * state_stride
     int64_t state_stride;
@@ -961,8 +963,8 @@ __global__ void __launch_bounds__(64) wkv_rows_kernel(const WkvRowsArgs a) {
     double aa = st[c], bb = st[C + c], pp = st[2 * C + c];
     for (int t = t0; t < t1; ++t) {
         const size_t i = (size_t)t * C + c;
-        const double y = wkv_step<double>(w, u, a.k[i], a.v[i], aa, bb, pp);
-        a.out[i] = y * (1.0 / (1.0 + exp(-a.r[i])));
+        const double y = wkv_step<double>(w, u, (double)a.k[i], (double)a.v[i], aa, bb, pp);
+        a.out[i] = y * (1.0 / (1.0 + exp(-(double)a.r[i])));
     }
     st[c] = aa; st[C + c] = bb; st[2 * C + c] = pp;
 }
@@ -986,7 +988,7 @@ __global__ void __launch_bounds__(64) wkv_chunk_local_kernel(const WkvRowsArgs a
     const double w = a.w[c], u = a.u[c];
     const int t0 = j * kWkvChunk, t1 = min(t0 + kWkvChunk, a.R);
     double aa = 0.0, bb = 0.0, pp = -1e30;
-    double kc[kWkvGroup], vc[kWkvGroup], kn[kWkvGroup], vn[kWkvGroup];
+    float kc[kWkvGroup], vc[kWkvGroup], kn[kWkvGroup], vn[kWkvGroup];
 #pragma unroll
     for (int i = 0; i < kWkvGroup; ++i) {
         const size_t o = (size_t)min(t0 + i, t1 - 1) * C + c;
@@ -1000,7 +1002,7 @@ __global__ void __launch_bounds__(64) wkv_chunk_local_kernel(const WkvRowsArgs a
         }
 #pragma unroll
         for (int i = 0; i < kWkvGroup; ++i)
-            if (g + i < t1) (void)wkv_step<double>(w, u, kc[i], vc[i], aa, bb, pp);
+            if (g + i < t1) (void)wkv_step<double>(w, u, (double)kc[i], (double)vc[i], aa, bb, pp);
 #pragma unroll
         for (int i = 0; i < kWkvGroup; ++i) { kc[i] = kn[i]; vc[i] = vn[i]; }
     }
@@ -1055,7 +1057,7 @@ __global__ void __launch_bounds__(64) wkv_chunk_replay_kernel(const WkvRowsArgs 
     const int t0 = j * kWkvChunk, t1 = min(t0 + kWkvChunk, a.R);
     const double *in = scr + (size_t)j * 3 * C;
     double aa = in[c], bb = in[C + c], pp = in[2 * C + c];
-    double kc[kWkvGroup], vc[kWkvGroup], rc[kWkvGroup], kn[kWkvGroup], vn[kWkvGroup], rn[kWkvGroup];
+    float kc[kWkvGroup], vc[kWkvGroup], rc[kWkvGroup], kn[kWkvGroup], vn[kWkvGroup], rn[kWkvGroup];
 #pragma unroll
     for (int i = 0; i < kWkvGroup; ++i) {
         const size_t o = (size_t)min(t0 + i, t1 - 1) * C + c;
@@ -1070,8 +1072,8 @@ __global__ void __launch_bounds__(64) wkv_chunk_replay_kernel(const WkvRowsArgs 
 #pragma unroll
         for (int i = 0; i < kWkvGroup; ++i) {
             if (g + i < t1) {
-                const double y = wkv_step<double>(w, u, kc[i], vc[i], aa, bb, pp);
-                a.out[(size_t)(g + i) * C + c] = y * (1.0 / (1.0 + exp(-rc[i])));
+                const double y = wkv_step<double>(w, u, (double)kc[i], (double)vc[i], aa, bb, pp);
+                a.out[(size_t)(g + i) * C + c] = y * (1.0 / (1.0 + exp(-(double)rc[i])));
             }
         }
 #pragma unroll
@@ -1227,11 +1229,11 @@ int rows_quant(hipStream_t st, int64_t R, int64_t K, const double *in, const flo
 }
 
 int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, int64_t R, int64_t K, int64_t N, int op,
-                  const double *gate) {
+                  const float *gate) {
     if (K % 64 != 0) return set_error(RWKV_ERR_SIZE, "rows_products: contraction length %lld is not a multiple of 64",
                                       (long long)K);
     if (n < 1 || n > kRowsMaxProducts) return set_error(RWKV_ERR_ARG, "rows_products: %d products in one launch", n);
-    if (op < ROW_STORE || op > ROW_GATE_ADD) return set_error(RWKV_ERR_ARG, "rows_products: unknown tail %d", op);
+    if (op < ROW_STORE || op > ROW_STORE_F32) return set_error(RWKV_ERR_ARG, "rows_products: unknown tail %d", op);
     GemmArgs g;
     FinishArgs f;
     for (int m = 0; m < kRowsMaxProducts; ++m) {
@@ -1273,13 +1275,14 @@ int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, i
         case ROW_STORE: hipLaunchKernelGGL(rows_finish_kernel<ROW_STORE>, fg, fb, 0, st, f); break;
         case ROW_RELU2: hipLaunchKernelGGL(rows_finish_kernel<ROW_RELU2>, fg, fb, 0, st, f); break;
         case ROW_ADD: hipLaunchKernelGGL(rows_finish_kernel<ROW_ADD>, fg, fb, 0, st, f); break;
+        case ROW_STORE_F32: hipLaunchKernelGGL(rows_finish_kernel<ROW_STORE_F32>, fg, fb, 0, st, f); break;
         default: hipLaunchKernelGGL(rows_finish_kernel<ROW_GATE_ADD>, fg, fb, 0, st, f); break;
     }
     RWKV_CHECK_LAUNCH("rows_finish_kernel");
     return RWKV_OK;
 }
 
-int rows_wkv(hipStream_t st, int64_t R, int C, bool sequence, const double *k, const double *v, const double *r,
+int rows_wkv(hipStream_t st, int64_t R, int C, bool sequence, const float *k, const float *v, const float *r,
              const double *w, const double *u, double *state, int64_t state_stride, double *out, double *scratch) {
     WkvRowsArgs a;
     a.C = C; a.R = (int)R; a.sequence = sequence ? 1 : 0; a.k = k; a.v = v; a.r = r; a.w = w; a.u = u;
