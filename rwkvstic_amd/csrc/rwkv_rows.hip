@@ -604,7 +604,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs &a, const v4i (&acc
                     else if (a.tail == ROW_STORE_F32) reinterpret_cast<float *>(outv)[(size_t)t * a.N + col] = (float)y;
                     else if (a.tail == ROW_RELU2) { const double r = y > 0.0 ? y : 0.0; *o = r * r; }              // block.py:97
                     else if (a.tail == ROW_ADD) *o += y;                                                            // block.py:80
-                    else *o += y * (1.0 / (1.0 + exp(-(double)a.gate[(size_t)t * a.N + col])));                     // block.py:95-100
+                    else *o += y * (double)sigmoid_f32(a.gate[(size_t)t * a.N + col]);       // block.py:95-100; the gate in float32 as in the single-token kernel
                 }
                 continue;
             }
@@ -937,11 +937,14 @@ __global__ void __launch_bounds__(256) rows_finish_kernel(const FinishArgs a) {
     else if (OP == ROW_STORE_F32) reinterpret_cast<float *>(outv)[(size_t)t * a.N + j] = (float)y;
     else if (OP == ROW_RELU2) { const double r = y > 0.0 ? y : 0.0; *o = r * r; }            // block.py:97
     else if (OP == ROW_ADD) *o += y;                                                          // block.py:80
-    else if (OP == ROW_GATE_ADD) *o += y * (1.0 / (1.0 + exp(-(double)a.gate[(size_t)t * a.N + j]))); // block.py:95-100
+    else if (OP == ROW_GATE_ADD) *o += y * (double)sigmoid_f32(a.gate[(size_t)t * a.N + j]);          // block.py:95-100
 }
 
 // ---------------------------------------------------------------------------
 // WKV + receptance gate           (block.py:69-78, wkv.py:23-39, operators.cu:6-37)
+// Arithmetic of the single-token kernel: sums, exponentials and the gate in float32, the exponent pp in float64
+// (wkv_step_f32).  A float64 exponential is some fifty dependent instructions, and with one wavefront per 64
+// channels and chunk there is nothing to hide them behind: the float64 form took three times as long.
 // sequence: thread = channel, serial over the T rows; batch: thread = (row, channel).
 // ---------------------------------------------------------------------------
 struct WkvRowsArgs {
@@ -960,13 +963,14 @@ __global__ void __launch_bounds__(64) wkv_rows_kernel(const WkvRowsArgs a) {
     const double w = a.w[c], u = a.u[c];
     const int t0 = a.sequence ? 0 : blockIdx.y, t1 = a.sequence ? a.R : blockIdx.y + 1;
     double *st = a.state + (a.sequence ? 0 : (size_t)blockIdx.y * a.state_stride);
-    double aa = st[c], bb = st[C + c], pp = st[2 * C + c];
+    float aa = (float)st[c], bb = (float)st[C + c];
+    double pp = st[2 * C + c];
     for (int t = t0; t < t1; ++t) {
         const size_t i = (size_t)t * C + c;
-        const double y = wkv_step<double>(w, u, (double)a.k[i], (double)a.v[i], aa, bb, pp);
-        a.out[i] = y * (1.0 / (1.0 + exp(-(double)a.r[i])));
+        const float y = wkv_step_f32(w, u, a.k[i], a.v[i], aa, bb, pp);
+        a.out[i] = (double)(y * sigmoid_f32(a.r[i]));
     }
-    st[c] = aa; st[C + c] = bb; st[2 * C + c] = pp;
+    st[c] = (double)aa; st[C + c] = (double)bb; st[2 * C + c] = pp;
 }
 
 
@@ -987,7 +991,8 @@ __global__ void __launch_bounds__(64) wkv_chunk_local_kernel(const WkvRowsArgs a
     const int C = a.C;
     const double w = a.w[c], u = a.u[c];
     const int t0 = j * kWkvChunk, t1 = min(t0 + kWkvChunk, a.R);
-    double aa = 0.0, bb = 0.0, pp = -1e30;
+    float aa = 0.f, bb = 0.f;
+    double pp = -1e30;
     float kc[kWkvGroup], vc[kWkvGroup], kn[kWkvGroup], vn[kWkvGroup];
 #pragma unroll
     for (int i = 0; i < kWkvGroup; ++i) {
@@ -1002,12 +1007,12 @@ __global__ void __launch_bounds__(64) wkv_chunk_local_kernel(const WkvRowsArgs a
         }
 #pragma unroll
         for (int i = 0; i < kWkvGroup; ++i)
-            if (g + i < t1) (void)wkv_step<double>(w, u, (double)kc[i], (double)vc[i], aa, bb, pp);
+            if (g + i < t1) (void)wkv_step_f32(w, u, kc[i], vc[i], aa, bb, pp);
 #pragma unroll
         for (int i = 0; i < kWkvGroup; ++i) { kc[i] = kn[i]; vc[i] = vn[i]; }
     }
     double *o = scr + (size_t)j * 3 * C;
-    o[c] = aa; o[C + c] = bb; o[2 * C + c] = pp;
+    o[c] = (double)aa; o[C + c] = (double)bb; o[2 * C + c] = pp;
 }
 
 __global__ void __launch_bounds__(64) wkv_chunk_prefix_kernel(const WkvRowsArgs a, double *scr, int n_chunks) {
@@ -1037,7 +1042,7 @@ __global__ void __launch_bounds__(64) wkv_chunk_prefix_kernel(const WkvRowsArgs 
                 const int n = min(kWkvChunk, a.R - j * kWkvChunk);
                 const double s = pp + (double)n * w;
                 const double p = fmax(s, lp[i]);
-                const double f1 = exp(s - p), f2 = exp(lp[i] - p);
+                const double f1 = (double)expf((float)(s - p)), f2 = (double)expf((float)(lp[i] - p));   // (one of them is e^0)
                 aa = f1 * aa + f2 * la[i];
                 bb = f1 * bb + f2 * lb[i];
                 pp = p;
@@ -1056,7 +1061,8 @@ __global__ void __launch_bounds__(64) wkv_chunk_replay_kernel(const WkvRowsArgs 
     const double w = a.w[c], u = a.u[c];
     const int t0 = j * kWkvChunk, t1 = min(t0 + kWkvChunk, a.R);
     const double *in = scr + (size_t)j * 3 * C;
-    double aa = in[c], bb = in[C + c], pp = in[2 * C + c];
+    float aa = (float)in[c], bb = (float)in[C + c];
+    double pp = in[2 * C + c];
     float kc[kWkvGroup], vc[kWkvGroup], rc[kWkvGroup], kn[kWkvGroup], vn[kWkvGroup], rn[kWkvGroup];
 #pragma unroll
     for (int i = 0; i < kWkvGroup; ++i) {
@@ -1072,8 +1078,8 @@ __global__ void __launch_bounds__(64) wkv_chunk_replay_kernel(const WkvRowsArgs 
 #pragma unroll
         for (int i = 0; i < kWkvGroup; ++i) {
             if (g + i < t1) {
-                const double y = wkv_step<double>(w, u, (double)kc[i], (double)vc[i], aa, bb, pp);
-                a.out[(size_t)(g + i) * C + c] = y * (1.0 / (1.0 + exp(-(double)rc[i])));
+                const float y = wkv_step_f32(w, u, kc[i], vc[i], aa, bb, pp);
+                a.out[(size_t)(g + i) * C + c] = (double)(y * sigmoid_f32(rc[i]));
             }
         }
 #pragma unroll
