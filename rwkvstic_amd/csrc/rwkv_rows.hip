@@ -107,9 +107,26 @@ __device__ __forceinline__ double emit_quad(const float (&x4)[4], double invS, i
                             __builtin_amdgcn_perm(y0, x0, 0x07060302u), __builtin_amdgcn_perm(y0, x0, 0x05040100u)};
     const int mt = t >> 2, m0 = (t & 3) * 4;
     const int kb = c0 >> 6, g = (c0 & 63) >> 4, j = (c0 & 15) >> 2;
-    signed char *frag = dig + ((size_t)mt * KB + kb) * 1024 + (16 * g + m0) * 16 + 4 * j;
-#pragma unroll
-    for (int d = 0; d < 4; ++d) *reinterpret_cast<unsigned *>(frag + d * 16) = pl[d];
+    // The four lanes j = 0..3 that hold the 16 channels of one fragment slot transpose their 4 x 4 dwords
+    // (two exchanges, with the neighbour and with the lane two further): lane j ends up with digit plane j of all 16
+    // channels and writes it with ONE 16-byte store; the four lanes together fill a whole 64-byte line.  (Four
+    // 4-byte stores per lane into four different lines cost the quantisers a third of their time.)  Callers
+    // guarantee whole groups of four lanes: c0 = 4 * (a multiple-of-4-aligned lane index), widths multiples of 16.
+    unsigned a4[4] = {pl[0], pl[1], pl[2], pl[3]};
+    {
+        const bool odd = j & 1;
+        const unsigned s0 = odd ? a4[0] : a4[1], s1 = odd ? a4[2] : a4[3];
+        const unsigned r0 = (unsigned)__builtin_amdgcn_update_dpp(0, (int)s0, 0xB1, 0xf, 0xf, false);
+        const unsigned r1 = (unsigned)__builtin_amdgcn_update_dpp(0, (int)s1, 0xB1, 0xf, 0xf, false);
+        if (odd) { a4[0] = r0; a4[2] = r1; } else { a4[1] = r0; a4[3] = r1; }
+        const bool hi = j & 2;
+        const unsigned t0 = hi ? a4[0] : a4[2], t1 = hi ? a4[1] : a4[3];
+        const unsigned q0 = (unsigned)__builtin_amdgcn_update_dpp(0, (int)t0, 0x4E, 0xf, 0xf, false);
+        const unsigned q1 = (unsigned)__builtin_amdgcn_update_dpp(0, (int)t1, 0x4E, 0xf, 0xf, false);
+        if (hi) { a4[0] = q0; a4[1] = q1; } else { a4[2] = q0; a4[3] = q1; }
+    }
+    signed char *slot = dig + ((size_t)mt * KB + kb) * 1024 + (16 * g + m0 + j) * 16;
+    *reinterpret_cast<uint4 *>(slot) = make_uint4(a4[0], a4[1], a4[2], a4[3]);
     return qsum;
 }
 
@@ -1217,7 +1234,7 @@ int rows_quant(hipStream_t st, int64_t R, int64_t K, const double *in, const flo
     const dim3 grid((unsigned)R), block(kRT);
     if (scratch && quant_uses_parts(R, K)) {
         QuantPartArgs pa;
-        pa.q = q; pa.G = (int)ceil_div(K, 4 * kRT * kQuantPartSeg); pa.quads_per_part = (int)ceil_div(K / 4, pa.G);
+        pa.q = q; pa.G = (int)ceil_div(K, 4 * kRT * kQuantPartSeg); pa.quads_per_part = (int)round_up(ceil_div(K / 4, pa.G), 4);    // whole groups of 16 values: four lanes share a fragment slot
         pa.part = scratch;
         const dim3 pg((unsigned)pa.G, (unsigned)R);
         hipLaunchKernelGGL(rows_quant_part_kernel<false>, pg, block, 0, st, pa);
