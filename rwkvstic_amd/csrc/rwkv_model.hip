@@ -607,8 +607,8 @@ int rows_layers(rwkv_model *m, hipStream_t st, const int64_t *tokens, int64_t R,
         for (int i = 0; i < 3; ++i) { pk[i].a = w.q[i]; pk[i].w16 = kvr[i]->packed16; pk[i].out = reinterpret_cast<double *>(kvr32 + i * RC); }
         RWKV_TRY(rows_products(st, 3, pk, w.tot, R, C, C, ROW_STORE_F32, nullptr));
         RWKV_TRY(rows_wkv(st, R, C, sequence, kvr32, kvr32 + RC, kvr32 + 2 * RC, L.time_decay, L.time_first,
-                          sl + 2 * (size_t)C, state_stride, w.att, w.wkv_scr));
-        RWKV_TRY(rows_quant(st, R, C, w.att, L.att_o.range, L.att_o.offset, w.q[0], (double *)w.tot));
+                          sl + 2 * (size_t)C, state_stride, reinterpret_cast<float *>(w.att), w.wkv_scr));
+        RWKV_TRY(rows_quant(st, R, C, w.att, true, L.att_o.range, L.att_o.offset, w.q[0], (double *)w.tot));    // att and h: float32 arrays
         const RowsProduct po = {w.q[0], L.att_o.packed16, w.x};
         RWKV_TRY(rows_products(st, 1, &po, w.tot, R, C, C, ROW_ADD, nullptr));
         // ChannelMix (block.py:82-100)
@@ -620,7 +620,7 @@ int rows_layers(rwkv_model *m, hipStream_t st, const int64_t *tokens, int64_t R,
         const RowsProduct pfk = {w.q[1], L.ffn_k.packed16, w.h}, pfr = {w.q[2], L.ffn_r.packed16, w.kvr};
         RWKV_TRY(rows_products(st, 1, &pfk, w.tot, R, C, F, ROW_RELU2, nullptr));
         RWKV_TRY(rows_products(st, 1, &pfr, w.tot, R, C, C, ROW_STORE_F32, nullptr));
-        RWKV_TRY(rows_quant(st, R, F, w.h, L.ffn_v.range, L.ffn_v.offset, w.q[0], (double *)w.tot));
+        RWKV_TRY(rows_quant(st, R, F, w.h, true, L.ffn_v.range, L.ffn_v.offset, w.q[0], (double *)w.tot));
         const RowsProduct pfv = {w.q[0], L.ffn_v.packed16, w.x};
         RWKV_TRY(rows_products(st, 1, &pfv, w.tot, R, F, C, ROW_GATE_ADD, kvr32));
     }
@@ -877,7 +877,7 @@ int rwkv_gemm8(rwkv_stream_t stream, int64_t T, int64_t n_in, int64_t n_out, con
     q.zp = (double *)p; p += round_up((size_t)T * 8, 256);
     q.dig = (signed char *)p; p += round_up(rows_dig_bytes(T, n_in), 256);
     const hipStream_t st = (hipStream_t)stream;
-    const int rc = rows_quant(st, T, n_in, x, range, offset, q, (double *)p);
+    const int rc = rows_quant(st, T, n_in, x, false, range, offset, q, (double *)p);
     if (rc) return rc;
     const RowsProduct pr = {q, packed16, y};
     return rows_products(st, 1, &pr, (long long *)p, T, n_in, n_out, ROW_STORE, nullptr);

@@ -7,6 +7,7 @@ namespace rwkv {
 
 // ROW_STORE_F32: the product's `out` points at a float32 [R, N] array (k, v, r and the ffn receptance: their consumers
 // round them to float32 anyway, as the single-token kernel does, and the arrays are read several times)
+// ROW_RELU2 also stores float32 (its only consumer, the row quantiser, scales the values to float32 next).
 enum RowTail { ROW_STORE = 0, ROW_RELU2 = 1, ROW_ADD = 2, ROW_GATE_ADD = 3, ROW_STORE_F32 = 4 };
 
 // One quantised left operand of a product: R rows rewritten as fixed-point digit fragments plus the
@@ -40,14 +41,14 @@ int rows_ln_mix_quant(hipStream_t st, int n_mix, int64_t R, int C, bool sequence
                       const RowsOperand *out);
 // Rows of float64 values quantised for a matrix with the given per-input-channel range / offset.
 // scratch: rows_quant_scratch_bytes(R, K) bytes (any buffer free until the product starts, e.g. its totals), or null.
-int rows_quant(hipStream_t st, int64_t R, int64_t K, const double *in, const float *range, const double *offset,
+int rows_quant(hipStream_t st, int64_t R, int64_t K, const void *in, bool in_f32, const float *range, const double *offset,
                const RowsOperand &out, double *scratch);
 // n (<= kRowsMaxProducts) products of the same shape [R, K] x [K, N] and tail in one launch;
 // tot: n * rows_tot_bytes(R, N) bytes of scratch.
 int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, int64_t R, int64_t K, int64_t N, int op,
                   const float *gate);
 int rows_wkv(hipStream_t st, int64_t R, int C, bool sequence, const float *k, const float *v, const float *r,
-             const double *w, const double *u, double *state, int64_t state_stride, double *out,
+             const double *w, const double *u, double *state, int64_t state_stride, float *out,
              double *scratch /* rows_wkv_scratch_bytes(R, C), or null: serial over the rows */);
 
 }  // namespace rwkv

@@ -326,21 +326,30 @@ __global__ void __launch_bounds__(kLT) rows_ln_mix_quant_kernel(const LnQuantArg
 // ---------------------------------------------------------------------------
 struct QuantArgs {
     int K;                      // contraction length, multiple of 64
-    const double *in;           // [R, K]
+    const void *in;             // [R, K] float64, or float32 (the kernels' TIn): what the WKV kernels and the relu^2 tail write
     const float *range;         // [K]
     const double *offset;       // [K]
     signed char *dig;           // fragments [ceil(R/4)][K/64][1024]
     double *S, *qs, *zp;        // [R]
 };
 
+// Two / four consecutive values of a float64 or float32 row as float64.
+__device__ __forceinline__ double2 row_ld2(const double *p) { return *reinterpret_cast<const double2 *>(p); }
+__device__ __forceinline__ double2 row_ld2(const float *p) { const float2 f = *reinterpret_cast<const float2 *>(p); return make_double2((double)f.x, (double)f.y); }
+__device__ __forceinline__ void row_ld4(const double *p, double2 &a, double2 &b) { a = row_ld2(p); b = row_ld2(p + 2); }
+__device__ __forceinline__ void row_ld4(const float *p, double2 &a, double2 &b) {
+    const float4 f = *reinterpret_cast<const float4 *>(p);
+    a = make_double2((double)f.x, (double)f.y); b = make_double2((double)f.z, (double)f.w);
+}
+
 // kQuantSeg: 16-element segments a thread keeps in registers (rows up to 16 * kRT * kQuantSeg long in one
 // read): 3 covers 12288 with registers to spare for four workgroups per compute unit, 5 covers 20480.
-template <int kQuantSeg>
+template <int kQuantSeg, typename TIn>
 __global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
     __shared__ double red[2 * kRW];
     __shared__ float redf[kRW];
     const int t = blockIdx.x, K = a.K;
-    const double *row = a.in + (size_t)t * K;
+    const TIn *row = static_cast<const TIn *>(a.in) + (size_t)t * K;
     // The thread that will write a 16-element group of digits reads it once: xs stays in registers
     // between the pass that finds the row's scale and the pass that forms the digits (longer rows
     // fall back to a second read).
@@ -355,7 +364,7 @@ __global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
             if (c0 < K) {
 #pragma unroll
                 for (int i = 0; i < 16; i += 2) {
-                    const double2 v = *reinterpret_cast<const double2 *>(row + c0 + i);
+                    const double2 v = row_ld2(row + c0 + i);
                     const float2 r = *reinterpret_cast<const float2 *>(a.range + c0 + i);
                     const double2 o = *reinterpret_cast<const double2 *>(a.offset + c0 + i);
                     xs[s][i] = (float)(v.x * (double)r.x);
@@ -368,7 +377,7 @@ __global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
         }
     } else {
         for (int c = threadIdx.x; c < K; c += kRT) {
-            const double v = row[c];
+            const double v = (double)row[c];
             amax = fmaxf(amax, fabsf((float)(v * (double)a.range[c])));
             z[0] += v * a.offset[c];
         }
@@ -419,7 +428,7 @@ __global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
         for (int c0 = threadIdx.x * 16; c0 < K; c0 += kRT * 16) {
             float x16[16];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) x16[i] = (float)(row[c0 + i] * (double)a.range[c0 + i]);
+            for (int i = 0; i < 16; ++i) x16[i] = (float)((double)row[c0 + i] * (double)a.range[c0 + i]);
             emit(c0, x16);
         }
     }
@@ -429,12 +438,12 @@ __global__ void __launch_bounds__(kRT) rows_quant_kernel(const QuantArgs a) {
 
 // The same quantiser with a thread owning groups of four values (NSEG of them, 4 * kRT * NSEG values per row in
 // one read): every thread of the workgroup has work whatever the row length, and few registers are held.
-template <int NSEG>
+template <int NSEG, typename TIn>
 __global__ void __launch_bounds__(kRT) rows_quant4_kernel(const QuantArgs a) {
     __shared__ double red[2 * kRW];
     __shared__ float redf[kRW];
     const int t = blockIdx.x, K = a.K, tid = threadIdx.x;
-    const double *row = a.in + (size_t)t * K;
+    const TIn *row = static_cast<const TIn *>(a.in) + (size_t)t * K;
     float xs[NSEG][4];
     float amax = 0.f;
     double z[1] = {0.0};
@@ -442,7 +451,8 @@ __global__ void __launch_bounds__(kRT) rows_quant4_kernel(const QuantArgs a) {
     for (int g = 0; g < NSEG; ++g) {
         const int c0 = 4 * (tid + g * kRT);
         if (c0 < K) {
-            const double2 v0 = *reinterpret_cast<const double2 *>(row + c0), v1 = *reinterpret_cast<const double2 *>(row + c0 + 2);
+            double2 v0, v1;
+            row_ld4(row + c0, v0, v1);
             const float4 r = *reinterpret_cast<const float4 *>(a.range + c0);
             const double2 o0 = *reinterpret_cast<const double2 *>(a.offset + c0), o1 = *reinterpret_cast<const double2 *>(a.offset + c0 + 2);
             xs[g][0] = (float)(v0.x * (double)r.x); xs[g][1] = (float)(v0.y * (double)r.y);
@@ -483,12 +493,12 @@ struct QuantPartArgs {
     double *part;               // [R][G][2]: max |xs|, zero-point share
 };
 
-template <bool EMIT>
+template <bool EMIT, typename TIn>
 __global__ void __launch_bounds__(kRT) rows_quant_part_kernel(const QuantPartArgs a) {
     __shared__ double red[2 * kRW];
     __shared__ float redf[kRW];
     const int g = blockIdx.x, t = blockIdx.y, K = a.q.K, tid = threadIdx.x;
-    const double *row = a.q.in + (size_t)t * K;
+    const TIn *row = static_cast<const TIn *>(a.q.in) + (size_t)t * K;
     const int q0 = g * a.quads_per_part, q1 = min(q0 + a.quads_per_part, K >> 2);
     float xs[kQuantPartSeg][4];
     float amax = 0.f;
@@ -498,7 +508,8 @@ __global__ void __launch_bounds__(kRT) rows_quant_part_kernel(const QuantPartArg
         const int qi = q0 + tid + s * kRT;
         if (qi < q1) {
             const int c0 = 4 * qi;
-            const double2 v0 = *reinterpret_cast<const double2 *>(row + c0), v1 = *reinterpret_cast<const double2 *>(row + c0 + 2);
+            double2 v0, v1;
+            row_ld4(row + c0, v0, v1);
             const float4 r = *reinterpret_cast<const float4 *>(a.q.range + c0);
             xs[s][0] = (float)(v0.x * (double)r.x); xs[s][1] = (float)(v0.y * (double)r.y);
             xs[s][2] = (float)(v1.x * (double)r.z); xs[s][3] = (float)(v1.y * (double)r.w);
@@ -619,7 +630,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs &a, const v4i (&acc
                     double *o = outv + (size_t)t * a.N + col;
                     if (a.tail == ROW_STORE) *o = y;
                     else if (a.tail == ROW_STORE_F32) reinterpret_cast<float *>(outv)[(size_t)t * a.N + col] = (float)y;
-                    else if (a.tail == ROW_RELU2) { const double r = y > 0.0 ? y : 0.0; *o = r * r; }              // block.py:97
+                    else if (a.tail == ROW_RELU2) {                                                                 // block.py:97, kept as float32 (see RowTail)
+                        const double r = y > 0.0 ? y : 0.0;
+                        reinterpret_cast<float *>(outv)[(size_t)t * a.N + col] = (float)(r * r);
+                    }
                     else if (a.tail == ROW_ADD) *o += y;                                                            // block.py:80
                     else *o += y * (double)sigmoid_f32(a.gate[(size_t)t * a.N + col]);       // block.py:95-100; the gate in float32 as in the single-token kernel
                 }
@@ -952,7 +966,7 @@ __global__ void __launch_bounds__(256) rows_finish_kernel(const FinishArgs a) {
     double *o = outv + (size_t)t * a.N + j;
     if (OP == ROW_STORE) *o = y;
     else if (OP == ROW_STORE_F32) reinterpret_cast<float *>(outv)[(size_t)t * a.N + j] = (float)y;
-    else if (OP == ROW_RELU2) { const double r = y > 0.0 ? y : 0.0; *o = r * r; }            // block.py:97
+    else if (OP == ROW_RELU2) { const double r = y > 0.0 ? y : 0.0; reinterpret_cast<float *>(outv)[(size_t)t * a.N + j] = (float)(r * r); }   // block.py:97
     else if (OP == ROW_ADD) *o += y;                                                          // block.py:80
     else if (OP == ROW_GATE_ADD) *o += y * (double)sigmoid_f32(a.gate[(size_t)t * a.N + j]);          // block.py:95-100
 }
@@ -970,7 +984,7 @@ struct WkvRowsArgs {
     const double *w, *u;        // [C]  (w = -exp(time_decay))
     double *state;              // rows aa, bb, pp of the layer: state + 2C; batch: + row * state_stride
     int64_t state_stride;
-    double *out;                // [R, C]  wkv * sigmoid(r)
+    float *out;                 // [R, C]  wkv * sigmoid(r): a float32 product
 };
 
 __global__ void __launch_bounds__(64) wkv_rows_kernel(const WkvRowsArgs a) {
@@ -985,7 +999,7 @@ __global__ void __launch_bounds__(64) wkv_rows_kernel(const WkvRowsArgs a) {
     for (int t = t0; t < t1; ++t) {
         const size_t i = (size_t)t * C + c;
         const float y = wkv_step_f32(w, u, a.k[i], a.v[i], aa, bb, pp);
-        a.out[i] = (double)(y * sigmoid_f32(a.r[i]));
+        a.out[i] = y * sigmoid_f32(a.r[i]);
     }
     st[c] = (double)aa; st[C + c] = (double)bb; st[2 * C + c] = pp;
 }
@@ -1096,7 +1110,7 @@ __global__ void __launch_bounds__(64) wkv_chunk_replay_kernel(const WkvRowsArgs 
         for (int i = 0; i < kWkvGroup; ++i) {
             if (g + i < t1) {
                 const float y = wkv_step_f32(w, u, kc[i], vc[i], aa, bb, pp);
-                a.out[(size_t)(g + i) * C + c] = (double)(y * sigmoid_f32(rc[i]));
+                a.out[(size_t)(g + i) * C + c] = y * sigmoid_f32(rc[i]);
             }
         }
 #pragma unroll
@@ -1225,7 +1239,7 @@ int rows_ln_mix_quant(hipStream_t st, int n_mix, int64_t R, int C, bool sequence
     return RWKV_OK;
 }
 
-int rows_quant(hipStream_t st, int64_t R, int64_t K, const double *in, const float *range, const double *offset,
+int rows_quant(hipStream_t st, int64_t R, int64_t K, const void *in, bool in_f32, const float *range, const double *offset,
                const RowsOperand &out, double *scratch) {
     if (K % 64 != 0) return set_error(RWKV_ERR_SIZE, "rows_quant: contraction length %lld is not a multiple of 64",
                                       (long long)K);
@@ -1237,16 +1251,27 @@ int rows_quant(hipStream_t st, int64_t R, int64_t K, const double *in, const flo
         pa.q = q; pa.G = (int)ceil_div(K, 4 * kRT * kQuantPartSeg); pa.quads_per_part = (int)round_up(ceil_div(K / 4, pa.G), 4);    // whole groups of 16 values: four lanes share a fragment slot
         pa.part = scratch;
         const dim3 pg((unsigned)pa.G, (unsigned)R);
-        hipLaunchKernelGGL(rows_quant_part_kernel<false>, pg, block, 0, st, pa);
-        hipLaunchKernelGGL(rows_quant_part_kernel<true>, pg, block, 0, st, pa);
+        if (in_f32) {
+            hipLaunchKernelGGL((rows_quant_part_kernel<false, float>), pg, block, 0, st, pa);
+            hipLaunchKernelGGL((rows_quant_part_kernel<true, float>), pg, block, 0, st, pa);
+        } else {
+            hipLaunchKernelGGL((rows_quant_part_kernel<false, double>), pg, block, 0, st, pa);
+            hipLaunchKernelGGL((rows_quant_part_kernel<true, double>), pg, block, 0, st, pa);
+        }
         RWKV_CHECK_LAUNCH("rows_quant_part_kernel");
         return RWKV_OK;
     }
-    if (K <= 3 * 4 * kRT) hipLaunchKernelGGL(rows_quant4_kernel<3>, grid, block, 0, st, q);
-    else if (K <= 6 * 4 * kRT) hipLaunchKernelGGL(rows_quant4_kernel<6>, grid, block, 0, st, q);
-    else if (K <= 10 * 4 * kRT) hipLaunchKernelGGL(rows_quant4_kernel<10>, grid, block, 0, st, q);
-    else if (K <= 20 * 4 * kRT) hipLaunchKernelGGL(rows_quant4_kernel<20>, grid, block, 0, st, q);
-    else hipLaunchKernelGGL(rows_quant_kernel<3>, grid, block, 0, st, q);      // any length: a second read past 12288
+#define RWKV_QUANT_LAUNCH(T)                                                                          \
+    do {                                                                                              \
+        if (K <= 3 * 4 * kRT) hipLaunchKernelGGL((rows_quant4_kernel<3, T>), grid, block, 0, st, q);          \
+        else if (K <= 6 * 4 * kRT) hipLaunchKernelGGL((rows_quant4_kernel<6, T>), grid, block, 0, st, q);     \
+        else if (K <= 10 * 4 * kRT) hipLaunchKernelGGL((rows_quant4_kernel<10, T>), grid, block, 0, st, q);   \
+        else if (K <= 20 * 4 * kRT) hipLaunchKernelGGL((rows_quant4_kernel<20, T>), grid, block, 0, st, q);   \
+        else hipLaunchKernelGGL((rows_quant_kernel<3, T>), grid, block, 0, st, q);      /* any length: a second read past 12288 */ \
+    } while (0)
+    if (in_f32) RWKV_QUANT_LAUNCH(float);
+    else RWKV_QUANT_LAUNCH(double);
+#undef RWKV_QUANT_LAUNCH
     RWKV_CHECK_LAUNCH("rows_quant_kernel");
     return RWKV_OK;
 }
@@ -1306,7 +1331,7 @@ int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, i
 }
 
 int rows_wkv(hipStream_t st, int64_t R, int C, bool sequence, const float *k, const float *v, const float *r,
-             const double *w, const double *u, double *state, int64_t state_stride, double *out, double *scratch) {
+             const double *w, const double *u, double *state, int64_t state_stride, float *out, double *scratch) {
     WkvRowsArgs a;
     a.C = C; a.R = (int)R; a.sequence = sequence ? 1 : 0; a.k = k; a.v = v; a.r = r; a.w = w; a.u = u;
     a.state = state; a.state_stride = state_stride; a.out = out;
