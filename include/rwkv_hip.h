@@ -215,8 +215,15 @@ typedef struct rwkv_model rwkv_model;
  * This is the one entry point that allocates device memory: one block with the
  * tables of the single-token kernel (packed per-layer constants, column sums,
  * 4 KiB of owner record and 128 bytes of job pointers per layer and
- * 16-channel tile, the exchange vectors); rwkv_model_destroy frees it.  One
- * forward call may be in flight per handle at a time. */
+ * 16-channel tile), which rwkv_model_destroy frees, and the kernel's exchange
+ * vectors, taken from a process-wide pool of uncached device memory that
+ * later handles reuse and that is never returned to the driver.
+ * One forward call may be in flight per handle at a time, on one stream; while
+ * a single-token step runs, that stream must have the device to itself: the
+ * workgroups of the persistent kernel (n_embd / 16, or n_embd / 32 at
+ * n_embd = 5120) wait for each other and must all be resident.  A step that
+ * cannot make progress gives up after a bounded wait and is reported by
+ * rwkv_model_check; it never hangs. */
 int rwkv_model_create(const rwkv_model_desc *desc, rwkv_model **out);
 void rwkv_model_destroy(rwkv_model *m);
 
@@ -227,12 +234,14 @@ int rwkv_model_has_fused_step(const rwkv_model *m);
 /* Diagnostics: when device_buffer is non-NULL, every workgroup g of every
  * following single-token launch writes 100 MHz wall-clock stamps of its phase
  * boundaries into device_buffer[g][layer][24], which must hold
- * (n_embd / 16) * n_layer * 24 int64 values; NULL switches it off. */
+ * (n_embd / 16) * n_layer * 24 int64 values (n_embd / 32 workgroups write at
+ * n_embd = 5120); NULL switches it off. */
 int rwkv_model_set_trace(rwkv_model *m, int64_t *device_buffer);
 
 /* Synchronises the device and returns RWKV_ERR_HIP if a single-token launch
- * gave up waiting for another workgroup (it then left logits/state
- * incomplete), else RWKV_OK.  For tests and diagnostics. */
+ * since the previous check gave up waiting for another workgroup (logits and
+ * state written since then are invalid), else RWKV_OK.  The condition is
+ * reported once: the flag is cleared, later steps run normally. */
 int rwkv_model_check(rwkv_model *m);
 
 /* Measurement aid (no counterpart in the reference): feeds the token at *token
