@@ -257,6 +257,7 @@ def test_pack_m16_round_trip(ops):
 @pytest.mark.parametrize("T,K,N", [(1, 64, 16), (5, 256, 100), (64, 2560, 2560), (130, 2560, 10240),
                                    (33, 10240, 2560), (8, 2560, 50277), (1000, 192, 2560), (1024, 320, 2500),
                                    (3, 20544, 32),      # a few long rows: the two-launch quantiser
+                                   (4, 8320, 48),       # the same with parts that have to be rounded up to whole groups of 16 values
                                    (9, 20544, 32),      # rows too long for the register-resident quantiser
                                    (20, 2560, 2560), (32, 640, 5000)])   # 9..32 rows: the few-row variant with LDS staging
 def test_gemm8_matches_fp64_dense(ops, T, K, N):
