@@ -762,6 +762,8 @@ int rwkv_model_time_token_kernel(rwkv_model *m, rwkv_stream_t stream, const int6
                                  int n, float *avg_us) {
     RWKV_CHECK_ARG(m && token && state && logits && avg_us, "rwkv_model_time_token_kernel: null pointer");
     RWKV_CHECK_ARG(n > 0 && n <= 4096, "rwkv_model_time_token_kernel: n must be in 1..4096");
+    if (reinterpret_cast<uintptr_t>(token) % 8 || reinterpret_cast<uintptr_t>(state) % 8 || reinterpret_cast<uintptr_t>(logits) % 8)
+        return set_error(RWKV_ERR_ALIGN, "rwkv_model_time_token_kernel: token, state and logits need 8-byte alignment");
     if (!m->fused) return set_error(RWKV_ERR_SIZE, "rwkv_model_time_token_kernel: this model does not run the persistent kernel");
     const hipStream_t st = (hipStream_t)stream;
     std::vector<hipEvent_t> ev((size_t)2 * n, nullptr);
@@ -788,6 +790,8 @@ int rwkv_model_time_token_kernel(rwkv_model *m, rwkv_stream_t stream, const int6
 
 int rwkv_model_selftest_timeout(rwkv_model *m, rwkv_stream_t stream, double *state, double *logits) {
     RWKV_CHECK_ARG(m && state && logits, "rwkv_model_selftest_timeout: null pointer");
+    if (reinterpret_cast<uintptr_t>(state) % 8 || reinterpret_cast<uintptr_t>(logits) % 8)
+        return set_error(RWKV_ERR_ALIGN, "rwkv_model_selftest_timeout: state and logits need 8-byte alignment");
     if (!m->fused) return set_error(RWKV_ERR_SIZE, "rwkv_model_selftest_timeout: this model does not run the persistent kernel");
     RWKV_TRY(fused_epochs(m, (hipStream_t)stream, 1));
     const int rc = decode_launch_unfed((hipStream_t)stream, m->dm, m->db, m->epoch, state, logits, 256u);
