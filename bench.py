@@ -26,7 +26,7 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E vendor peak
 # both scaled by a 1 GiB device copy in the same run; profiles/decode_kernel_3B_b1_hbm_traffic.md): a measured
 # constant per shape, not something this script can read live.  It is tied to the kernel sources it was measured on
 # by their digest (csrc_digest() below): with any other sources the bench reports null instead of a stale figure.
-PMC_TRAFFIC = {"3B": {"bytes": 2_965_400_000, "csrc_digest": "e1258757ee341066"}}
+PMC_TRAFFIC = {"3B": {"bytes": 2_965_300_000, "csrc_digest": "5714cff758c70fe3"}}
 
 
 def csrc_digest() -> str:
