@@ -41,11 +41,14 @@ def csrc_digest() -> str:
     return h.hexdigest()[:16]
 
 
+kCpuTokens = 12     # timed decode tokens of the CPU leg: about 10 s at the 3B shape on 16 host threads
+
+
 def cpu_baseline(shape, threads: int, layers_timed: int):
     """The CPU oracle (the reference's torch CPU path restated: float32 matmul on a per-call uint8 -> float32 cast,
     float64 element-wise, Python WKV step) on this box's host cores, decoding at batch 1 on a bounded sample:
-    `layers_timed` of the shape's layers (0 = all) + embedding + head, 1 untimed and 3 timed tokens; the layer time
-    is scaled to the full depth.  The matrices are drawn directly as codes (oracle QMat.synthetic): the cost of the
+    `layers_timed` of the shape's layers (0 = all, the default) + embedding + head, 1 untimed and `kCpuTokens` timed
+    tokens; with fewer layers the layer time is scaled to the full depth.  The matrices are drawn directly as codes (oracle QMat.synthetic): the cost of the
     path does not depend on their values and running the quantiser over the model would take longer than the
     sample itself."""
     import torch
@@ -56,7 +59,7 @@ def cpu_baseline(shape, threads: int, layers_timed: int):
     Ls = L if layers_timed <= 0 else min(layers_timed, L)
     m = O.OracleModel.synthetic(Ls, C, F, V, seed=1)
     state = m.emptyState.clone()
-    toks = synth.random_tokens(4, V=V, seed=2).tolist()
+    toks = synth.random_tokens(1 + kCpuTokens, V=V, seed=2).tolist()
     m.forward([toks[0]], state)                       # warm-up
     t_layers = t_rest = 0.0
     n = 0
@@ -278,8 +281,8 @@ def main() -> int:
                          "64-token random prompt, decoded greedily one batch step at a time (the 14B configuration's "
                          "batch-32 decode); prints its own JSON line")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-baseline-layers", type=int, default=8,
-                    help="layers of the shape the CPU baseline times (0 = all of them; the rest is scaled)")
+    ap.add_argument("--cpu-baseline-layers", type=int, default=0,
+                    help="layers of the shape the CPU baseline times (0 = all of them, the default; fewer: scaled to the full depth)")
     ap.add_argument("--no-isolated", action="store_true", help="skip the isolated matvec / WKV measurements")
     ap.add_argument("--isolated-only", action="store_true",
                     help="only the isolated matvec and WKV kernels (for profiling them on their own)")
