@@ -26,18 +26,21 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E vendor peak
 # both scaled by a 1 GiB device copy in the same run; profiles/decode_kernel_3B_b1_hbm_traffic.md): a measured
 # constant per shape, not something this script can read live.  It is tied to the kernel sources it was measured on
 # by their digest (csrc_digest() below): with any other sources the bench reports null instead of a stale figure.
-PMC_TRAFFIC = {"3B": {"bytes": 2_965_300_000, "csrc_digest": "5714cff758c70fe3"}}
+PMC_TRAFFIC = {"3B": {"bytes": 2_965_300_000, "csrc_digest": "0dc82f02332f326f"}}
+
+
+DECODE_SOURCES = ("gen_decode_back.py", "rwkv_common.h", "rwkv_decode.h", "rwkv_decode.hip", "rwkv_decode_back.inc")
 
 
 def csrc_digest() -> str:
-    """sha256 over the kernel sources of the library, in name order (what `traffic` was measured on)."""
+    """sha256 over the sources of the single-token kernel (what `traffic` was measured on): the kernel, its
+    generated weight-streaming program and the generator, and the common header they include."""
     import hashlib
     d = os.path.join(ROOT, "rwkvstic_amd", "csrc")
     h = hashlib.sha256()
-    for name in sorted(os.listdir(d)):
-        if name.endswith((".hip", ".h", ".inc", ".py")):
-            h.update(name.encode())
-            h.update(open(os.path.join(d, name), "rb").read())
+    for name in DECODE_SOURCES:
+        h.update(name.encode())
+        h.update(open(os.path.join(d, name), "rb").read())
     return h.hexdigest()[:16]
 
 
