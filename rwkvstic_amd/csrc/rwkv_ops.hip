@@ -128,6 +128,94 @@ wkv_f32_kernel(int B, int T, int C, const float *__restrict__ w, const float *__
     aa[idx] = a; bb[idx] = bsum; pp[idx] = (float)p;
 }
 
+// Long sequences: the same recurrence as a two-pass scan inside one workgroup.  The recurrence is linear in
+// (aa, bb), so the T steps split into kWkvScanChunks chunks: (1) every chunk scans its steps from an empty
+// state, (2) its incoming state is the call's state joined with the contributions of the chunks before it
+// (a chunk of n steps decays what came in by e^{n w}), (3) it replays its steps from there and writes y.  A
+// thread's serial chain is 2 T / kWkvScanChunks steps instead of T, there are five wavefronts per SIMD instead
+// of a third of one, and k and v are read twice (the second time mostly out of the memory-side cache).
+// Workgroup = 32 channels of one sequence; lane = (chunk parity, channel), wavefront w holds chunks 2w, 2w + 1.
+constexpr int kWkvScanWaves = 8, kWkvScanChunks = 2 * kWkvScanWaves, kWkvScanGroup = 8;
+constexpr int kWkvScanMinT = 256;       // shorter sequences stay with the serial kernel
+
+__device__ __forceinline__ void wkv_scan_join(double w, int n, double la, double lb, double lp, double &aa, double &bb, double &pp) {
+    const double s = pp + (double)n * w;
+    const double p = fmax(s, lp);
+    const double f1 = (double)expf((float)(s - p)), f2 = (double)expf((float)(lp - p));   // (one of them is e^0)
+    aa = f1 * aa + f2 * la;
+    bb = f1 * bb + f2 * lb;
+    pp = p;
+}
+
+__global__ void __launch_bounds__(kWkvScanWaves * 64)
+wkv_f32_scan_kernel(int T, int C, int chunk, const float *__restrict__ w, const float *__restrict__ u,
+                    const float *__restrict__ k, const float *__restrict__ v, float *__restrict__ y,
+                    float *__restrict__ aa, float *__restrict__ bb, float *__restrict__ pp) {
+    __shared__ double sa[kWkvScanChunks][32], sb[kWkvScanChunks][32], sp[kWkvScanChunks][32];
+    const int per_b = C / 32;
+    const int b = blockIdx.x / per_b, c = (blockIdx.x % per_b) * 32 + (threadIdx.x & 31);
+    const int ch = threadIdx.x & 31, j = (int)(threadIdx.x >> 5);      // chunk of this thread
+    const int idx = b * C + c;
+    const size_t base = (size_t)b * T * C + c;
+    const double wc = (double)w[c], uc = (double)u[c];
+    const int t0 = min(j * chunk, T), t1 = min(t0 + chunk, T);
+    float kc[kWkvScanGroup], vc[kWkvScanGroup], kn[kWkvScanGroup], vn[kWkvScanGroup];
+    // (1) this chunk from an empty state
+    float a = 0.f, bs = 0.f;
+    double p = -1e30;
+    if (t0 < t1) {
+#pragma unroll
+        for (int i = 0; i < kWkvScanGroup; ++i) {
+            const size_t o = base + (size_t)min(t0 + i, t1 - 1) * C;
+            kc[i] = k[o]; vc[i] = v[o];
+        }
+        for (int g = t0; g < t1; g += kWkvScanGroup) {
+#pragma unroll
+            for (int i = 0; i < kWkvScanGroup; ++i) {       // the next group (past the end: the last row again, unused)
+                const size_t o = base + (size_t)min(g + kWkvScanGroup + i, t1 - 1) * C;
+                kn[i] = k[o]; vn[i] = v[o];
+            }
+#pragma unroll
+            for (int i = 0; i < kWkvScanGroup; ++i)
+                if (g + i < t1) (void)wkv_step_f32(wc, uc, kc[i], vc[i], a, bs, p);
+#pragma unroll
+            for (int i = 0; i < kWkvScanGroup; ++i) { kc[i] = kn[i]; vc[i] = vn[i]; }
+        }
+    }
+    sa[j][ch] = (double)a; sb[j][ch] = (double)bs; sp[j][ch] = p;
+    // the first rows of the replay are on their way while the joins run
+    if (t0 < t1) {
+#pragma unroll
+        for (int i = 0; i < kWkvScanGroup; ++i) {
+            const size_t o = base + (size_t)min(t0 + i, t1 - 1) * C;
+            kc[i] = k[o]; vc[i] = v[o];
+        }
+    }
+    __syncthreads();
+    // (2) the state before this chunk
+    double ja = (double)aa[idx], jb = (double)bb[idx], jp = (double)pp[idx];
+    for (int jj = 0; jj < j; ++jj) {
+        const int n = min(chunk, T - min(jj * chunk, T));
+        if (n > 0) wkv_scan_join(wc, n, sa[jj][ch], sb[jj][ch], sp[jj][ch], ja, jb, jp);
+    }
+    if (t0 >= t1) return;
+    // (3) replay
+    a = (float)ja; bs = (float)jb; p = jp;
+    for (int g = t0; g < t1; g += kWkvScanGroup) {
+#pragma unroll
+        for (int i = 0; i < kWkvScanGroup; ++i) {
+            const size_t o = base + (size_t)min(g + kWkvScanGroup + i, t1 - 1) * C;
+            kn[i] = k[o]; vn[i] = v[o];
+        }
+#pragma unroll
+        for (int i = 0; i < kWkvScanGroup; ++i)
+            if (g + i < t1) y[base + (size_t)(g + i) * C] = wkv_step_f32(wc, uc, kc[i], vc[i], a, bs, p);
+#pragma unroll
+        for (int i = 0; i < kWkvScanGroup; ++i) { kc[i] = kn[i]; vc[i] = vn[i]; }
+    }
+    if (t1 == T) { aa[idx] = a; bb[idx] = bs; pp[idx] = (float)p; }     // the chunk with the last step: the state after it
+}
+
 // Reference convention (cuda/operators.cu:6-37): naive pre-multiplied state in
 // and out, pp untouched; the max-shifted form runs in between.
 __global__ void __launch_bounds__(64)
@@ -406,6 +494,13 @@ int rwkv_wkv_f32(rwkv_stream_t stream, int64_t B, int64_t T, int64_t C, const fl
     RWKV_CHECK_ARG(w && u && k && v && y && aa && bb && pp, "rwkv_wkv_f32: null pointer");
     RWKV_CHECK_ARG(B > 0 && T > 0 && C > 0 && B * C < (1ll << 31) && T < (1ll << 31), "rwkv_wkv_f32: bad sizes");
     RWKV_CHECK_ALIGN(k, 4); RWKV_CHECK_ALIGN(v, 4); RWKV_CHECK_ALIGN(y, 4);
+    if (T >= kWkvScanMinT && C % 32 == 0 && B * (C / 32) < (1ll << 31)) {
+        const int chunk = (int)round_up((size_t)ceil_div(T, kWkvScanChunks), kWkvScanGroup);
+        hipLaunchKernelGGL(wkv_f32_scan_kernel, dim3((unsigned)(B * (C / 32))), dim3(kWkvScanWaves * 64), 0,
+                           (hipStream_t)stream, (int)T, (int)C, chunk, w, u, k, v, y, aa, bb, pp);
+        RWKV_CHECK_LAUNCH("wkv_f32_scan_kernel");
+        return RWKV_OK;
+    }
     hipLaunchKernelGGL(wkv_f32_kernel, dim3((unsigned)ceil_div(B * C, 64)), dim3(64), 0, (hipStream_t)stream,
                        (int)B, (int)T, (int)C, w, u, k, v, y, aa, bb, pp);
     RWKV_CHECK_LAUNCH("wkv_f32_kernel");

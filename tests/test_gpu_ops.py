@@ -209,6 +209,33 @@ def test_wkv_f32_split_invariance_and_large_k(ops):
     assert (y_all[0].cpu().double() - yr).abs().max() < 1e-4 * max(1.0, float(yr.abs().max()))
 
 
+@pytest.mark.parametrize("T", [256, 333, 1000])
+def test_wkv_f32_long_sequences_carry_a_state_in_and_out(ops, T):
+    """Sequences of 256 steps and more run as a two-pass scan inside a workgroup (ragged last chunks at 333 and
+    1000): a state carried in from a first call, the outputs and the state carried out against the float64
+    recurrence over both calls; large |k| must not overflow."""
+    _say(f"wkv_f32 scan T={T}")
+    B, C, T0 = 3, 96, 40
+    w, u, k, v = _wkv_case(B, T0 + T, C, seed=11)
+    k = k * 8
+    d = lambda t: t.cuda()
+    st = [torch.zeros(B, C).cuda(), torch.zeros(B, C).cuda(), torch.full((B, C), -1e38).cuda()]
+    ya = ops.wkv_f32(d(w), d(u), d(k[:, :T0].contiguous()), d(v[:, :T0].contiguous()), *st)
+    yb = ops.wkv_f32(d(w), d(u), d(k[:, T0:].contiguous()), d(v[:, T0:].contiguous()), *st)
+    y = torch.cat([ya, yb], 1).cpu().double()
+    assert torch.isfinite(y).all()
+    for b in range(B):
+        z = torch.zeros(C).double()
+        yr, ar, br, _ = O.wkv_naive(w.double(), u.double(), k[b].double(), v[b].double(), z, z.clone(), torch.full((C,), -1e38).double())
+        assert (y[b] - yr).abs().max() < 1e-4 * max(1.0, float(yr.abs().max()))
+        ys, a_s, b_s, p_s = O.wkv_stable(w.double(), u.double(), k[b].double(), v[b].double(), z, z.clone(), torch.full((C,), -1e38).double())
+        # the state in its shifted form: aa e^pp and bb e^pp are what the next call continues from
+        got_a, got_b, got_p = st[0][b].cpu().double(), st[1][b].cpu().double(), st[2][b].cpu().double()
+        scale = torch.exp(got_p - p_s)
+        assert ((got_b * scale - b_s).abs() <= 1e-4 * b_s.abs()).all()
+        assert ((got_a * scale - a_s).abs() <= 1e-4 * torch.maximum(a_s.abs(), b_s.abs())).all()
+
+
 def test_wkv_forward_f64_reference_convention(ops):
     """Drop-in for torch.ops.rwkv.wkv_forward: naive state in/out, pp untouched."""
     B, T, C = 1, 50, 96
