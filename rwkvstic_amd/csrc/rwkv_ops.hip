@@ -129,13 +129,16 @@ wkv_f32_kernel(int B, int T, int C, const float *__restrict__ w, const float *__
 }
 
 // Long sequences: the same recurrence as a two-pass scan inside one workgroup.  The recurrence is linear in
-// (aa, bb), so the T steps split into kWkvScanChunks chunks: (1) every chunk scans its steps from an empty
+// (aa, bb), so the T steps split into 2 NW chunks: (1) every chunk scans its steps from an empty
 // state, (2) its incoming state is the call's state joined with the contributions of the chunks before it
 // (a chunk of n steps decays what came in by e^{n w}), (3) it replays its steps from there and writes y.  A
-// thread's serial chain is 2 T / kWkvScanChunks steps instead of T, there are five wavefronts per SIMD instead
-// of a third of one, and k and v are read twice (the second time mostly out of the memory-side cache).
-// Workgroup = 32 channels of one sequence; lane = (chunk parity, channel), wavefront w holds chunks 2w, 2w + 1.
-constexpr int kWkvScanWaves = 8, kWkvScanChunks = 2 * kWkvScanWaves, kWkvScanGroup = 8;
+// thread's serial chain is T / NW steps instead of T, there are several wavefronts per SIMD instead
+// of a third of one, and k and v are read twice.
+// Workgroup = 32 channels of one sequence and NW wavefronts; lane = (chunk parity, channel), wavefront w holds
+// chunks 2w and 2w + 1.  Both passes are bound by their vector instructions and the memory traffic once there are
+// a few wavefronts per SIMD, so the host picks 8 chunks where that already fills the device and 16 otherwise
+// (8 sequences of 2560 channels and 1024 steps: 94-97 us with 8 chunks, 98 with 16, 109 with 32).
+constexpr int kWkvScanGroup = 8;
 constexpr int kWkvScanMinT = 256;       // shorter sequences stay with the serial kernel
 
 __device__ __forceinline__ void wkv_scan_join(double w, int n, double la, double lb, double lp, double &aa, double &bb, double &pp) {
@@ -147,11 +150,13 @@ __device__ __forceinline__ void wkv_scan_join(double w, int n, double la, double
     pp = p;
 }
 
-__global__ void __launch_bounds__(kWkvScanWaves * 64)
+template <int NW>
+__global__ void __launch_bounds__(NW * 64)
 wkv_f32_scan_kernel(int T, int C, int chunk, const float *__restrict__ w, const float *__restrict__ u,
                     const float *__restrict__ k, const float *__restrict__ v, float *__restrict__ y,
                     float *__restrict__ aa, float *__restrict__ bb, float *__restrict__ pp) {
-    __shared__ double sa[kWkvScanChunks][32], sb[kWkvScanChunks][32], sp[kWkvScanChunks][32];
+    constexpr int kChunks = 2 * NW;
+    __shared__ double sa[kChunks][32], sb[kChunks][32], sp[kChunks][32];
     const int per_b = C / 32;
     const int b = blockIdx.x / per_b, c = (blockIdx.x % per_b) * 32 + (threadIdx.x & 31);
     const int ch = threadIdx.x & 31, j = (int)(threadIdx.x >> 5);      // chunk of this thread
@@ -495,9 +500,16 @@ int rwkv_wkv_f32(rwkv_stream_t stream, int64_t B, int64_t T, int64_t C, const fl
     RWKV_CHECK_ARG(B > 0 && T > 0 && C > 0 && B * C < (1ll << 31) && T < (1ll << 31), "rwkv_wkv_f32: bad sizes");
     RWKV_CHECK_ALIGN(k, 4); RWKV_CHECK_ALIGN(v, 4); RWKV_CHECK_ALIGN(y, 4);
     if (T >= kWkvScanMinT && C % 32 == 0 && B * (C / 32) < (1ll << 31)) {
-        const int chunk = (int)round_up((size_t)ceil_div(T, kWkvScanChunks), kWkvScanGroup);
-        hipLaunchKernelGGL(wkv_f32_scan_kernel, dim3((unsigned)(B * (C / 32))), dim3(kWkvScanWaves * 64), 0,
-                           (hipStream_t)stream, (int)T, (int)C, chunk, w, u, k, v, y, aa, bb, pp);
+        const dim3 grid((unsigned)(B * (C / 32)));
+        if (B * (C / 32) * 4 >= 2048) {         // 8 chunks already give every SIMD two wavefronts
+            const int chunk = (int)round_up((size_t)ceil_div(T, 8), kWkvScanGroup);
+            hipLaunchKernelGGL(wkv_f32_scan_kernel<4>, grid, dim3(4 * 64), 0, (hipStream_t)stream, (int)T, (int)C, chunk,
+                               w, u, k, v, y, aa, bb, pp);
+        } else {
+            const int chunk = (int)round_up((size_t)ceil_div(T, 16), kWkvScanGroup);
+            hipLaunchKernelGGL(wkv_f32_scan_kernel<8>, grid, dim3(8 * 64), 0, (hipStream_t)stream, (int)T, (int)C, chunk,
+                               w, u, k, v, y, aa, bb, pp);
+        }
         RWKV_CHECK_LAUNCH("wkv_f32_scan_kernel");
         return RWKV_OK;
     }
