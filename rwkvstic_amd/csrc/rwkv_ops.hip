@@ -13,8 +13,8 @@ namespace rwkv {
 // in chunks of kc_rows rows (NB * kc_rows * 4 bytes <= 64 KiB); the matrix is
 // read exactly once, with one 16-byte load per lane per 1 KiB block.
 // ---------------------------------------------------------------------------
-template <int NB>
-__global__ void __launch_bounds__(kThreads)
+template <int NB, int NT, int NW>
+__global__ void __launch_bounds__(NW * 64)
 mm8_packed_kernel(int n_in, int n_out, int n_kb, int kc_blocks,
                   const float *__restrict__ x, const uint8_t *__restrict__ packed,
                   const float *__restrict__ r_row, const double *__restrict__ m_row,
@@ -23,17 +23,30 @@ mm8_packed_kernel(int n_in, int n_out, int n_kb, int kc_blocks,
     extern __shared__ __align__(16) unsigned char smem[];
     float *xs = reinterpret_cast<float *>(smem);                    // [NB][kc_rows]
     const int kc_rows = kc_blocks * kBlockRows;
-    double *dred = reinterpret_cast<double *>(xs + (size_t)NB * kc_rows);   // [2*NB*kWaves]
-    float *fred = reinterpret_cast<float *>(dred + 2 * NB * kWaves);        // [NB*kWaves*8]
+    constexpr int kPT = NW * 64;                                           // threads
+    double *dred = reinterpret_cast<double *>(xs + (size_t)NB * kc_rows);   // [2*NB*NW]
+    float *fred = reinterpret_cast<float *>(dred + 2 * NB * NW);            // [NT*NB*NW*8]
 
-    const int ct = blockIdx.x;
-    const uint8_t *const wtile[1] = {packed + (size_t)ct * n_kb * kBlockBytes};
-    const float *const xsp[1] = {xs};
+    // NT neighbouring column tiles per workgroup share one staging of the activations and every LDS read of
+    // them: with NB = 8 a tile's weights (n_in x 8 bytes) are a quarter of the activations staged for it
+    // (n_in x NB x 4 bytes), and each 16-byte LDS read feeds only four multiply-adds per tile.
+    const int n_tiles = (n_out + kTileCols - 1) / kTileCols;
+    const int ct0 = blockIdx.x * NT;
+    const uint8_t *wtile[NT];
+#pragma unroll
+    for (int m = 0; m < NT; ++m)
+        wtile[m] = packed + (size_t)min(ct0 + m, n_tiles - 1) * n_kb * kBlockBytes;       // past the end: the last tile again, its sums dropped
 
-    float acc[1][NB];
+    float acc[NT][NB];
     double zsum[2 * NB];   // [b]: sum x*m_row ; [NB+b]: sum x
 #pragma unroll
-    for (int b = 0; b < NB; ++b) { acc[0][b] = 0.f; zsum[b] = 0.0; zsum[NB + b] = 0.0; }
+    for (int b = 0; b < NB; ++b) {
+        zsum[b] = 0.0; zsum[NB + b] = 0.0;
+#pragma unroll
+        for (int m = 0; m < NT; ++m) acc[m][b] = 0.f;
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, s8 = lane >> 3;
+    constexpr int kAhead = NT >= 4 ? 2 : NT == 2 ? 3 : kUnroll;     // blocks per tile a wavefront has in flight
 
     for (int kb0 = 0; kb0 < n_kb; kb0 += kc_blocks) {
         const int kb1 = min(kb0 + kc_blocks, n_kb);
@@ -42,12 +55,12 @@ mm8_packed_kernel(int n_in, int n_out, int n_kb, int kc_blocks,
         // otherwise a chain of dependent memory latencies (NB loads of x per row, one row after the other)
         constexpr int kStageAhead = NB >= 4 ? 4 : 8;
         const int rows_here = (kb1 - kb0) * kBlockRows;
-        for (int i0 = threadIdx.x; i0 < rows_here; i0 += kStageAhead * kThreads) {
+        for (int i0 = threadIdx.x; i0 < rows_here; i0 += kStageAhead * kPT) {
             float xv[kStageAhead][NB], rr[kStageAhead];
             double mr[kStageAhead];
 #pragma unroll
             for (int u = 0; u < kStageAhead; ++u) {
-                const int i = i0 + u * kThreads, j = j0 + i;
+                const int i = i0 + u * kPT, j = j0 + i;
                 const bool in = i < rows_here && j < n_in;
                 rr[u] = in ? r_row[j] : 0.f;
                 mr[u] = in ? m_row[j] : 0.0;
@@ -56,7 +69,7 @@ mm8_packed_kernel(int n_in, int n_out, int n_kb, int kc_blocks,
             }
 #pragma unroll
             for (int u = 0; u < kStageAhead; ++u) {
-                const int i = i0 + u * kThreads;
+                const int i = i0 + u * kPT;
                 if (i < rows_here) {
 #pragma unroll
                     for (int b = 0; b < NB; ++b) {
@@ -69,20 +82,85 @@ mm8_packed_kernel(int n_in, int n_out, int n_kb, int kc_blocks,
             }
         }
         __syncthreads();
-        tile_accumulate<1, NB>(wtile, xsp, kc_rows, kb0, kb1, acc);
+        // wave w takes blocks kb0 + w, + kWaves, ...; lane (s8, column) accumulates its column over rows 32 q + 4 s8 + e
+        // of each block (the order of tile_accumulate, so one tile per workgroup gives the same bits as before)
+        for (int kbw = kb0 + wave; kbw < kb1; kbw += NW * kAhead) {
+            uint4 wv[NT][kAhead];
+#pragma unroll
+            for (int u = 0; u < kAhead; ++u) {
+                const int kb = kbw + u * NW;
+                if (kb < kb1) {
+#pragma unroll
+                    for (int m = 0; m < NT; ++m)
+                        wv[m][u] = *reinterpret_cast<const uint4 *>(wtile[m] + (size_t)kb * kBlockBytes + lane * 16);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kAhead; ++u) {
+                const int kb = kbw + u * NW;
+                if (kb < kb1) {
+#pragma unroll
+                    for (int b = 0; b < NB; ++b) {
+                        const float4 *xp = reinterpret_cast<const float4 *>(xs + (size_t)b * kc_rows + (kb - kb0) * kBlockRows + 4 * s8);
+                        const float4 x0 = xp[0], x1 = xp[8], x2 = xp[16], x3 = xp[24];
+#pragma unroll
+                        for (int m = 0; m < NT; ++m) {
+                            acc[m][b] = dot4_u8(wv[m][u].x, x0, acc[m][b]);
+                            acc[m][b] = dot4_u8(wv[m][u].y, x1, acc[m][b]);
+                            acc[m][b] = dot4_u8(wv[m][u].z, x2, acc[m][b]);
+                            acc[m][b] = dot4_u8(wv[m][u].w, x3, acc[m][b]);
+                        }
+                    }
+                }
+            }
+        }
         __syncthreads();
     }
-    block_sum<2 * NB>(zsum, dred);
-    float out[1][NB];
-    tile_reduce<1, NB>(acc, fred, out);
-    if (threadIdx.x < kTileCols) {
-        const int k = ct * kTileCols + threadIdx.x;
-        if (k < n_out) {
-            const double rc = r_col ? (double)r_col[k] : 1.0;
-            const double mc = m_col ? (double)m_col[k] : 0.0;
+    // sums over the workgroup's NW wavefronts in a fixed order (block_sum and tile_reduce for any NW)
 #pragma unroll
-            for (int b = 0; b < NB; ++b)
-                y[(size_t)b * n_out + k] = rc * (double)out[0][b] + zsum[b] + mc * zsum[NB + b];
+    for (int i = 0; i < 2 * NB; ++i) {
+        const double t = wave_sum(zsum[i]);
+        if (lane == 0) dred[i * NW + wave] = t;
+    }
+    float out[NT][NB];
+#pragma unroll
+    for (int m = 0; m < NT; ++m)
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            float t = acc[m][b];
+            t += __shfl_xor(t, 8, 64);
+            t += __shfl_xor(t, 16, 64);
+            t += __shfl_xor(t, 32, 64);
+            if (lane < 8) fred[((m * NB + b) * NW + wave) * 8 + lane] = t;
+        }
+    __syncthreads();
+    if (threadIdx.x < kTileCols) {
+#pragma unroll
+        for (int i = 0; i < 2 * NB; ++i) {
+            double t = 0.0;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) t += dred[i * NW + w];
+            zsum[i] = t;
+        }
+#pragma unroll
+        for (int m = 0; m < NT; ++m)
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                float t = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) t += fred[((m * NB + b) * NW + w) * 8 + threadIdx.x];
+                out[m][b] = t;
+            }
+#pragma unroll
+        for (int m = 0; m < NT; ++m) {
+            const int k = (ct0 + m) * kTileCols + threadIdx.x;
+            if (ct0 + m < n_tiles && k < n_out) {
+                const double rc = r_col ? (double)r_col[k] : 1.0;
+                const double mc = m_col ? (double)m_col[k] : 0.0;
+#pragma unroll
+                for (int b = 0; b < NB; ++b)
+                    y[(size_t)b * n_out + k] = rc * (double)out[m][b] + zsum[b] + mc * zsum[NB + b];
+            }
         }
     }
 }
@@ -540,17 +618,23 @@ int rwkv_mm8_packed(rwkv_stream_t stream, int64_t B, int64_t n_in, int64_t n_out
     // LDS budget for the staged activations: 48 KiB per chunk
     int kc_blocks = (int)(49152 / (B * kBlockRows * 4));
     if (kc_blocks > n_kb) kc_blocks = n_kb;
-    const size_t lds = (size_t)B * kc_blocks * kBlockRows * 4 + 2 * B * kWaves * 8 + B * kWaves * 8 * 4;
-    dim3 grid((unsigned)ceil_div(n_out, kTileCols));
+    // Four column tiles per workgroup where four or eight activation vectors meet a wide matrix: the staging and
+    // the LDS reads of the activations, shared by the four tiles, are then the larger part of a workgroup's
+    // work, and the grid still has more workgroups than compute units.  (Measured at 8 vectors: [2560 x 10240]
+    // 36 -> 29 us; with 320 tiles, two tiles per workgroup lose 1 to 5 us, and workgroups of 16 wavefronts lose more.)
+    const int64_t n_tiles = ceil_div(n_out, kTileCols);
+    const int nt = (B >= 4 && n_tiles >= 1024) ? 4 : 1;
+    const size_t lds = (size_t)B * kc_blocks * kBlockRows * 4 + 2 * B * kWaves * 8 + (size_t)nt * B * kWaves * 8 * 4;
+    dim3 grid((unsigned)ceil_div(n_tiles, nt));
     hipStream_t st = (hipStream_t)stream;
-#define LAUNCH_B(NB) \
-    hipLaunchKernelGGL(mm8_packed_kernel<NB>, grid, dim3(kThreads), lds, st, (int)n_in, (int)n_out, n_kb, kc_blocks, \
+#define LAUNCH_B(NB, NT) \
+    hipLaunchKernelGGL((mm8_packed_kernel<NB, NT, kWaves>), grid, dim3(kThreads), lds, st, (int)n_in, (int)n_out, n_kb, kc_blocks, \
                        x, packed, r_row, m_row, r_col, m_col, y)
     switch (B) {
-        case 1: LAUNCH_B(1); break;
-        case 2: LAUNCH_B(2); break;
-        case 4: LAUNCH_B(4); break;
-        default: LAUNCH_B(8); break;
+        case 1: LAUNCH_B(1, 1); break;
+        case 2: LAUNCH_B(2, 1); break;
+        case 4: if (nt == 4) LAUNCH_B(4, 4); else LAUNCH_B(4, 1); break;
+        default: if (nt == 4) LAUNCH_B(8, 4); else LAUNCH_B(8, 1); break;
     }
 #undef LAUNCH_B
     RWKV_CHECK_LAUNCH("mm8_packed_kernel");

@@ -57,8 +57,11 @@ def test_pack_strided_and_ragged(ops):
 SHAPES = [(2560, 2560), (2560, 10240), (10240, 2560)]
 
 
-@pytest.mark.parametrize("n_in,n_out", SHAPES + [(96, 40), (130, 77), (768, 50277)])
-@pytest.mark.parametrize("B", [1, 8])
+PACKED_CASES = [(n_in, n_out, B) for (n_in, n_out) in SHAPES + [(96, 40), (130, 77), (768, 50277)] for B in (1, 8)]
+PACKED_CASES += [(256, 8200, 4), (256, 8200, 2)]     # 1025 column tiles: four per workgroup at B = 4 (ragged last group), one at B = 2
+
+
+@pytest.mark.parametrize("n_in,n_out,B", PACKED_CASES)
 def test_mm8_packed_general_form(ops, n_in, n_out, B):
     _say(f"mm8_packed in={n_in} out={n_out} B={B}")
     g = torch.Generator().manual_seed(n_in + 3 * n_out + B)
