@@ -274,9 +274,10 @@ wkv_f32_scan_kernel(int T, int C, int chunk, const float *__restrict__ w, const 
             kc[i] = k[o]; vc[i] = v[o];
         }
     }
+    // the call's state is read ahead of the barrier: the thread with the last chunk overwrites it when it is done
+    double ja = (double)aa[idx], jb = (double)bb[idx], jp = (double)pp[idx];
     __syncthreads();
     // (2) the state before this chunk
-    double ja = (double)aa[idx], jb = (double)bb[idx], jp = (double)pp[idx];
     for (int jj = 0; jj < j; ++jj) {
         const int n = min(chunk, T - min(jj * chunk, T));
         if (n > 0) wkv_scan_join(wc, n, sa[jj][ch], sb[jj][ch], sp[jj][ch], ja, jb, jp);
