@@ -165,8 +165,11 @@ int rwkv_mm8_packed(rwkv_stream_t stream, int64_t B, int64_t n_in, int64_t n_out
                     const float *r_col, const float *m_col,
                     double *y);
 
-/* Max-shifted float32 WKV recurrence, one thread per (b, c), state in
- * registers.  k, v, y [B, T, C]; w, u [C]; state (aa, bb, pp) [B, C] updated
+/* Max-shifted float32 WKV recurrence, state in registers: one thread per
+ * (b, c) for short sequences; from 256 steps on (and C a multiple of 32) a
+ * two-pass scan over 8 or 16 chunks of the sequence inside a workgroup, whose
+ * results differ from the serial order by float32 rounding only.
+ * k, v, y [B, T, C]; w, u [C]; state (aa, bb, pp) [B, C] updated
  * in place and related to the reference's naive state by
  * aa_ref = aa*exp(pp), bb_ref = bb*exp(pp) (operators.cu:21-36; closed form
  * of the shifted recurrence: agnostic/agnosticRwkv.py:68-103). */
