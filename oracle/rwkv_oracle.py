@@ -30,15 +30,19 @@ the checks live in ``tests/test_oracle_*.py``):
 * ``typical_distribution`` – hand-worked kept sets and probabilities for the
   distribution (1/2, 1/4, 1/8, 1/8) at four values of tau and with a
   temperature; uniform logits keep every token.
-* ``block_forward`` / ``model_forward`` – composition of the above; token
-  shift and state rows pinned by chunk-size invariance (T tokens at once ==
-  T single-token calls) and by ``state[0]/state[1]`` equalling the last
-  LayerNorm outputs.
-* No reference-generated vectors exist (the reference has no tests and its
-  package does not import here without an absent dependency), so end-to-end
-  op *ordering* (k,v,r order of the mix rows, state row map, head on the last
-  token) is "parity unpinned" beyond a line-by-line reading of
-  ``agnostic/backends/modules/block.py:56-102`` and ``agnostic/backends/opt.py:61-76``.
+* ``block_forward`` / ``forward`` – with ``matmul_dtype=float64`` the model equals,
+  to 1e-12 (logits and every carried state row, prompt fed in two calls), a
+  textbook RWKV-4 written with ``nn.functional`` ops and the direct-sum WKV on
+  the canonically dequantised matrices; the same check is shown to fail (by
+  >= 1e-3) for swapped mix rows, reversed mix direction, a dropped bonus, a
+  changed decay, swapped key/receptance matrices, swapped LayerNorms and
+  swapped state rows.  The float32 default differs from that only by the
+  accumulation type of the products.  Also: chunk-size invariance and
+  ``state[0]/state[1]`` equalling the last LayerNorm outputs.
+* No reference-generated vectors exist (the reference has no tests and was not
+  imported), so what stays "parity unpinned" is what only its own run could
+  show: bit-exact ``(code, range, offset)`` triples from its torch build and
+  the attribute tree of its ``.rwkv`` export.
 """
 from __future__ import annotations
 

@@ -264,6 +264,156 @@ def test_model_matches_unquantised_float64_network(tiny):
     assert torch.corrcoef(torch.stack([got, want]))[0, 1] > 0.995
 
 
+# ------------------------------------------------ composition: exact, on the dequantised weights
+MATRIX_KEYS = ("att.key", "att.value", "att.receptance", "att.output", "ffn.key", "ffn.receptance", "ffn.value")
+
+
+def _dequantised_checkpoint(sd):
+    """The checkpoint whose matrices are what the quantised layout represents: W'[out,in] = (code * range + offset)^T
+    in float64 (quantiser pinned above).  Everything else is taken over in float64."""
+    d = {k: v.double() for k, v in sd.items()}
+    for key in [k for k in sd if k.endswith(".weight") and (k == "head.weight" or any(m in k for m in MATRIX_KEYS))]:
+        c, r, o = O.quantize_matrix(sd[key].float())
+        d[key] = (c.double() * r.double()[:, None] + o[:, None]).t().contiguous()
+    return d
+
+
+def _independent_network(d, toks, layers, C):
+    """Textbook RWKV-4 (BlinkDL's formulation: lerp token shift, sigmoid receptance, relu^2 channel mix, WKV as a
+    direct O(T^2) sum over the history) in float64 with nn.functional ops on the weights ``d``; shares no code with
+    the oracle's block/model composition.  Returns logits of the last token and the state the reference keeps:
+    per layer (last ln1 output, last ln2 output, aa, bb) with aa, bb the e^w-premultiplied history sums."""
+    F = torch.nn.functional
+    T = len(toks)
+    x = F.layer_norm(d["emb.weight"][toks], (C,), d["blocks.0.ln0.weight"], d["blocks.0.ln0.bias"])
+    rows = []
+    for i in range(layers):
+        p = f"blocks.{i}."
+        xx = F.layer_norm(x, (C,), d[p + "ln1.weight"], d[p + "ln1.bias"])
+        sx = torch.cat([torch.zeros(1, C, dtype=torch.float64), xx[:-1]])
+        mk, mv, mr = (d[p + f"att.time_mix_{c}"].reshape(-1) for c in "kvr")
+        k = torch.lerp(sx, xx, mk) @ d[p + "att.key.weight"].t()
+        v = torch.lerp(sx, xx, mv) @ d[p + "att.value.weight"].t()
+        r = torch.sigmoid(torch.lerp(sx, xx, mr) @ d[p + "att.receptance.weight"].t())
+        w = -torch.exp(d[p + "att.time_decay"])
+        wkv = O.wkv_direct_sum(w, d[p + "att.time_first"], k, v)
+        age = torch.arange(T, 0, -1, dtype=torch.float64)[:, None]          # token i has been decayed T - i times
+        e = torch.exp(age * w[None, :] + k)
+        aa, bb = (e * v).sum(0), e.sum(0)
+        x = x + (r * wkv) @ d[p + "att.output.weight"].t()
+        x2 = F.layer_norm(x, (C,), d[p + "ln2.weight"], d[p + "ln2.bias"])
+        sx2 = torch.cat([torch.zeros(1, C, dtype=torch.float64), x2[:-1]])
+        fk, fr = (d[p + f"ffn.time_mix_{c}"].reshape(-1) for c in "kr")
+        kk = torch.relu(torch.lerp(sx2, x2, fk) @ d[p + "ffn.key.weight"].t()) ** 2
+        x = x + torch.sigmoid(torch.lerp(sx2, x2, fr) @ d[p + "ffn.receptance.weight"].t()) * (
+            kk @ d[p + "ffn.value.weight"].t())
+        rows.append((xx[-1], x2[-1], aa, bb))
+    x = F.layer_norm(x, (C,), d["ln_out.weight"], d["ln_out.bias"])
+    return x[-1] @ d["head.weight"].t(), rows
+
+
+def _composition_error(m, d, toks, split):
+    """Largest deviation (logits absolute, state relative to the row's scale) of the oracle ``m``, fed ``toks`` in
+    two calls split at ``split`` so that every state row is carried across a call, from the independent network."""
+    want, rows = _independent_network(d, toks, m.layers, m.dims)
+    st = m.emptyState.clone()
+    _, st = m.forward(toks[:split].tolist(), st)
+    got, st = m.forward(toks[split:].tolist(), st)
+    err = float((got - want).abs().max())
+    for i, (x1, x2, aa, bb) in enumerate(rows):
+        for row, ref in ((0, x1), (1, x2), (2, aa), (3, bb)):
+            err = max(err, float(((st[i, row] - ref).abs() / (ref.abs().max() + 1e-300)).max()))
+    return err
+
+
+class _RowsSwapped(O.OracleModel):
+    """The oracle with the att-shift and ffn-shift state rows exchanged (a wrong state row map)."""
+
+    def block_forward(self, blk, x, state):
+        perm = torch.tensor([1, 0, 2, 3, 4])
+        s = state[perm].clone()
+        out = super().block_forward(blk, x, s)
+        state.copy_(s[perm])
+        return out
+
+
+def _mutants():
+    def kv_mix(m):
+        for b in m.blocks:
+            b["attmix"] = b["attmix"][[1, 0, 2]]
+
+    def ffn_mix(m):
+        for b in m.blocks:
+            b["ffnmix"] = b["ffnmix"][[1, 0]]
+
+    def no_bonus(m):
+        for b in m.blocks:
+            b["time_first"] = torch.zeros_like(b["time_first"])
+
+    def mix_reversed(m):
+        for b in m.blocks:
+            b["attmix"] = 1 - b["attmix"]
+            b["ffnmix"] = 1 - b["ffnmix"]
+
+    def decay_sign(m):
+        for b in m.blocks:
+            b["time_decay"] = b["time_decay"] * 0.5
+
+    def kr_matrices(m):
+        for b in m.blocks:
+            b["att_k"], b["att_r"] = b["att_r"], b["att_k"]
+
+    def ln_swapped(m):
+        for b in m.blocks:
+            b["ln1"], b["ln2"] = b["ln2"], b["ln1"]
+
+    return dict(kv_mix_rows_swapped=kv_mix, ffn_mix_rows_swapped=ffn_mix, time_first_zero=no_bonus,
+                mix_direction_reversed=mix_reversed, decay_halved=decay_sign, key_receptance_swapped=kr_matrices,
+                ln1_ln2_swapped=ln_swapped)
+
+
+COMPOSITION_TOL = 1e-12
+
+
+def test_model_composition_is_exact_on_dequantised_weights(tiny):
+    """With float64 products the oracle is the textbook network on the dequantised matrices, to rounding: logits and
+    every carried state row (shift rows, aa, bb) agree to 1e-12 with a network that shares no composition code.
+    Pins block_forward / forward: mix row order and direction, bonus, decay, which matrix gets which mix, the
+    state row map, the head on the last token (agnostic/backends/modules/block.py:56-102, opt.py:61-76)."""
+    sd, _ = tiny
+    m = O.OracleModel(sd, matmul_dtype=torch.float64)
+    toks = synth.random_tokens(7, V=512, seed=2)
+    err = _composition_error(m, _dequantised_checkpoint(sd), toks, split=3)
+    assert err < COMPOSITION_TOL, err
+
+
+@pytest.mark.parametrize("name", sorted(_mutants()) + ["state_rows_0_1_swapped"])
+def test_model_composition_pin_rejects_plausible_mistakes(tiny, name):
+    """Each one-line mistake in the composition moves the result by nine orders of magnitude more than the pin
+    allows, so the pin above cannot pass on a wrong oracle."""
+    sd, _ = tiny
+    if name == "state_rows_0_1_swapped":
+        m = _RowsSwapped(sd, matmul_dtype=torch.float64)
+    else:
+        m = O.OracleModel(sd, matmul_dtype=torch.float64)
+        _mutants()[name](m)
+    toks = synth.random_tokens(7, V=512, seed=2)
+    err = _composition_error(m, _dequantised_checkpoint(sd), toks, split=3)
+    assert err > 1e-4, (name, err)
+
+
+def test_float32_oracle_is_the_float64_oracle_up_to_accumulation_noise(tiny):
+    """matmul_dtype only changes the accumulation type of the products (matmul.py:124-142 naivedtype): the default
+    float32 oracle stays within float32 summation noise of the pinned float64 one."""
+    sd, m32 = tiny
+    m64 = O.OracleModel(sd, matmul_dtype=torch.float64)
+    toks = synth.random_tokens(7, V=512, seed=2).tolist()
+    l32, s32 = m32.forward(toks, m32.emptyState.clone())
+    l64, s64 = m64.forward(toks, m64.emptyState.clone())
+    assert (l32 - l64).abs().max() < 2e-5
+    assert torch.allclose(s32, s64, rtol=1e-4, atol=1e-5)
+
+
 # ---------------------------------------------------------------- sampler
 def test_typical_distribution_hand_worked_cases():
     """Probabilities (1/2, 1/4, 1/8, 1/8): surprises (1, 2, 3, 3) ln 2, entropy 1.75 ln 2, distances to the entropy
