@@ -73,7 +73,12 @@ int rwkv_mm8_one(rwkv_stream_t stream, int64_t n_in, int64_t n_out,
  * (rwkv_mm8_workspace_bytes(n_in, n_out, 1) > the maximum) are rejected with
  * RWKV_ERR_SIZE.  Same arithmetic, same kernels and bit-identical results as
  * rwkv_mm8_one.  All calls on one GPU share the array: calls that overlap on
- * one GPU (two streams, two threads) race; calls on one stream do not. */
+ * one GPU (two streams, two threads) race; calls on one stream do not.
+ * The first use on a device looks up the array's device address (a symbol
+ * look-up, not a stream operation): it must happen outside a stream capture.
+ * rwkv_mm8_one_static_max_bytes() performs that look-up for the current device,
+ * so a caller about to capture calls it (or the entry point itself) once
+ * before; later calls enqueue two kernels and nothing else. */
 size_t rwkv_mm8_one_static_max_bytes(void);
 int rwkv_mm8_one_static(rwkv_stream_t stream, int64_t n_in, int64_t n_out,
                         const float *x, const uint8_t *w, int64_t w_stride,

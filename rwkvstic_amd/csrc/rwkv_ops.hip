@@ -528,7 +528,14 @@ int rwkv_mm8_one(rwkv_stream_t stream, int64_t n_in, int64_t n_out, const float 
     return mm8_ref_launch((hipStream_t)stream, 1, n_in, n_out, xs, ws_, st, ys, rs, workspace, workspace_bytes);
 }
 
-size_t rwkv_mm8_one_static_max_bytes(void) { return kStaticScratchBytes; }
+size_t rwkv_mm8_one_static_max_bytes(void) {
+    // Also the warm-up of rwkv_mm8_one_static on the current device: the symbol look-up of the first call is not
+    // something a stream capture should contain, so a caller about to capture asks for the limit first.  Best
+    // effort: without a usable device the limit is still returned and the entry point itself reports the error.
+    void *p = nullptr;
+    (void)static_scratch(&p);
+    return kStaticScratchBytes;
+}
 
 int rwkv_mm8_one_static(rwkv_stream_t stream, int64_t n_in, int64_t n_out, const float *x, const uint8_t *w,
                         int64_t w_stride, float *y, const float *r) {

@@ -132,8 +132,11 @@ sample_kernel(SampleArgs a) {
         }
         // Radix search, most significant bits first, two bits per round: the largest prefix P with mass{key < P} < tau.
         // `below` = mass{key < prefix}.
+        // A prefix with no mass at all below it is always taken: typical.py:13-14 keeps the token at position
+        // #(cumulative < tau) of the sorted distances, so the token nearest the entropy stays even with tau = 0.
         unsigned prefix = 0;
         float below = 0.f;
+#define RWKV_BELOW(t) ((t) < a.tau || (t) <= 0.f)
 #define RWKV_FULL_ROUND(shift)                                                                                           \
         {                                                                                                                \
             float m1 = 0.f, m2 = 0.f, m3 = 0.f;                                                                          \
@@ -150,8 +153,8 @@ sample_kernel(SampleArgs a) {
             __syncthreads();                                                                                             \
             float t1 = 0.f, t2 = 0.f, t3 = 0.f;                                                                          \
             _Pragma("unroll") for (int w = 0; w < kST / 64; ++w) { t1 += scr[w]; t2 += scr[kST / 64 + w]; t3 += scr[2 * (kST / 64) + w]; } \
-            if (t3 < a.tau) { prefix = c3; below = t3; } else if (t2 < a.tau) { prefix = c2; below = t2; }               \
-            else if (t1 < a.tau) { prefix = c1; below = t1; }                                                            \
+            if (RWKV_BELOW(t3)) { prefix = c3; below = t3; } else if (RWKV_BELOW(t2)) { prefix = c2; below = t2; }       \
+            else if (RWKV_BELOW(t1)) { prefix = c1; below = t1; }                                                        \
         }
         // After 16 (or 20, 24, 28) bits only the tokens that share those bits with the cut can still decide the rest.
         // As soon as they fit a list of kSList entries, one wave finishes alone: no pass over all tokens, no barriers.
@@ -190,7 +193,7 @@ sample_kernel(SampleArgs a) {
                         m3 += key < c3 ? pi : 0.f;
                     }
                     const float t1 = below + wave_sum(m1), t2 = below + wave_sum(m2), t3 = below + wave_sum(m3);
-                    if (t3 < a.tau) prefix = c3; else if (t2 < a.tau) prefix = c2; else if (t1 < a.tau) prefix = c1;
+                    if (RWKV_BELOW(t3)) prefix = c3; else if (RWKV_BELOW(t2)) prefix = c2; else if (RWKV_BELOW(t1)) prefix = c1;
                 }
                 if (tid == 0) s_prefix = prefix;
             }
@@ -198,6 +201,7 @@ sample_kernel(SampleArgs a) {
             prefix = s_prefix;
         }
 #undef RWKV_FULL_ROUND
+#undef RWKV_BELOW
         // prefix = d* as bits (mass{key < d*} < tau <= mass{key <= d*}); if the whole mass stays below tau every
         // finite key passes.  Kept tokens, temperature, total.
         const float inv_t = a.temp != 1.0f ? 1.0f / a.temp : 1.0f;
@@ -209,7 +213,6 @@ sample_kernel(SampleArgs a) {
             p[k] = w;
             q += w;
         }
-#undef RWKV_KEY
         // inverse CDF in the order (thread, k): scan of the per-thread sums, then a walk inside one thread's tokens
         float own = q;
         float incl = own;
@@ -239,17 +242,22 @@ sample_kernel(SampleArgs a) {
             atomicMax(&s_tok, pick);
         }
         __syncthreads();
-        if (s_tok < 0) {                               // target fell on a boundary nobody claimed (or the total is 0): most probable token
-            // argmax over float32 logits kept in key order is gone; fall back on the first maximum of p
-            float bp = -1.f; int bi = 0;
+        if (s_tok < 0) {
+            // The target fell on a boundary nobody claimed, or every kept weight underflowed under the temperature
+            // (total 0): the kept token with the largest logit, the first of equals.  p[] holds the weights by now, so
+            // the logits are read again; the kept set is never empty (the token nearest the entropy is always in it).
+            double bp = -INFINITY; int bi = 0x7fffffff;
 #pragma unroll
-            for (int k = 0; k < PER; ++k) if (p[k] > bp) { bp = p[k]; bi = tid + kST * k; }
+            for (int k = 0; k < PER; ++k) {
+                const int i = tid + kST * k;
+                if (i < V && RWKV_KEY(k) <= prefix) { const double x = a.logits[i]; if (x > bp) { bp = x; bi = i; } }
+            }
 #pragma unroll
             for (int off = 32; off >= 1; off >>= 1) {
-                const float ob = __shfl_xor(bp, off, 64); const int oi = __shfl_xor(bi, off, 64);
+                const double ob = __shfl_xor(bp, off, 64); const int oi = __shfl_xor(bi, off, 64);
                 if (ob > bp || (ob == bp && oi < bi)) { bp = ob; bi = oi; }
             }
-            __shared__ float fv[kST / 64]; __shared__ int fi[kST / 64];
+            __shared__ double fv[kST / 64]; __shared__ int fi[kST / 64];
             if ((tid & 63) == 0) { fv[tid >> 6] = bp; fi[tid >> 6] = bi; }
             __syncthreads();
             if (tid == 0) {
@@ -258,6 +266,7 @@ sample_kernel(SampleArgs a) {
             }
             __syncthreads();
         }
+#undef RWKV_KEY
         token = s_tok;
     }
     if (tid == 0) {

@@ -17,6 +17,7 @@ from typing import Callable, Dict, Iterable, List, Optional, Sequence, Union
 import torch
 
 MODE = "hip-fastquant"
+DEVICE_SAMPLER_MAX_VOCAB = 53248        # rwkv_sample_token: 1024 threads x 52 values in registers
 
 
 def _clone(x):
@@ -103,7 +104,13 @@ class RWKVMaster:
             return False
         if len(self.lastToken) != 1 or set(kwargs) - {"temp", "top_p_usual"}:
             return False
-        return not stopStrings or isinstance(self.tokenizer, TokenIds)
+        if getattr(m, "vocab", 0) > DEVICE_SAMPLER_MAX_VOCAB:
+            return False                         # the device sampler keeps the whole distribution in one workgroup
+        if not stopStrings:
+            return True
+        # decoded ids are digits and spaces: a stop string of only those (or an empty one) can end the text
+        # (rwkvMaster.py:53), every other one never can
+        return isinstance(self.tokenizer, TokenIds) and all(s.strip("0123456789 ") != "" for s in stopStrings)
 
     def forward(self, state=None, number: int = 1, stopStrings: Sequence[str] = ("<|endoftext|>",),
                 stopTokens: Sequence[int] = (0,), progressLambda: Callable[[Dict], None] = _no_progress,
@@ -111,11 +118,13 @@ class RWKVMaster:
         ostate = self.myState if state is None else state
         if self._device_loop(number, stopStrings, progressLambda, kwargs):
             # one call: token kernel, sampler, stop test and the next embedding all stay on the GPU
-            self._draws = getattr(self, "_draws", 0) + 1
+            # the seed of a call comes from torch's global generator: reproducible under torch.manual_seed, and two
+            # masters in one process do not repeat each other's draws
+            seed = int(torch.randint(0, 2 ** 62, (1,)))
             toks, logits, ostate = self.model.decode_sample(
                 self.lastToken[0], number, ostate, greedy=self.sampler is greedy, temp=kwargs.get("temp", 1.0),
                 tau=kwargs.get("top_p_usual", 0.8), end_adj=end_adj,
-                seed=(torch.initial_seed() * 1000003 + self._draws) & (2 ** 63 - 1), stop_tokens=list(stopTokens))
+                seed=seed, stop_tokens=list(stopTokens))
             tokens = [int(t) for t in toks.tolist()]
             self.myState = ostate
             self.lastToken = [tokens[-1]]

@@ -129,6 +129,36 @@ def test_3b_width_two_layers_against_oracle():
     hip.check()
 
 
+def test_3b_width_900_token_prompt_against_fp64_oracle():
+    """Full width, 2 layers, a 900-token prompt in one call: the [900 x 2560]-output products take the 160-column
+    workgroups with a split contraction, and the WKV runs as the chunked scan at the real width; logits 1e-4 and
+    state 1e-4 against the CPU oracle with exact accumulation, and the same prompt fed as 450 + 450."""
+    from rwkvstic_amd.model import HipRWKV, wkv_state_to_reference
+    _, C, F, V = synth.SHAPES["3B"]
+    sd = synth.make_state_dict(2, C, F, V, seed=9, ln="random")
+    sd["blocks.0.att.time_decay"][::3] = -6.5          # slowly forgetting channels: the state spans the whole prompt
+    exact = O.OracleModel(sd, matmul_dtype=torch.float64)
+    hip = HipRWKV(sd)
+    prompt = synth.random_tokens(900, V=V, seed=17).tolist()
+    _say("oracle, 900 tokens")
+    le, se = exact.forward(prompt, exact.emptyState.clone())
+    _say("gpu, 900 tokens in one call")
+    lg, sg = hip.forward(prompt, hip.emptyState.clone())
+    e64 = float((lg.cpu() - le).abs().max())
+    _say(f"  |gpu - fp64 oracle| {e64:.2e}")
+    assert e64 < 1e-4 and int(lg.argmax()) == int(le.argmax())
+    s = wkv_state_to_reference(sg).cpu()
+    assert (s[:, :2] - se[:, :2]).abs().max() < 1e-3
+    assert ((s[:, 3] - se[:, 3]).abs() <= 1e-4 * se[:, 3].abs() + 1e-30).all()
+    assert ((s[:, 2] - se[:, 2]).abs() <= 1e-4 * torch.maximum(se[:, 2].abs(), se[:, 3]) + 1e-30).all()
+    s2 = hip.emptyState.clone()
+    _, s2 = hip.forward(prompt[:450], s2)
+    l2, s2 = hip.forward(prompt[450:], s2)
+    assert float((l2 - lg).abs().max()) < 5e-5
+    shift, wkv = _rel_state_err(s2, sg)
+    assert shift < 5e-5 and wkv < 1e-5
+
+
 def test_14b_width_two_layers_prompt_chunks_batch_and_oracle():
     """The 14B shape's width (C=5120, F=20480, V=50277), 2 layers: a prompt in chunks of 16 through the many-row
     kernels, single tokens through the persistent kernel (two groups of 16 channels per workgroup at this width:

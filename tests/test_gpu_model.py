@@ -321,6 +321,35 @@ def test_prompt_longer_than_one_pass(tiny):
     assert (lg - l2).abs().max() < 1e-5 and (sg[:, :2] - s2[:, :2]).abs().max() < 1e-6
 
 
+def test_long_prompts_hold_the_state_bound_against_exact_accumulation():
+    """2200 tokens on a model with slowly forgetting channels (time_decay down to -8: histories of thousands of
+    tokens): the float32 sums of the chunked WKV scan, carried from pass to pass, stay within the 1e-4 state bound
+    of the float64 recurrence (operators.cu:21-36), whether the prompt is one call or 1024-token chunks."""
+    from rwkvstic_amd.model import HipRWKV
+    sd = synth.make_state_dict(layers=3, C=64, V=512, seed=15, ln="random")
+    for i in range(3):
+        sd[f"blocks.{i}.att.time_decay"][: 32] = torch.linspace(-8.0, -5.0, 32)
+    exact, hip = O.OracleModel(sd, matmul_dtype=torch.float64), HipRWKV(sd)
+    toks = synth.random_tokens(2200, V=512, seed=13).tolist()
+    le, se = exact.forward(toks, exact.emptyState.clone())
+    lg, sg = hip.forward(toks, hip.emptyState.clone())
+    _say(f"2200-token prompt |dlogits| vs float64-accumulation oracle {(lg.cpu() - le).abs().max().item():.2e}")
+    assert (lg.cpu() - le).abs().max() < 1e-4 and int(lg.argmax()) == int(le.argmax())
+    _state_close(sg, se, tol=STATE_TOL)
+    s2 = hip.emptyState.clone()
+    for i in range(0, len(toks), 1024):
+        l2, s2 = hip.forward(toks[i:i + 1024], s2)
+    assert (l2.cpu() - le).abs().max() < 1e-4
+    _state_close(s2, se, tol=STATE_TOL)
+    # and token by token through the per-phase kernels for the last stretch
+    s3 = hip.emptyState.clone()
+    _, s3 = hip.forward(toks[:2100], s3)
+    for t in toks[2100:]:
+        l3, s3 = hip.forward([t], s3)
+    assert (l3.cpu() - le).abs().max() < 1e-4
+    _state_close(s3, se, tol=STATE_TOL)
+
+
 def test_prompt_gemm_path_mid_shape_vs_fp64_oracle():
     """C=256, F=1024, ragged vocabulary; 70 tokens (18 M-tiles: a partial 64-token workgroup tile)."""
     from rwkvstic_amd.model import HipRWKV

@@ -46,6 +46,31 @@ def test_typical_draws_follow_the_reference_distribution(V, temp, tau):
     assert chi < dof + 5.0 * (2 * dof) ** 0.5 + 10       # about five standard deviations
 
 
+def test_tau_zero_and_a_vanishing_temperature_never_fall_back_to_token_0():
+    """Probabilities (1/8, 1/4, 1/2, 1/8): distances of the surprises from the entropy are (1.25, 0.25, 0.75, 1.25) ln 2.
+    tau = 0 keeps position #(cumulative < 0) = 0 of the sorted distances (typical.py:13-14): token 1, always.  With a
+    temperature so small that every kept weight p^(1/temp) underflows the draw has nothing to draw from (the reference's
+    multinomial raises there); the device sampler then returns the kept token with the largest logit, never token 0
+    (which would read as end-of-text)."""
+    from rwkvstic_amd import ops
+    logits = torch.log(torch.tensor([0.125, 0.25, 0.5, 0.125], dtype=torch.float64)) - 1.5
+    want = O.typical_distribution(logits, 1.0, 0.0)
+    assert want.tolist() == [0.0, 1.0, 0.0, 0.0]
+    got = _draws(ops, logits, 64, temp=1.0, tau=0.0, seed=5)
+    assert got.tolist() == [1] * 64
+    got = _draws(ops, logits, 64, temp=1e-3, tau=0.8, seed=5)          # kept: everything; 0.5 ** 1000 underflows
+    assert got.tolist() == [2] * 64
+    got = _draws(ops, logits, 64, temp=1e-3, tau=0.2, seed=5)          # kept: token 1 only
+    assert got.tolist() == [1] * 64
+    # the same on a real-sized vocabulary (the variant with keys in LDS and registers)
+    g = torch.Generator().manual_seed(3)
+    big = torch.randn(50277, generator=g, dtype=torch.float64) * 2.5
+    want = O.typical_distribution(big, 1.0, 0.0)
+    assert int((want > 0).sum()) == 1
+    got = _draws(ops, big, 16, temp=1.0, tau=0.0, seed=9)
+    assert got.tolist() == [int(want.argmax())] * 16
+
+
 @pytest.mark.parametrize("spread,tau", [(0.02, 0.5), (0.3, 0.8)])
 def test_typical_cut_on_a_nearly_flat_distribution(spread, tau):
     """Logits of a random-init model: 50277 tokens of almost equal probability, so tens of thousands of distances

@@ -61,6 +61,44 @@ def test_forward_stops_on_stop_token_and_stop_string():
     assert r.forward(number=3, end_adj=100.0)["output"] == "0"      # token 0 wins, and it is a stop token
 
 
+class DeviceLoopStub(StubModel):
+    """A model that offers the device-side loop: records whether it was used."""
+    fused_step = True
+    vocab = 16
+
+    def decode_sample(self, token, n, state, **kw):
+        self.device_calls = getattr(self, "device_calls", 0) + 1
+        self.seeds = getattr(self, "seeds", []) + [kw["seed"]]
+        toks = torch.tensor([(int(token) + 1 + i) % self.V for i in range(n)])
+        return toks, torch.zeros(self.V, dtype=torch.float64), state
+
+
+def test_device_loop_is_taken_only_when_it_cannot_change_the_result():
+    """The whole-loop call is an optimisation of rwkvMaster.py:28-56: it must step aside for a vocabulary the device
+    sampler cannot hold, and for stop strings that the decoded text could end with (ids decode to digits and spaces)."""
+    def run(model, **kw):
+        r = RWKVMaster(model, torch.zeros(1, dtype=torch.float64), greedy)
+        r.lastToken = [2]
+        out = r.forward(number=3, stopTokens=[], **kw)
+        return getattr(model, "device_calls", 0), out["output"]
+    assert run(DeviceLoopStub()) == (1, "3 4 5")                                   # the default stop string cannot match ids
+    assert run(DeviceLoopStub(), stopStrings=[]) == (1, "3 4 5")
+    assert run(DeviceLoopStub(), stopStrings=["4"]) == (0, "3 4")                  # host loop, and it stops as the reference does
+    assert run(DeviceLoopStub(), stopStrings=["<|endoftext|>", "3 4"]) == (0, "3 4")
+    assert run(DeviceLoopStub(), stopStrings=[""]) == (0, "3")                     # every text ends with the empty string
+    big = DeviceLoopStub()
+    big.vocab = 65536
+    assert run(big) == (0, "3 4 5")
+    # seeds: reproducible under torch.manual_seed, different from call to call and from master to master
+    seeds = []
+    for _ in range(2):
+        torch.manual_seed(11)
+        a, b = DeviceLoopStub(), DeviceLoopStub()
+        run(a), run(a), run(b)
+        seeds.append(a.seeds + b.seeds)
+    assert seeds[0] == seeds[1] and len(set(seeds[0])) == 3
+
+
 def test_forward_progress_callback_payload():
     m, r = _master()
     r.lastToken = [0]

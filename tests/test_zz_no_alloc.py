@@ -39,3 +39,37 @@ def test_mm8_one_static_equals_mm8_one_on_two_calls_in_a_row():
     assert L.rwkv_mm8_workspace_bytes(big_in, big_out, 1) > L.rwkv_mm8_one_static_max_bytes()
     assert L.rwkv_mm8_one_static(st, big_in, big_out, x.data_ptr(), w.data_ptr(), big_out, y_st.data_ptr(), r.data_ptr()) == -3
     assert b"built-in" in L.rwkv_last_error()
+
+
+def test_mm8_one_static_under_graph_capture_replays_bit_for_bit():
+    """The use the entry point exists for: captured into a HIP graph (after the warm-up call that resolves the
+    array's address on this device) and replayed several times, with eager work and synchronisations between the
+    replays; every replay must equal the eager result bit for bit.  The operator accumulates into y, so y is
+    restored by a copy kernel inside the graph (no memset node)."""
+    from rwkvstic_amd import _native as N
+    L = N.lib()
+    assert L.rwkv_mm8_one_static_max_bytes() == 12 << 20                 # also the warm-up on this device
+    n_in, n_out = 1024, 4096
+    x, w, r, y0 = _case(n_in, n_out, 3)
+    eager = y0.clone()
+    N.check(L.rwkv_mm8_one_static(torch.cuda.current_stream().cuda_stream, n_in, n_out, x.data_ptr(), w.data_ptr(),
+                                  w.stride(0), eager.data_ptr(), r.data_ptr()))
+    torch.cuda.synchronize()
+    y = torch.empty_like(y0)
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.graph(graph, stream=side):
+        y.copy_(y0)
+        N.check(L.rwkv_mm8_one_static(torch.cuda.current_stream().cuda_stream, n_in, n_out, x.data_ptr(), w.data_ptr(),
+                                      w.stride(0), y.data_ptr(), r.data_ptr()))
+    for i in range(4):
+        y.fill_(float("nan"))
+        # other users of the array between replays: an eager call on a different shape
+        x2, w2, r2, y2 = _case(300 + i, 500, 10 + i)
+        N.check(L.rwkv_mm8_one_static(torch.cuda.current_stream().cuda_stream, 300 + i, 500, x2.data_ptr(), w2.data_ptr(),
+                                      w2.stride(0), y2.data_ptr(), r2.data_ptr()))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager), f"replay {i}"
