@@ -197,19 +197,25 @@ class RWKVMaster:
 def RWKV(path: Union[str, Dict[str, torch.Tensor]], mode: str = MODE, *, tokenizer=None, device: str = "cuda",
          sampler: Optional[Callable] = typical, **kwargs) -> RWKVMaster:
     """``path``: a BlinkDL ``.pth`` checkpoint, a file written by ``HipRWKV.save_quantized`` (the quantised
-    attribute tree of the reference's .rwkv export, opt.py:89-92, as plain tensors; by convention ``.rwkvq``), both
-    loaded with ``weights_only=True``, or an already loaded dict of either kind.  TorchScript ``.rwkv`` archives
-    themselves are not read: loading one runs the code stored in it.  Only the FASTQUANT mode exists in this
-    backend (load.py:42-47); other modes raise."""
+    attribute tree of the reference's .rwkv export as plain tensors; by convention ``.rwkvq``), both loaded with
+    ``weights_only=True``; a TorchScript ``.rwkv`` archive (opt.py:89-92), of which only the tensors are read, by
+    attribute path, without compiling or running the code stored in it (``rwkvstic_amd.archive``); or an already
+    loaded dict of either kind.  Only the FASTQUANT mode exists in this backend (load.py:42-47); other modes raise."""
     if mode != MODE:
         raise ValueError(f"mode {mode!r} is not provided by this backend (only {MODE!r})")
     if kwargs:
         raise TypeError(f"unsupported options for mode {MODE!r}: {sorted(kwargs)}")
     from .model import HipRWKV
     if isinstance(path, str):
-        if not (path.endswith(".pth") or path.endswith(".rwkvq")):
-            raise ValueError("only .pth checkpoints and .rwkvq quantised trees are supported")
-        weights = torch.load(path, map_location="cpu", weights_only=True)
+        if path.endswith(".rwkv"):
+            from .archive import read_archive_tensors
+            weights = read_archive_tensors(path)
+            if "emb.w" not in weights or "head.weights.0.weight" not in weights:
+                raise ValueError(f"{path}: no FASTQUANT attribute tree (emb.w, head.weights.0.weight, ...) in the archive")
+        elif path.endswith(".pth") or path.endswith(".rwkvq"):
+            weights = torch.load(path, map_location="cpu", weights_only=True)
+        else:
+            raise ValueError("only .pth checkpoints, .rwkvq quantised trees and .rwkv archives are supported")
     else:
         weights = path
     model = HipRWKV.from_quantized(weights, device=device) if "emb.w" in weights else HipRWKV(weights, device=device)

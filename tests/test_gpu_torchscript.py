@@ -187,3 +187,28 @@ def test_archive_with_the_reference_attribute_tree_rebuilds_the_model(tmp_path):
     ref = O.OracleModel(sd)
     lr, _ = ref.forward(toks, ref.emptyState.clone())
     assert (l2.cpu() - lr).abs().max() < 1e-3
+
+
+def test_rwkv_archive_is_read_without_running_its_code(tmp_path):
+    """RWKV("model.rwkv") (load.py:42-47 -> opt.py:89-92): the archive's tensors are taken by attribute path with a
+    restricted unpickler (no torch.jit.load), the codes are only repacked; same results as the model quantised here
+    from the float checkpoint.  The archive is this test's own, with the reference's attribute tree held as plain
+    tensor attributes; a real export of the reference does not exist here (parity with one: unpinned)."""
+    from archive_standins import write_archive
+    from rwkvstic_amd.master import RWKV, greedy
+    from rwkvstic_amd.model import HipRWKV
+    sd = synth.make_state_dict(layers=2, C=64, V=300, seed=14, ln="random")
+    path = str(tmp_path / "model.rwkv")
+    write_archive(sd, path)
+    r = RWKV(path, sampler=greedy)
+    hip = HipRWKV(sd)
+    toks = synth.random_tokens(9, V=300, seed=3).tolist()
+    l1, s1 = hip.forward(toks, hip.emptyState.clone())
+    l2, s2 = r.model.forward(toks, r.emptyState.clone())
+    # codes and ranges are bit-equal; the offsets hold a mean whose summation order differs in the last bits
+    assert (l1 - l2).abs().max() < 1e-9 and (s1[:, :2] - s2[:, :2]).abs().max() < 1e-9
+    ref = O.OracleModel(sd)
+    lr, _ = ref.forward(toks, ref.emptyState.clone())
+    assert (l2.cpu() - lr).abs().max() < 1e-3
+    out = r.forward(number=3, stopTokens=[], end_adj=0.0)
+    assert len(out["output"].split()) == 3

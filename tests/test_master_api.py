@@ -139,6 +139,8 @@ def test_rwkv_rejects_unknown_modes_and_files():
         RWKV("model.pth", mode="jax")
     with pytest.raises(ValueError):
         RWKV("model.onnx")
+    with pytest.raises((ValueError, FileNotFoundError)):
+        RWKV("no_such_model.rwkv")
     with pytest.raises(TypeError):
         RWKV({}, strategy="cuda fp16")
 
