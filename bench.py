@@ -110,7 +110,8 @@ def isolated_matvec(device="cuda"):
     of at least 512 MB, so no matrix is served from L2 or the 256 MB memory-side cache: GB/s = in x out bytes
     per call / time per call over HIP events."""
     import torch
-    from rwkvstic_amd import ops
+    from rwkvstic_amd import _native, ops
+    N_ws = _native.lib().rwkv_mm8_m16_workspace_bytes
     out = []
     pool = torch.randint(0, 256, (640 << 20,), dtype=torch.uint8, device=device)       # random bytes are valid packed codes
     g = torch.Generator(device=device).manual_seed(3)
@@ -145,7 +146,30 @@ def isolated_matvec(device="cuda"):
             e1.record()
             torch.cuda.synchronize()
             us = e0.elapsed_time(e1) / calls * 1e3
-            out.append({"shape": f"{n_in}x{n_out}", "batch": B, "us_per_call": round(us, 2),
+            out.append({"shape": f"{n_in}x{n_out}", "batch": B, "kernel": "mm8_packed", "us_per_call": round(us, 2),
+                        "GB_per_s": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                        "distinct_matrices": n_mats})
+            # the matrix-core route (rwkv_mm8_m16: digits once, then int8 MFMA on the M16 layout); random bytes
+            # are valid M16 blocks too
+            ws = torch.empty(N_ws(B, n_in), dtype=torch.uint8, device=device)
+
+            def run16(k):
+                for i in range(k):
+                    off = (i % n_mats) * nbytes
+                    ops.mm8_m16(x, pool[off:off + nbytes], n_in, n_out, r_row, m_row, r_col, m_col, out=y, workspace=ws)
+            run16(n_mats)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                run16(calls)
+            graph.replay()
+            torch.cuda.synchronize()
+            e0.record()
+            graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) / calls * 1e3
+            out.append({"shape": f"{n_in}x{n_out}", "batch": B, "kernel": "mm8_m16", "us_per_call": round(us, 2),
                         "GB_per_s": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                         "distinct_matrices": n_mats})
     return out

@@ -160,7 +160,7 @@ int rwkv_dequant_packed(rwkv_stream_t stream, const uint8_t *packed,
  *   dq[j,k] = code[j,k]*r_row[j]*r_col[k] + m_row[j] + m_col[k]
  *   y[b,k]  = r_col[k]*sum_j fp32(x[b,j]*r_row[j])*code[j,k]
  *             + sum_j x[b,j]*m_row[j] + m_col[k]*sum_j x[b,j]
- * for b < B <= 8.  x[B, n_in] float32, y[B, n_out] float64 (float32
+ * for b < B, B in {1, 2, 4, 8}.  x[B, n_in] float32, y[B, n_out] float64 (float32
  * accumulation of the matrix term, float64 zero-point terms, as in
  * MM8.forward matmul.py:51-62).  r_col / m_col may be NULL (= 1 / 0): that
  * is the reference layout.  Replaces MM8.forward for T == 1. */
@@ -169,6 +169,24 @@ int rwkv_mm8_packed(rwkv_stream_t stream, int64_t B, int64_t n_in, int64_t n_out
                     const float *r_row, const double *m_row,
                     const float *r_col, const float *m_col,
                     double *y);
+
+/* The same product on the matrix cores, for any B in 1..8, on the M16 layout
+ * (rwkv_pack_m16).  Two launches: the vectors are rewritten once as exact
+ * fixed-point digits (fp32(x*r_row) to 30 bits, one power-of-two scale per
+ * vector and chunk of 256 input rows), then every 16-column tile is
+ * multiplied with v_mfma_i32_16x16x64_i8; the integer sums are exact and the
+ * result is the real-number sum over the float32 values fp32(x*r_row) to
+ * float64 rounding: where rwkv_mm8_packed accumulates in float32 (as
+ * operators32.cu:18-40 does), this one does not round at all.  With B >= 2 the
+ * vector pipeline of rwkv_mm8_packed is the limit, not memory; this routine
+ * stays memory-bound.  workspace: rwkv_mm8_m16_workspace_bytes(B, n_in) bytes,
+ * 256-byte aligned, overwritten. */
+size_t rwkv_mm8_m16_workspace_bytes(int64_t B, int64_t n_in);
+int rwkv_mm8_m16(rwkv_stream_t stream, int64_t B, int64_t n_in, int64_t n_out,
+                 const float *x, const uint8_t *packed16,
+                 const float *r_row, const double *m_row,
+                 const float *r_col, const float *m_col,
+                 double *y, void *workspace, size_t workspace_bytes);
 
 /* Max-shifted float32 WKV recurrence, state in registers: one thread per
  * (b, c) for short sequences; from 256 steps on (and C a multiple of 32) a

@@ -18,7 +18,7 @@ EXPORTS = (
     "rwkv_mm8_one_static", "rwkv_mm8_one_static_max_bytes",
     "rwkv_quantize_u8", "rwkv_packed_bytes", "rwkv_pack_u8", "rwkv_unpack_u8", "rwkv_dequant_packed",
     "rwkv_packed_m16_bytes", "rwkv_pack_m16", "rwkv_unpack_m16",
-    "rwkv_mm8_packed", "rwkv_wkv_f32",
+    "rwkv_mm8_packed", "rwkv_mm8_m16_workspace_bytes", "rwkv_mm8_m16", "rwkv_wkv_f32",
     "rwkv_model_create", "rwkv_model_destroy", "rwkv_model_workspace_bytes",
     "rwkv_model_has_fused_step", "rwkv_model_check", "rwkv_model_set_trace", "rwkv_model_selftest_timeout", "rwkv_model_time_token_kernel",
     "rwkv_model_forward", "rwkv_model_decode_greedy", "rwkv_argmax_f64",
@@ -95,6 +95,9 @@ def lib() -> C.CDLL:
     L.rwkv_model_selftest_timeout.argtypes = [vp, vp, vp, vp]
     L.rwkv_model_time_token_kernel.argtypes = [vp, vp, vp, vp, vp, ci, C.POINTER(C.c_float)]
     L.rwkv_mm8_packed.argtypes = [vp, i64, i64, i64, vp, vp, vp, vp, vp, vp, vp]
+    L.rwkv_mm8_m16_workspace_bytes.restype = sz
+    L.rwkv_mm8_m16_workspace_bytes.argtypes = [i64, i64]
+    L.rwkv_mm8_m16.argtypes = [vp, i64, i64, i64, vp, vp, vp, vp, vp, vp, vp, vp, sz]
     L.rwkv_wkv_f32.argtypes = [vp, i64, i64, i64] + [vp] * 8
     L.rwkv_model_create.argtypes = [C.POINTER(ModelDesc), C.POINTER(vp)]
     L.rwkv_model_destroy.argtypes = [vp]

@@ -1,6 +1,7 @@
 // Stand-alone operators: the packed uint8 matvec, the WKV recurrences, argmax,
 // and the reference-layout mm8_one / mm8_three drop-ins.
 #include "rwkv_common.h"
+#include "rwkv_rows.h"
 
 #include <mutex>
 
@@ -161,6 +162,113 @@ mm8_packed_kernel(int n_in, int n_out, int n_kb, int kc_blocks,
                 for (int b = 0; b < NB; ++b)
                     y[(size_t)b * n_out + k] = rc * (double)out[m][b] + zsum[b] + mc * zsum[NB + b];
             }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// The same product for ONE vector, laid out so that a compute unit moves little besides its share of the matrix:
+// a workgroup of NW wavefronts owns NT neighbouring column tiles over the whole contraction (about one workgroup
+// per compute unit), stages the scaled vector once for all of them, and every wavefront requests ALL its weight
+// blocks (block kb = wave + NW v of each tile, v < VB) right after the loads of the staging - loads return in the
+// order they were issued, so the staging data arrives first and is converted while the matrix is on its way.
+// With one 8-column tile per workgroup the vector, its ranges and its float64 offsets (16 bytes per input row,
+// re-read by every workgroup) are more bytes through a compute unit's vector-memory path than the tile itself.
+// Arithmetic as in mm8_packed_kernel: float32 multiply-adds, fixed order (per lane by block, then lanes, then
+// wavefronts).
+// ---------------------------------------------------------------------------
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+constexpr int kOneStage = 10;           // input rows per thread: up to 10240 rows with 1024 threads
+
+template <int NT, int VB>
+__global__ void __launch_bounds__(1024)
+mm8_packed_one_kernel(int n_in, int n_out, int n_kb,
+                      const float *__restrict__ x, const uint8_t *__restrict__ packed,
+                      const float *__restrict__ r_row, const double *__restrict__ m_row,
+                      const float *__restrict__ r_col, const float *__restrict__ m_col,
+                      double *__restrict__ y) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    float *xs = reinterpret_cast<float *>(smem);                            // [n_kb * 128]
+    const int NW = blockDim.x >> 6, kPT = blockDim.x;
+    const int n_rows = n_kb * kBlockRows;
+    double *dred = reinterpret_cast<double *>(xs + n_rows);                 // [2 * NW]
+    float *fred = reinterpret_cast<float *>(dred + 2 * NW);                 // [NT][NW][8]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, s8 = lane >> 3;
+    const int n_tiles = (n_out + kTileCols - 1) / kTileCols;
+    // 1. the loads of the staging ...
+    float xv[kOneStage], rr[kOneStage];
+    double mr[kOneStage];
+#pragma unroll
+    for (int u = 0; u < kOneStage; ++u) {
+        const int j = threadIdx.x + u * kPT;
+        const bool in = j < n_in;
+        xv[u] = in ? x[j] : 0.f;
+        rr[u] = in ? r_row[j] : 0.f;
+        mr[u] = in ? m_row[j] : 0.0;
+    }
+    // 2. ... then every weight block of this wavefront
+    v4u wv[NT][VB];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const uint8_t *wtile = packed + (size_t)min(blockIdx.x * NT + t, n_tiles - 1) * n_kb * kBlockBytes;   // past the end: the last tile again, its sums dropped
+#pragma unroll
+        for (int v = 0; v < VB; ++v) {
+            const int kb = min(wave + v * NW, n_kb - 1);                    // past the end: a block nobody multiplies
+            wv[t][v] = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(wtile + (size_t)kb * kBlockBytes) + lane);
+        }
+    }
+    // 3. the staging data is here first
+    double zs = 0.0, xsum = 0.0;
+#pragma unroll
+    for (int u = 0; u < kOneStage; ++u) {
+        const int j = threadIdx.x + u * kPT;
+        if (j < n_rows) {
+            const double xd = (double)xv[u];
+            xs[j] = (float)(xd * (double)rr[u]);                            // matmul.py:131
+            zs += xd * mr[u];
+            xsum += xd;
+        }
+    }
+    zs = wave_sum(zs); xsum = wave_sum(xsum);
+    if (lane == 0) { dred[wave] = zs; dred[NW + wave] = xsum; }
+    __syncthreads();
+    float acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = 0.f;
+#pragma unroll
+    for (int v = 0; v < VB; ++v) {
+        const int kb = wave + v * NW;
+        if (kb < n_kb) {
+            const float4 *xp = reinterpret_cast<const float4 *>(xs + kb * kBlockRows + 4 * s8);
+            const float4 x0 = xp[0], x1 = xp[8], x2 = xp[16], x3 = xp[24];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                acc[t] = dot4_u8(wv[t][v].x, x0, acc[t]);
+                acc[t] = dot4_u8(wv[t][v].y, x1, acc[t]);
+                acc[t] = dot4_u8(wv[t][v].z, x2, acc[t]);
+                acc[t] = dot4_u8(wv[t][v].w, x3, acc[t]);
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        float a = acc[t];
+        a += __shfl_xor(a, 8, 64);
+        a += __shfl_xor(a, 16, 64);
+        a += __shfl_xor(a, 32, 64);
+        if (lane < 8) fred[(t * NW + wave) * 8 + lane] = a;
+    }
+    __syncthreads();
+    if (threadIdx.x < NT * kTileCols) {
+        const int t = threadIdx.x >> 3, c = threadIdx.x & 7;
+        double z = 0.0, xm = 0.0;
+        float sum = 0.f;
+        for (int w = 0; w < NW; ++w) { z += dred[w]; xm += dred[NW + w]; sum += fred[(t * NW + w) * 8 + c]; }
+        const int k = (blockIdx.x * NT + t) * kTileCols + c;
+        if (blockIdx.x * NT + t < n_tiles && k < n_out) {
+            const double rc = r_col ? (double)r_col[k] : 1.0;
+            const double mc = m_col ? (double)m_col[k] : 0.0;
+            y[k] = rc * (double)sum + z + mc * xm;
         }
     }
 }
@@ -623,6 +731,34 @@ int rwkv_mm8_packed(rwkv_stream_t stream, int64_t B, int64_t n_in, int64_t n_out
     RWKV_CHECK_ALIGN(packed, 16);
     RWKV_CHECK_ALIGN(x, 4); RWKV_CHECK_ALIGN(r_row, 4); RWKV_CHECK_ALIGN(m_row, 8); RWKV_CHECK_ALIGN(y, 8);
     const int n_kb = (int)ceil_div(n_in, kBlockRows);
+    hipStream_t st = (hipStream_t)stream;
+    if (B == 1 && n_in <= kOneStage * 1024) {
+        // One vector: the variant that stages once per workgroup and requests the whole matrix up front.
+        // Workgroups of nw wavefronts (each takes every nw-th block of a tile, at most vb of them), nt tiles each,
+        // so that there is about one workgroup per compute unit.
+        const int64_t n_tiles1 = ceil_div(n_out, kTileCols);
+        int nw = 4;
+        while (nw < 16 && (ceil_div(n_kb, nw) > 5 || nw * 64 * kOneStage < n_in)) nw += (nw == 8 ? 2 : nw == 10 ? 6 : 4);   // 4, 8, 10, 16
+        if (n_kb % 10 == 0 && n_kb / 10 <= 2 && nw < 10 && n_in <= 640 * kOneStage) nw = 10;     // 1280 or 2560 rows: an exact split over 10 wavefronts
+        const int vb = (int)ceil_div(n_kb, nw);
+        // as many tiles per workgroup as leave at least 160 workgroups: fewer re-reads of the vector, and every
+        // workgroup resident at once (one workgroup of 10 or 16 wavefronts fills a compute unit's registers)
+        const int nt = (vb <= 2 && n_tiles1 >= 5 * 160) ? 5 : n_tiles1 >= 2 * 160 ? 2 : 1;
+        if (vb <= 5 && nw * 64 * kOneStage >= n_in) {
+            const size_t lds1 = (size_t)n_kb * kBlockRows * 4 + 2 * nw * 8 + (size_t)nt * nw * 8 * 4;
+            const dim3 grid1((unsigned)ceil_div(n_tiles1, nt)), block1((unsigned)(nw * 64));
+#define LAUNCH_ONE(NT, VB) \
+            hipLaunchKernelGGL((mm8_packed_one_kernel<NT, VB>), grid1, block1, lds1, st, (int)n_in, (int)n_out, n_kb, \
+                               x, packed, r_row, m_row, r_col, m_col, y)
+            if (nt == 5) LAUNCH_ONE(5, 2);
+            else if (nt == 2) { if (vb <= 2) LAUNCH_ONE(2, 2); else LAUNCH_ONE(2, 5); }
+            else if (vb <= 2) LAUNCH_ONE(1, 2);
+            else LAUNCH_ONE(1, 5);
+#undef LAUNCH_ONE
+            RWKV_CHECK_LAUNCH("mm8_packed_one_kernel");
+            return RWKV_OK;
+        }
+    }
     // LDS budget for the staged activations: 48 KiB per chunk
     int kc_blocks = (int)(49152 / (B * kBlockRows * 4));
     if (kc_blocks > n_kb) kc_blocks = n_kb;
@@ -634,7 +770,6 @@ int rwkv_mm8_packed(rwkv_stream_t stream, int64_t B, int64_t n_in, int64_t n_out
     const int nt = (B >= 4 && n_tiles >= 1024) ? 4 : 1;
     const size_t lds = (size_t)B * kc_blocks * kBlockRows * 4 + 2 * B * kWaves * 8 + (size_t)nt * B * kWaves * 8 * 4;
     dim3 grid((unsigned)ceil_div(n_tiles, nt));
-    hipStream_t st = (hipStream_t)stream;
 #define LAUNCH_B(NB, NT) \
     hipLaunchKernelGGL((mm8_packed_kernel<NB, NT, kWaves>), grid, dim3(kThreads), lds, st, (int)n_in, (int)n_out, n_kb, kc_blocks, \
                        x, packed, r_row, m_row, r_col, m_col, y)
@@ -647,6 +782,26 @@ int rwkv_mm8_packed(rwkv_stream_t stream, int64_t B, int64_t n_in, int64_t n_out
 #undef LAUNCH_B
     RWKV_CHECK_LAUNCH("mm8_packed_kernel");
     return RWKV_OK;
+}
+
+size_t rwkv_mm8_m16_workspace_bytes(int64_t B, int64_t n_in) {
+    if (B <= 0 || B > 8 || n_in <= 0) return 0;
+    return rows_mv16_workspace_bytes(B, n_in);
+}
+
+int rwkv_mm8_m16(rwkv_stream_t stream, int64_t B, int64_t n_in, int64_t n_out, const float *x,
+                 const uint8_t *packed16, const float *r_row, const double *m_row,
+                 const float *r_col, const float *m_col, double *y, void *workspace, size_t workspace_bytes) {
+    RWKV_CHECK_ARG(x && packed16 && r_row && m_row && y, "rwkv_mm8_m16: null pointer");
+    RWKV_CHECK_ARG(n_in > 0 && n_out > 0 && n_in < (1 << 30) && n_out < (1 << 30), "rwkv_mm8_m16: bad sizes");
+    if (B < 1 || B > 8) return set_error(RWKV_ERR_SIZE, "rwkv_mm8_m16: B must be 1..8 (got %lld)", (long long)B);
+    RWKV_CHECK_ALIGN(packed16, 16);
+    RWKV_CHECK_ALIGN(x, 4); RWKV_CHECK_ALIGN(r_row, 4); RWKV_CHECK_ALIGN(m_row, 8); RWKV_CHECK_ALIGN(y, 8);
+    const size_t need = rows_mv16_workspace_bytes(B, n_in);
+    if (!workspace || workspace_bytes < need)
+        return set_error(RWKV_ERR_WORKSPACE, "rwkv_mm8_m16: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    RWKV_CHECK_ALIGN(workspace, 256);
+    return rows_mv16((hipStream_t)stream, B, n_in, n_out, x, packed16, r_row, m_row, r_col, m_col, y, workspace);
 }
 
 }  // extern "C"

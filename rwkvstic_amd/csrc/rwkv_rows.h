@@ -51,4 +51,10 @@ int rows_wkv(hipStream_t st, int64_t R, int C, bool sequence, const float *k, co
              const double *w, const double *u, double *state, int64_t state_stride, float *out,
              double *scratch /* rows_wkv_scratch_bytes(R, C), or null: serial over the rows */);
 
+// Stand-alone product of 1..8 float32 vectors with one matrix in M16 blocks, four-vector dequantisation (row and
+// column ranges / offsets; r_col, m_col may be null); ws: rows_mv16_workspace_bytes(B, n_in) bytes, 256-byte aligned.
+size_t rows_mv16_workspace_bytes(int64_t B, int64_t n_in);
+int rows_mv16(hipStream_t st, int64_t B, int64_t n_in, int64_t n_out, const float *x, const uint8_t *w16,
+              const float *r_row, const double *m_row, const float *r_col, const float *m_col, double *y, void *ws);
+
 }  // namespace rwkv

@@ -1122,6 +1122,186 @@ __global__ void __launch_bounds__(64) wkv_chunk_replay_kernel(const WkvRowsArgs 
     }
 }
 
+// ---------------------------------------------------------------------------
+// Stand-alone matrix-vector product for 1..8 vectors on the M16 layout, four-vector dequantisation
+//   y[b,k] = r_col[k] * sum_j fp32(x[b,j] r_row[j]) code[j,k] + sum_j x[b,j] m_row[j] + m_col[k] sum_j x[b,j]
+// (the T == 1 branch of MM8.forward, matmul.py:51-62, with per-column factors on top).
+//
+// Two launches.  mv16_quant_kernel rewrites the vectors once, for every workgroup of the product, as fixed-point
+// digit fragments; the contraction is cut into chunks of CB = 4 blocks (256 rows) and every (vector, chunk) has its
+// own power-of-two scale, so no workgroup of the quantiser waits for another and the fixed point is as fine as
+// the chunk allows.  mv16_kernel gives one 16-column tile to a workgroup whose wavefronts take the chunks in
+// turn: all loads of a chunk (CB weight blocks from HBM, CB fragments per group of four vectors from L2) are
+// requested before the first matrix instruction, the integer digit sums of a chunk are exact and enter a float64
+// sum scaled by the chunk's scale; the wavefronts' sums are added in a fixed order.
+// ---------------------------------------------------------------------------
+struct Mv16Args {
+    int B, n_in, n_out, KB, n_chunks;
+    const float *x;             // [B, n_in]
+    const float *r_row;         // [n_in]
+    const double *m_row;        // [n_in]
+    const float *r_col, *m_col; // [n_out] or null
+    const uint8_t *w16;         // M16 blocks [ceil(n_out/16)][KB][1024]
+    signed char *dig;           // fragments [ceil(B/4)][KB][1024]
+    double *rec;                // [B][n_chunks][4]: scale, 128 * scale * sum q, zero-point share, sum x
+    double *y;                  // [B, n_out]
+};
+
+template <int CB>
+__global__ void __launch_bounds__(256) mv16_quant_kernel(const Mv16Args a) {
+    // workgroup = (chunk, group of four vectors); wavefront = one vector; a lane holds CB / 4 groups of four values
+    constexpr int QPT = CB / 4;
+    const int c = blockIdx.x, mt = blockIdx.y;
+    const int lane = threadIdx.x & 63, t = 4 * mt + (threadIdx.x >> 6);
+    if (t >= a.B) return;                          // (whole wavefronts; the kernel has no barrier)
+    float xs[QPT][4];
+    float amax = 0.f;
+    double zp = 0.0, xsum = 0.0;
+    const bool vec = (a.n_in & 3) == 0 && ((reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.r_row)) & 15) == 0 &&
+                     (reinterpret_cast<uintptr_t>(a.m_row) & 15) == 0;
+#pragma unroll
+    for (int s = 0; s < QPT; ++s) {
+        const int c0 = c * CB * 64 + 4 * (lane + 64 * s);
+        float xv[4] = {0.f, 0.f, 0.f, 0.f}, rv[4] = {0.f, 0.f, 0.f, 0.f};
+        double mv[4] = {0.0, 0.0, 0.0, 0.0};
+        if (vec && c0 + 3 < a.n_in) {
+            const float4 x4 = *reinterpret_cast<const float4 *>(a.x + (size_t)t * a.n_in + c0);
+            const float4 r4 = *reinterpret_cast<const float4 *>(a.r_row + c0);
+            const double2 m0 = *reinterpret_cast<const double2 *>(a.m_row + c0), m1 = *reinterpret_cast<const double2 *>(a.m_row + c0 + 2);
+            xv[0] = x4.x; xv[1] = x4.y; xv[2] = x4.z; xv[3] = x4.w;
+            rv[0] = r4.x; rv[1] = r4.y; rv[2] = r4.z; rv[3] = r4.w;
+            mv[0] = m0.x; mv[1] = m0.y; mv[2] = m1.x; mv[3] = m1.y;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int j = c0 + i;
+                if (j < a.n_in) { xv[i] = a.x[(size_t)t * a.n_in + j]; rv[i] = a.r_row[j]; mv[i] = a.m_row[j]; }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const double xd = (double)xv[i];
+            xs[s][i] = (float)(xd * (double)rv[i]);                                   // matmul.py:131
+            zp += xd * mv[i];
+            xsum += xd;
+            amax = fmaxf(amax, fabsf(xs[s][i]));
+        }
+    }
+    amax = wmaxf(amax);
+    double S, invS;
+    row_scale(amax, S, invS);
+    double qsum = 0.0;
+#pragma unroll
+    for (int s = 0; s < QPT; ++s) {
+        const int c0 = c * CB * 64 + 4 * (lane + 64 * s);
+        if (c0 < a.KB * 64) qsum += emit_quad(xs[s], invS, c0, t, a.KB, a.dig);      // (whole groups of 16 lanes)
+    }
+    qsum = wsum(qsum); zp = wsum(zp); xsum = wsum(xsum);
+    if (lane == 0) {
+        double *r = a.rec + ((size_t)t * a.n_chunks + c) * 4;
+        r[0] = S; r[1] = 128.0 * (S * qsum); r[2] = zp; r[3] = xsum;
+    }
+}
+
+template <int MT, int CB, int NTW>
+__global__ void __launch_bounds__(1024) mv16_kernel(const Mv16Args a) {
+    extern __shared__ double mv_red[];            // [NW][MT][NTW][64] tile sums, then [4 MT][3] row constants
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), NW = blockDim.x >> 6;
+    const int g = lane >> 4, n = lane & 15, NT = (a.n_out + 15) >> 4;
+    // NTW neighbouring tiles per workgroup share every digit fragment a wavefront fetches
+    const v4i *bsrc[NTW];
+#pragma unroll
+    for (int j = 0; j < NTW; ++j)
+        bsrc[j] = reinterpret_cast<const v4i *>(a.w16 + (size_t)min((int)blockIdx.x * NTW + j, NT - 1) * a.KB * 1024) + lane;
+    const v4i *asrc[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) asrc[m] = reinterpret_cast<const v4i *>(a.dig + (size_t)m * a.KB * 1024) + lane;
+    double sum[MT][NTW];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int j = 0; j < NTW; ++j) sum[m][j] = 0.0;
+    double *red = mv_red, *rc3 = mv_red + (size_t)NW * MT * NTW * 64;
+    for (int c = wave; c < a.n_chunks; c += NW) {
+        v4i Bf[NTW][CB], Af[MT][CB];
+        const int kb0 = c * CB;
+#pragma unroll
+        for (int i = 0; i < CB; ++i) {
+            const size_t o = (size_t)min(kb0 + i, a.KB - 1) * 64;                   // past the end: a block nobody multiplies
+#pragma unroll
+            for (int j = 0; j < NTW; ++j) Bf[j][i] = __builtin_nontemporal_load(bsrc[j] + o);
+#pragma unroll
+            for (int m = 0; m < MT; ++m) Af[m][i] = asrc[m][o];
+        }
+        double rS[MT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m) rS[m] = a.rec[((size_t)min(4 * m + g, a.B - 1) * a.n_chunks + c) * 4];
+        if (c == wave && wave == NW - 1) {
+            // The last wavefront, while its first blocks travel: the per-vector constants.  Lane 8 t + p adds the
+            // chunks p, p + 8, ... of vector t (its loads are independent of each other), then the eight partial
+            // sums are added in a fixed order.
+            const int t = lane >> 3, p8 = lane & 7;
+            double ad = 0.0, z = 0.0, xsm = 0.0;
+            const double *r = a.rec + (size_t)min(t, a.B - 1) * a.n_chunks * 4;
+#pragma unroll 4
+            for (int cc = p8; cc < a.n_chunks; cc += 8) { ad += r[4 * cc + 1]; z += r[4 * cc + 2]; xsm += r[4 * cc + 3]; }
+#pragma unroll
+            for (int off = 1; off < 8; off <<= 1) {
+                ad += __shfl_xor(ad, off, 64); z += __shfl_xor(z, off, 64); xsm += __shfl_xor(xsm, off, 64);
+            }
+            if (p8 == 0 && t < 4 * MT) { rc3[3 * t] = ad; rc3[3 * t + 1] = z; rc3[3 * t + 2] = xsm; }
+        }
+        v4i acc[MT][NTW];
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int j = 0; j < NTW; ++j) acc[m][j] = v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < CB; ++i) {
+            if (kb0 + i < a.KB) {                                                     // uniform for the wavefront
+#pragma unroll
+                for (int m = 0; m < MT; ++m)
+#pragma unroll
+                    for (int j = 0; j < NTW; ++j)
+                        acc[m][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Af[m][i], Bf[j][i], acc[m][j], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int j = 0; j < NTW; ++j) {
+                // digit sums of at most 64 CB terms of magnitude <= 2^14 each; the weighted total is below 2^53: exact
+                const v4i d = acc[m][j];
+                const long long tot = ((((long long)d.x * 256 + d.y) * 256 + d.z) * 256) + d.w;
+                sum[m][j] += rS[m] * (double)tot;
+            }
+    }
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int j = 0; j < NTW; ++j) red[(((size_t)wave * MT + m) * NTW + j) * 64 + lane] = sum[m][j];
+    __syncthreads();
+    // wavefront j adds up tile j (fixed order) and writes its 16 columns
+    if (wave >= NTW) return;
+#pragma unroll
+    for (int j = 0; j < NTW; ++j) {
+        if (j != wave) continue;
+        const int nt = blockIdx.x * NTW + j, col = 16 * nt + n;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            double s = 0.0;
+            for (int w = 0; w < NW; ++w) s += red[(((size_t)w * MT + m) * NTW + j) * 64 + lane];
+            const int t = 4 * m + g;
+            if (nt < NT && t < a.B && col < a.n_out) {
+                const double rc = a.r_col ? (double)a.r_col[col] : 1.0;
+                const double mc = a.m_col ? (double)a.m_col[col] : 0.0;
+                a.y[(size_t)t * a.n_out + col] = rc * (s + rc3[3 * t]) + rc3[3 * t + 1] + mc * rc3[3 * t + 2];
+            }
+        }
+    }
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------
@@ -1350,6 +1530,61 @@ int rows_wkv(hipStream_t st, int64_t R, int C, bool sequence, const float *k, co
     }
     hipLaunchKernelGGL(wkv_rows_kernel, dim3((unsigned)ceil_div(C, 64), sequence ? 1u : (unsigned)R), dim3(64), 0, st, a);
     RWKV_CHECK_LAUNCH("wkv_rows_kernel");
+    return RWKV_OK;
+}
+
+// Plan of the stand-alone product: tiles per workgroup ntw and wavefronts per workgroup nw (chunks of kMvCB blocks).
+// Every workgroup must be resident at once - a second round of workgroups would start its loads only when the
+// first has drained - so the wavefronts take several chunks in turn where one chunk each would not fit.  Two
+// tiles per workgroup (half the fragment traffic) only where that leaves a workgroup for every compute unit.
+constexpr int kMvCB = 4;
+struct Mv16Plan { int ntw, nw, n_chunks; };
+
+static Mv16Plan mv16_plan(int64_t KB, int64_t NT, int MT) {
+    const int n_chunks = (int)ceil_div(KB, kMvCB);
+    const int ntw = NT >= 512 ? 2 : 1;
+    const int vgprs = ntw == 2 ? (MT == 2 ? 112 : 88) : (MT == 2 ? 96 : 64);      // mv16_kernel<MT, ntw> as compiled
+    const int waves_per_cu = 4 * (512 / vgprs > 8 ? 8 : 512 / vgprs);
+    const int64_t grid = ceil_div(NT, ntw);
+    for (int rounds = 1; rounds <= n_chunks; ++rounds) {
+        const int nw = (int)ceil_div(n_chunks, rounds);
+        if (nw > 16) continue;
+        if (nw <= ntw || grid <= 256 * (int64_t)(waves_per_cu / nw)) return Mv16Plan{ntw, nw < ntw ? ntw : nw, n_chunks};
+    }
+    return Mv16Plan{ntw, ntw, n_chunks};
+}
+
+size_t rows_mv16_workspace_bytes(int64_t B, int64_t n_in) {
+    if (B <= 0 || n_in <= 0) return 0;
+    const int64_t KB = ceil_div(n_in, 64), MT = ceil_div(B, 4);
+    return (size_t)(MT * KB * 1024) + (size_t)round_up(B * ceil_div(KB, 4) * 4 * 8, 256);
+}
+
+int rows_mv16(hipStream_t st, int64_t B, int64_t n_in, int64_t n_out, const float *x, const uint8_t *w16,
+              const float *r_row, const double *m_row, const float *r_col, const float *m_col, double *y, void *ws) {
+    Mv16Args a;
+    a.B = (int)B; a.n_in = (int)n_in; a.n_out = (int)n_out; a.KB = (int)ceil_div(n_in, 64);
+    const int MT = (int)ceil_div(B, 4);
+    const int64_t NT = ceil_div(n_out, 16);
+    const Mv16Plan pl = mv16_plan(a.KB, NT, MT);
+    const int nw = pl.nw, ntw = pl.ntw;
+    a.n_chunks = pl.n_chunks;
+    a.x = x; a.r_row = r_row; a.m_row = m_row; a.r_col = r_col; a.m_col = m_col; a.w16 = w16; a.y = y;
+    a.dig = static_cast<signed char *>(ws);
+    a.rec = reinterpret_cast<double *>(static_cast<char *>(ws) + (size_t)MT * a.KB * 1024);
+    const dim3 qg((unsigned)a.n_chunks, (unsigned)MT);
+    hipLaunchKernelGGL(mv16_quant_kernel<kMvCB>, qg, dim3(256), 0, st, a);
+    RWKV_CHECK_LAUNCH("mv16_quant_kernel");
+    const dim3 grid((unsigned)ceil_div(NT, ntw)), block((unsigned)(64 * nw));
+    const size_t lds = ((size_t)nw * MT * ntw * 64 + 4 * MT * 3) * sizeof(double);
+    if (ntw == 2) {
+        if (MT == 1) hipLaunchKernelGGL((mv16_kernel<1, kMvCB, 2>), grid, block, lds, st, a);
+        else hipLaunchKernelGGL((mv16_kernel<2, kMvCB, 2>), grid, block, lds, st, a);
+    } else {
+        if (MT == 1) hipLaunchKernelGGL((mv16_kernel<1, kMvCB, 1>), grid, block, lds, st, a);
+        else hipLaunchKernelGGL((mv16_kernel<2, kMvCB, 1>), grid, block, lds, st, a);
+    }
+    RWKV_CHECK_LAUNCH("mv16_kernel");
     return RWKV_OK;
 }
 

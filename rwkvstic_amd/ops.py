@@ -209,6 +209,35 @@ def mm8_packed(x: torch.Tensor, packed: torch.Tensor, n_in: int, n_out: int,
     return y
 
 
+def mm8_m16(x: torch.Tensor, packed16: torch.Tensor, n_in: int, n_out: int,
+            r_row: torch.Tensor, m_row: torch.Tensor,
+            r_col: Optional[torch.Tensor] = None, m_col: Optional[torch.Tensor] = None,
+            out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``mm8_packed`` on the matrix cores: ``y[B, out]`` float64 for ``x[B, in]`` float32, any B in 1..8, weights in
+    the M16 layout (``pack_m16``); exact integer sums instead of float32 accumulation."""
+    _req(x, torch.float32, "x"); _contig(x, "x")
+    _req(packed16, torch.uint8, "packed16"); _req(r_row, torch.float32, "r_row"); _req(m_row, torch.float64, "m_row")
+    if x.dim() != 2 or x.shape[1] != n_in:
+        raise ValueError("x must be [B, n_in]")
+    L = N.lib()
+    if packed16.numel() < L.rwkv_packed_m16_bytes(n_in, n_out) or r_row.numel() < n_in or m_row.numel() < n_in:
+        raise ValueError("buffer too small")
+    for t, nm in ((r_col, "r_col"), (m_col, "m_col")):
+        if t is not None:
+            _req(t, torch.float32, nm)
+            if t.numel() < n_out:
+                raise ValueError(f"{nm} too small")
+    B = x.shape[0]
+    y = out if out is not None else torch.empty((B, n_out), dtype=torch.float64, device=x.device)
+    _req(y, torch.float64, "out"); _contig(y, "out")
+    need = L.rwkv_mm8_m16_workspace_bytes(B, n_in)
+    ws = workspace if workspace is not None else torch.empty(max(need, 1), dtype=torch.uint8, device=x.device)
+    N.check(L.rwkv_mm8_m16(_stream(), B, n_in, n_out, x.data_ptr(), packed16.data_ptr(), r_row.data_ptr(),
+                           m_row.data_ptr(), r_col.data_ptr() if r_col is not None else None,
+                           m_col.data_ptr() if m_col is not None else None, y.data_ptr(), ws.data_ptr(), ws.numel()))
+    return y
+
+
 def gemm8(x: torch.Tensor, packed16: torch.Tensor, rng: torch.Tensor, off: torch.Tensor,
           n_in: int, n_out: int) -> torch.Tensor:
     """``y[T, n_out] = x[T, n_in] @ dequantised matrix`` with the single-token arithmetic

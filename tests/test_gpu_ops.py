@@ -83,6 +83,61 @@ def test_mm8_packed_general_form(ops, n_in, n_out, B):
     assert err <= tol
 
 
+M16_CASES = [(n_in, n_out, B) for (n_in, n_out) in SHAPES for B in (1, 8)]
+M16_CASES += [(96, 40, 3), (130, 77, 5), (768, 50277, 2), (4160, 48, 7), (20480, 32, 8), (64, 16, 1)]
+
+
+@pytest.mark.parametrize("n_in,n_out,B", M16_CASES)
+def test_mm8_m16_general_form(ops, n_in, n_out, B):
+    """The matrix-core route of the same product (any B in 1..8, M16 layout): exact integer sums over fp32(x * r_row),
+    so it is held to a bound 64 times tighter than the float32-accumulating kernel - what is left is the float32
+    rounding of x * r_row itself."""
+    _say(f"mm8_m16 in={n_in} out={n_out} B={B}")
+    g = torch.Generator().manual_seed(n_in + 3 * n_out + B)
+    codes = torch.randint(0, 256, (n_in, n_out), generator=g, dtype=torch.uint8)
+    m_row = torch.randn(n_in, generator=g) * 0.01
+    m_col = torch.randn(n_out, generator=g) * 0.01
+    r_row = torch.rand(n_in, generator=g) * 9e-4 + 1e-4
+    r_col = torch.rand(n_out, generator=g) * 9e-4 + 1e-4
+    x = torch.randn(B, n_in, generator=g)
+    x[0, : n_in // 3] *= 300.0                      # chunks of very different magnitude inside one vector
+    want = O.mm8_general_f64(x, codes, r_row, m_row, r_col, m_col)
+    p16 = ops.pack_m16(codes.cuda())
+    got = ops.mm8_m16(x.cuda(), p16, n_in, n_out, r_row.cuda(), m_row.double().cuda(), r_col.cuda(), m_col.cuda()).cpu()
+    scale = (x.abs().double() * r_row.double()) @ codes.double() * r_col.double()
+    tol = 2.0 ** -23 * scale.max(dim=1, keepdim=True).values / 8
+    err = ((got - want).abs() / tol).max()
+    _say(f"  max err / tol {err:.3e}")
+    assert err <= 1.0
+    # the reference layout (no per-column vectors) against the oracle's mm8_naive with exact accumulation
+    got = ops.mm8_m16(x.cuda(), p16, n_in, n_out, r_row.cuda(), m_row.double().cuda()).cpu()
+    want = O.mm8_naive(x.double(), codes, r_row, m_row.double(), dtype=torch.float64)
+    scale = (x.abs().double() * r_row.double()) @ codes.double()
+    assert ((got - want).abs() <= 2.0 ** -23 * scale.max(dim=1, keepdim=True).values / 8).all()
+
+
+def test_mm8_m16_agrees_with_mm8_packed_and_rejects_bad_arguments(ops):
+    from rwkvstic_amd._native import RwkvHipError
+    g = torch.Generator().manual_seed(77)
+    n_in, n_out = 2560, 2560
+    codes = torch.randint(0, 256, (n_in, n_out), generator=g, dtype=torch.uint8).cuda()
+    r = (torch.rand(n_in, generator=g) * 9e-4 + 1e-4).cuda()
+    m = (torch.randn(n_in, generator=g) * 0.01).double().cuda()
+    x = torch.randn(8, n_in, generator=g).cuda()
+    a = ops.mm8_packed(x, ops.pack(codes), n_in, n_out, r, m)
+    b = ops.mm8_m16(x, ops.pack_m16(codes), n_in, n_out, r, m)
+    assert (a - b).abs().max() < 2e-4 * float(b.abs().max())
+    # one vector of the eight on its own: the same bits (a vector's digits do not depend on its neighbours)
+    b3 = ops.mm8_m16(x[3:4].contiguous(), ops.pack_m16(codes), n_in, n_out, r, m)
+    assert torch.equal(b3[0], b[3])
+    with pytest.raises(RwkvHipError):
+        ops.mm8_m16(torch.zeros(9, n_in, device="cuda"), ops.pack_m16(codes), n_in, n_out, r, m)      # B > 8
+    with pytest.raises(RwkvHipError):
+        ops.mm8_m16(x, ops.pack_m16(codes), n_in, n_out, r, m, workspace=torch.empty(1024, dtype=torch.uint8, device="cuda"))
+    with pytest.raises(ValueError):
+        ops.mm8_m16(x, ops.pack_m16(codes)[:1000], n_in, n_out, r, m)
+
+
 @pytest.mark.parametrize("B", [1, 2, 4])
 def test_mm8_packed_reference_form_matches_cpu_path(ops, B):
     """r_col = m_col = None is MM8.forward; compare with the oracle's mm8_naive."""
