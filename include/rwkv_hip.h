@@ -190,9 +190,12 @@ int rwkv_mm8_m16(rwkv_stream_t stream, int64_t B, int64_t n_in, int64_t n_out,
 
 /* Max-shifted float32 WKV recurrence, state in registers: one thread per
  * (b, c) for short sequences; from 256 steps on (and C a multiple of 32) a
- * two-pass scan over 8 or 16 chunks of the sequence inside a workgroup, whose
- * results differ from the serial order by float32 rounding only.
- * k, v, y [B, T, C]; w, u [C]; state (aa, bb, pp) [B, C] updated
+ * scan over chunks of the sequence inside a workgroup.  With at least 512
+ * groups of 32 channels (B * C / 32) every chunk stays in registers between
+ * the pass that sums it up and the pass that writes y, so k and v are read
+ * once; smaller problems use 8 or 16 chunks per sequence and read them twice.
+ * Either way the results differ from the serial order by float32 rounding
+ * only.  k, v, y [B, T, C]; w, u [C]; state (aa, bb, pp) [B, C] updated
  * in place and related to the reference's naive state by
  * aa_ref = aa*exp(pp), bb_ref = bb*exp(pp) (operators.cu:21-36; closed form
  * of the shifted recurrence: agnostic/agnosticRwkv.py:68-103). */

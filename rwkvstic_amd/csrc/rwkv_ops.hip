@@ -408,6 +408,154 @@ wkv_f32_scan_kernel(int T, int C, int chunk, const float *__restrict__ w, const 
     if (t1 == T) { aa[idx] = a; bb[idx] = bs; pp[idx] = (float)p; }     // the chunk with the last step: the state after it
 }
 
+// The same scan with one read of k and v: the sequence is cut into blocks of kWbNC * kWbSB steps that a workgroup
+// (32 channels x kWbNC chunk positions) takes one after the other; a thread keeps the kWbSB steps of its chunk in
+// registers from the pass that sums them up to the pass that writes y, and the block after next is requested
+// while this one is computed.  One barrier per block (summaries and carried state are double-buffered in LDS).
+//
+// Written for the instruction count - with two and a half wavefronts per SIMD the scan is bound by its vector
+// instructions as much as by memory:
+//  * e^x for x <= 0 is one scaled v_exp_f32, the division a reciprocal and a multiply (a few ulp each, far inside
+//    the 1e-4 the recurrence is held to);
+//  * a chunk's summary is a direct sum: step i of n contributes e^{k_i + (n - i) w}, so with m = max_i of those
+//    exponents the summary is (sum e^{x_i - m} v_i, sum e^{x_i - m}, m): float32 throughout, no chain;
+//  * the state a chunk starts from, and the state a block hands on, are direct sums too: the carried state and
+//    the summaries before the chunk, each decayed over the steps in between, with float64 exponents (one
+//    exponential per term).  The exponent pp therefore never accumulates float32 roundings along the sequence;
+//  * inside a chunk's second pass the exponent is float32, starting from the float32 rounding of the float64
+//    exponent the chunk starts with: kWbSB roundings of 2^-24 |pp| at most, that end with the chunk.
+template <int kWbNC, int kWbSB>
+struct WkvBlockState {
+    float kc[kWbSB], vc[kWbSB], kn[kWbSB], vn[kWbSB];
+};
+
+__device__ __forceinline__ float wkv_exp_neg(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896341f); }   // x <= 0
+
+// One block of kWbNC * kWbSB steps from step tb; buf = parity of the block.  FULL: the block and the block after
+// it lie inside the sequence, so no load is clamped and no step is guarded.
+template <int kWbNC, int kWbSB, bool FULL>
+__device__ __forceinline__ void wkv_block(WkvBlockState<kWbNC, kWbSB> &st, int tb, int T, int C, int j, int ch, unsigned col,
+                                          int buf, float wf, float uwf, const float *__restrict__ kb,
+                                          const float *__restrict__ vb, float *__restrict__ yb,
+                                          float (*sa)[kWbNC][32], float (*sb)[kWbNC][32], double (*sp)[kWbNC][32],
+                                          float (*ca)[32], float (*cb)[32], double (*cp)[32]) {
+    constexpr int kBlk = kWbNC * kWbSB;
+    const double wc = (double)wf;
+    const int t0 = FULL ? tb + j * kWbSB : min(tb + j * kWbSB, T), t1 = FULL ? t0 + kWbSB : min(t0 + kWbSB, T);
+    const int tbn = FULL ? tb + kBlk : min(tb + kBlk, T), n = t1 - t0;
+    // the next block's rows are requested one by one between the steps below, so that the requests of a compute
+    // unit form a stream instead of a burst per block (past the end: the last row again, unused)
+    const int tn = tb + kBlk + j * kWbSB;
+    auto fetch_next = [&](int i) {
+        const unsigned o = (unsigned)(FULL ? tn + i : min(tn + i, T - 1)) * (unsigned)C + col;
+        st.kn[i] = __builtin_nontemporal_load(kb + o); st.vn[i] = __builtin_nontemporal_load(vb + o);
+    };
+    // (1) the chunk's summary
+    float x[kWbSB], m = -1e30f;
+#pragma unroll
+    for (int i = 0; i < kWbSB; ++i) {
+        x[i] = (FULL || i < n) ? st.kc[i] + (float)(n - i) * wf : -1e30f;
+        m = fmaxf(m, x[i]);
+    }
+    float a = 0.f, bs = 0.f;
+#pragma unroll
+    for (int i = 0; i < kWbSB; ++i) {
+        const float f = (FULL || i < n) ? wkv_exp_neg(x[i] - m) : 0.f;
+        a = fmaf(f, st.vc[i], a);
+        bs += f;
+        if (i < kWbSB / 2) fetch_next(i);
+    }
+    sa[buf][j][ch] = a; sb[buf][j][ch] = bs; sp[buf][j][ch] = (double)m;
+    __syncthreads();
+    // (2) the state before this chunk: the carried state decayed over t0 - tb steps plus the summaries of the
+    // chunks before it, each decayed over the steps between its end and t0; all on the common exponent pm
+    const float car_a = ca[buf][ch], car_b = cb[buf][ch];
+    const double car_p = cp[buf][ch];
+    double e[kWbNC];
+    const double e_car = car_p + (double)(t0 - tb) * wc;
+    double pm = e_car;
+#pragma unroll
+    for (int i = 0; i < kWbNC - 1; ++i) {
+        const int end_i = FULL ? tb + (i + 1) * kWbSB : min(tb + (i + 1) * kWbSB, T);
+        e[i] = i < j ? sp[buf][i][ch] + (double)(t0 - end_i) * wc : -1e300;
+        pm = fmax(pm, e[i]);
+    }
+    {
+        const float f = wkv_exp_neg((float)(e_car - pm));
+        a = f * car_a; bs = f * car_b;
+    }
+#pragma unroll
+    for (int i = 0; i < kWbNC - 1; ++i) {
+        if (i < j) {
+            const float f = wkv_exp_neg((float)(e[i] - pm));
+            a = fmaf(f, sa[buf][i][ch], a); bs = fmaf(f, sb[buf][i][ch], bs);
+        }
+    }
+    // the thread of the last chunk position hands the block's end state on: the same sum taken at tbn, its own
+    // summary included
+    if (j == kWbNC - 1) {
+        const double own = sp[buf][j][ch] + (double)(tbn - t1) * wc;
+        const double shift = (double)(tbn - t0) * wc;               // everything above, decayed on to tbn
+        const double pn = fmax(pm + shift, own);
+        const float f0 = wkv_exp_neg((float)(pm + shift - pn)), f1 = wkv_exp_neg((float)(own - pn));
+        ca[buf ^ 1][ch] = f0 * a + f1 * sa[buf][j][ch];
+        cb[buf ^ 1][ch] = f0 * bs + f1 * sb[buf][j][ch];
+        cp[buf ^ 1][ch] = pn;
+    }
+    // (3) second pass: the outputs (wkv_step_f32 with a float32 exponent)
+    float pf = (float)pm;
+#pragma unroll
+    for (int i = 0; i < kWbSB; ++i) {
+        if (FULL || i < n) {
+            const float kk = st.kc[i], vv = st.vc[i];
+            const float d2 = pf - kk, d = d2 - uwf;
+            const float ee = wkv_exp_neg(-fabsf(d)), ff = wkv_exp_neg(-fabsf(d2));
+            const float e1 = d >= 0.f ? 1.f : ee, e2 = d >= 0.f ? ee : 1.f;
+            const float yv = (e1 * a + e2 * vv) * __builtin_amdgcn_rcpf(fmaf(e1, bs, e2));
+            const float f1 = d2 >= 0.f ? 1.f : ff, f2 = d2 >= 0.f ? ff : 1.f;
+            a = fmaf(f1, a, f2 * vv);
+            bs = fmaf(f1, bs, f2);
+            pf = fmaxf(pf, kk) + wf;
+            __builtin_nontemporal_store(yv, yb + ((unsigned)(t0 + i) * (unsigned)C + col));
+        }
+        if (i < kWbSB - kWbSB / 2) fetch_next(kWbSB / 2 + i);
+    }
+#pragma unroll
+    for (int i = 0; i < kWbSB; ++i) { st.kc[i] = st.kn[i]; st.vc[i] = st.vn[i]; }
+}
+
+template <int kWbNC, int kWbSB>
+__global__ void __launch_bounds__(kWbNC * 32)
+wkv_f32_block_kernel(int T, int C, const float *__restrict__ w, const float *__restrict__ u,
+                     const float *__restrict__ k, const float *__restrict__ v, float *__restrict__ y,
+                     float *__restrict__ aa, float *__restrict__ bb, float *__restrict__ pp) {
+    __shared__ float sa[2][kWbNC][32], sb[2][kWbNC][32], ca[2][32], cb[2][32];
+    __shared__ double sp[2][kWbNC][32], cp[2][32];
+    const int per_b = C / 32;
+    const int b = blockIdx.x / per_b, ch = threadIdx.x & 31, j = (int)(threadIdx.x >> 5);
+    const unsigned col = (unsigned)((blockIdx.x % per_b) * 32 + ch);
+    const int idx = b * C + (int)col;
+    // element offsets inside one sequence fit 32 bits (the host checks T * C < 2^30): one uniform base per array
+    const float *kb = k + (size_t)b * T * C, *vb = v + (size_t)b * T * C;
+    float *yb = y + (size_t)b * T * C;
+    const float wf = w[col], uwf = (float)((double)u[col] + (double)wf);
+    constexpr int kBlk = kWbNC * kWbSB;
+    WkvBlockState<kWbNC, kWbSB> st;
+#pragma unroll
+    for (int i = 0; i < kWbSB; ++i) {
+        const unsigned o = (unsigned)min(j * kWbSB + i, T - 1) * (unsigned)C + col;
+        st.kc[i] = __builtin_nontemporal_load(kb + o); st.vc[i] = __builtin_nontemporal_load(vb + o);
+    }
+    if (j == 0) { ca[0][ch] = aa[idx]; cb[0][ch] = bb[idx]; cp[0][ch] = (double)pp[idx]; }      // (read after the first block's barrier)
+    int tb = 0, buf = 0;
+    for (; tb + 2 * kBlk <= T; tb += kBlk, buf ^= 1)
+        wkv_block<kWbNC, kWbSB, true>(st, tb, T, C, j, ch, col, buf, wf, uwf, kb, vb, yb, sa, sb, sp, ca, cb, cp);
+    for (; tb < T; tb += kBlk, buf ^= 1)
+        wkv_block<kWbNC, kWbSB, false>(st, tb, T, C, j, ch, col, buf, wf, uwf, kb, vb, yb, sa, sb, sp, ca, cb, cp);
+    __syncthreads();
+    if (j == 0) { aa[idx] = ca[buf][ch]; bb[idx] = cb[buf][ch]; pp[idx] = (float)cp[buf][ch]; }
+}
+
 // Reference convention (cuda/operators.cu:6-37): naive pre-multiplied state in
 // and out, pp untouched; the max-shifted form runs in between.
 __global__ void __launch_bounds__(64)
@@ -695,6 +843,13 @@ int rwkv_wkv_f32(rwkv_stream_t stream, int64_t B, int64_t T, int64_t C, const fl
     RWKV_CHECK_ALIGN(k, 4); RWKV_CHECK_ALIGN(v, 4); RWKV_CHECK_ALIGN(y, 4);
     if (T >= kWkvScanMinT && C % 32 == 0 && B * (C / 32) < (1ll << 31)) {
         const dim3 grid((unsigned)(B * (C / 32)));
+        if (B * (C / 32) >= 512 && T * C < (1ll << 30)) {     // enough workgroups for the one-read form
+            // 4 chunk positions of 16 steps: 128 threads, five workgroups per compute unit at 8 x 2560 channels
+            hipLaunchKernelGGL((wkv_f32_block_kernel<4, 16>), grid, dim3(4 * 32), 0, (hipStream_t)stream, (int)T, (int)C,
+                               w, u, k, v, y, aa, bb, pp);
+            RWKV_CHECK_LAUNCH("wkv_f32_block_kernel");
+            return RWKV_OK;
+        }
         if (B * (C / 32) * 4 >= 2048) {         // 8 chunks already give every SIMD two wavefronts
             const int chunk = (int)round_up((size_t)ceil_div(T, 8), kWkvScanGroup);
             hipLaunchKernelGGL(wkv_f32_scan_kernel<4>, grid, dim3(4 * 64), 0, (hipStream_t)stream, (int)T, (int)C, chunk,

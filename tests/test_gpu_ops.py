@@ -294,6 +294,31 @@ def test_wkv_f32_long_sequences_carry_a_state_in_and_out(ops, T):
         assert ((got_a * scale - a_s).abs() <= 1e-4 * torch.maximum(a_s.abs(), b_s.abs())).all()
 
 
+@pytest.mark.parametrize("T", [300, 1000])
+def test_wkv_f32_one_read_scan_with_ragged_blocks_and_a_carried_state(ops, T):
+    """With 512 and more groups of 32 channels the scan keeps each chunk's k and v in registers between its two passes
+    and reads them once (blocks of 128 steps; 300 and 1000 end inside a block and inside a chunk): outputs and the
+    state carried out, after a state carried in from a first call, against the float64 recurrence; large |k|."""
+    _say(f"wkv_f32 one-read scan T={T}")
+    B, C, T0 = 8, 2048, 30
+    w, u, k, v = _wkv_case(B, T0 + T, C, seed=21)
+    k = k * 6
+    d = lambda t: t.cuda()
+    st = [torch.zeros(B, C).cuda(), torch.zeros(B, C).cuda(), torch.full((B, C), -1e38).cuda()]
+    ya = ops.wkv_f32(d(w), d(u), d(k[:, :T0].contiguous()), d(v[:, :T0].contiguous()), *st)
+    yb = ops.wkv_f32(d(w), d(u), d(k[:, T0:].contiguous()), d(v[:, T0:].contiguous()), *st)
+    y = torch.cat([ya, yb], 1).cpu().double()
+    assert torch.isfinite(y).all()
+    for b in (0, 3, 7):
+        z = torch.zeros(C).double()
+        ys, a_s, b_s, p_s = O.wkv_stable(w.double(), u.double(), k[b].double(), v[b].double(), z, z.clone(), torch.full((C,), -1e38).double())
+        assert (y[b] - ys).abs().max() < 1e-4 * max(1.0, float(ys.abs().max()))
+        got_a, got_b, got_p = st[0][b].cpu().double(), st[1][b].cpu().double(), st[2][b].cpu().double()
+        scale = torch.exp(got_p - p_s)
+        assert ((got_b * scale - b_s).abs() <= 1e-4 * b_s.abs()).all()
+        assert ((got_a * scale - a_s).abs() <= 1e-4 * torch.maximum(a_s.abs(), b_s.abs())).all()
+
+
 def test_wkv_forward_f64_reference_convention(ops):
     """Drop-in for torch.ops.rwkv.wkv_forward: naive state in/out, pp untouched."""
     B, T, C = 1, 50, 96
