@@ -212,17 +212,19 @@ def phase_trace(model, L: int, C: int) -> int:
     if not model.fused_step:
         print("phase trace: this shape does not run the persistent kernel", file=sys.stderr)
         return 2
-    G, per = (C // 32 if C > 4096 else C // 16), 24          # workgroups of the persistent kernel
+    G, per = (C // 32 if C > 4096 else C // 16), 24          # owner workgroups of the persistent kernel
+    GA = N.lib().rwkv_model_trace_workgroups(model._handle)  # ... and the helper workgroups behind them
     st = model.emptyState.clone()
     for t in range(5):
         _, st = model.forward([t + 3], st)
-    buf = torch.zeros(G * L * per, dtype=torch.int64, device="cuda")
+    buf = torch.zeros(GA * L * per, dtype=torch.int64, device="cuda")
     N.check(N.lib().rwkv_model_set_trace(model._handle, buf.data_ptr()))
     model.forward([77], st)
     torch.cuda.synchronize()
     model.check()
     N.check(N.lib().rwkv_model_set_trace(model._handle, None))
-    t = buf.cpu().numpy().astype("float64").reshape(G, L, per) * 0.01          # microseconds
+    t_all = buf.cpu().numpy().astype("float64").reshape(GA, L, per) * 0.01     # microseconds
+    t, th = t_all[:G], t_all[G:]
     names = {0: "start", 16: "A:polled", 1: "A:stats", 2: "A:digits", 3: "A:mfma", 20: "A:sums", 4: "finA",
              17: "B:polled", 5: "B:scale", 6: "B:digits", 7: "B:mfma", 21: "B:sums", 8: "finB",
              18: "C:polled", 9: "C:stats", 10: "C:digits", 11: "C:mfma", 12: "finC",
@@ -240,6 +242,15 @@ def phase_trace(model, L: int, C: int) -> int:
             med = float(np.median(v))
             print(f"  {name:9s} min {v.min():6.2f}  med {med:6.2f}  max {v.max():6.2f}   (+{med - prev:5.2f} after the previous boundary)")
             prev = med
+        if GA > G:
+            print("  helper workgroups (ffn key), same time base:")
+            prev = float(np.median(t[:, l, 8] - base))
+            print(f"    (owners' finB, the input of this phase: med {prev:6.2f})")
+            for i, name in enumerate(("records", "stats", "digits", "parked", "published", "next weights")):
+                v = th[:, l, i] - base
+                med = float(np.median(v))
+                print(f"    {name:12s} min {v.min():6.2f}  med {med:6.2f}  max {v.max():6.2f}   (+{med - prev:5.2f})")
+                prev = med
     if L > 3:
         print(f"per layer, workgroup 0, layers 1..{L - 2}: {(t[0, L - 1, 0] - t[0, 1, 0]) / (L - 2):.2f} us")
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

@@ -262,9 +262,13 @@ int rwkv_model_has_fused_step(const rwkv_model *m);
 
 /* Diagnostics: when device_buffer is non-NULL, every workgroup g of every
  * following single-token launch writes 100 MHz wall-clock stamps of its phase
- * boundaries into device_buffer[g][layer][24], which must hold
- * (n_embd / 16) * n_layer * 24 int64 values (n_embd / 32 workgroups write at
- * n_embd = 5120); NULL switches it off. */
+ * boundaries into device_buffer[g][layer][24]; NULL switches it off.  The
+ * buffer must hold rwkv_model_trace_workgroups(m) * n_layer * 24 int64 values:
+ * the owner workgroups (n_embd / 16, or n_embd / 32 at n_embd = 5120) followed
+ * by the helper workgroups of the ffn key matrix where the kernel has them
+ * (80 at n_embd = 2560), whose six stamps are: records seen, statistics,
+ * digits written, tiles multiplied, results published, next weights fetched. */
+int rwkv_model_trace_workgroups(const rwkv_model *m);
 int rwkv_model_set_trace(rwkv_model *m, int64_t *device_buffer);
 
 /* Synchronises the device and returns RWKV_ERR_HIP if a single-token launch

@@ -20,7 +20,7 @@ EXPORTS = (
     "rwkv_packed_m16_bytes", "rwkv_pack_m16", "rwkv_unpack_m16",
     "rwkv_mm8_packed", "rwkv_mm8_m16_workspace_bytes", "rwkv_mm8_m16", "rwkv_wkv_f32",
     "rwkv_model_create", "rwkv_model_destroy", "rwkv_model_workspace_bytes",
-    "rwkv_model_has_fused_step", "rwkv_model_check", "rwkv_model_set_trace", "rwkv_model_selftest_timeout", "rwkv_model_time_token_kernel",
+    "rwkv_model_has_fused_step", "rwkv_model_check", "rwkv_model_set_trace", "rwkv_model_trace_workgroups", "rwkv_model_selftest_timeout", "rwkv_model_time_token_kernel",
     "rwkv_model_forward", "rwkv_model_decode_greedy", "rwkv_argmax_f64",
     "rwkv_sample_token", "rwkv_model_decode_sample",
     "rwkv_gemm8_workspace_bytes", "rwkv_gemm8", "rwkv_gemm8_plan",
@@ -92,6 +92,7 @@ def lib() -> C.CDLL:
     L.rwkv_model_has_fused_step.argtypes = [vp]
     L.rwkv_model_check.argtypes = [vp]
     L.rwkv_model_set_trace.argtypes = [vp, vp]
+    L.rwkv_model_trace_workgroups.argtypes = [vp]
     L.rwkv_model_selftest_timeout.argtypes = [vp, vp, vp, vp]
     L.rwkv_model_time_token_kernel.argtypes = [vp, vp, vp, vp, vp, ci, C.POINTER(C.c_float)]
     L.rwkv_mm8_packed.argtypes = [vp, i64, i64, i64, vp, vp, vp, vp, vp, vp, vp]

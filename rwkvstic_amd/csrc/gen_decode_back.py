@@ -53,6 +53,10 @@ GATE_WIDE = [int(x) for x in os.environ.get("RWKV_BACK_GATE_WIDE", "16,8,16,12")
 BARGATE = int(os.environ.get("RWKV_BACK_BARGATE", "1"))   # reloads deferred past the att output and ffn value phases follow the next phase's first barrier
 CARRYK = int(os.environ.get("RWKV_BACK_CARRYK", "0"))     # the carried reloads follow this barrier of the LayerNorm phase (0: statistics, 1: digits ready)
 CARRYW = int(os.environ.get("RWKV_BACK_CARRYW", "0"))     # window of the carried reloads (0: the phase's)
+# the same for workgroups whose ffn key tiles are streamed by helper workgroups (9 jobs per layer)
+GATE_HELP = [int(x) for x in os.environ.get("RWKV_BACK_GATE_HELP", "8,2,12,6").split(",")]
+WINDOW_HELP = int(os.environ.get("RWKV_BACK_WINDOW_HELP", "5"))
+R_HELP = int(os.environ.get("RWKV_BACK_R_HELP", "23"))
 GATE_SPINS = 1 << 16     # the gate gives way after this many looks (a few milliseconds): it only orders loads, it must never hold a wave
 S_SEQ = 98        # phases finished by this wave (the front waves' exchange sequence number runs one ahead)
 SLEEP = int(os.environ.get("RWKV_BACK_SLEEP", "0"))      # s_sleep units (64 cycles) between a phase's barrier and its reloads   # weight loads a wave keeps in flight while it reloads slots
@@ -77,7 +81,10 @@ class Emit:
 S_TMP = 62        # scratch pair for a block's address where block offsets are added on the scalar side
 
 
-def gen(KW, R, NV, NSH):
+def gen(KW, R, NV, NSH, HELP=False):
+    """HELP: the four ffn key tiles of a group are not this workgroup's (helper workgroups on the otherwise idle
+    compute units own that matrix): 9 jobs per layer instead of 13, and the ffn receptance tile takes its digits
+    from the first set of planes."""
     C = 512 * KW
     F = 4 * C
     PS, PSF = C + 64, F + 64
@@ -89,10 +96,12 @@ def gen(KW, R, NV, NSH):
     # and no register for the flag address leave room for a ring of 26 blocks in 128 registers.
     V_OFF, V_D, V_A, NA = (7, 8, 16, 2) if SADDR else (globals()["V_OFF"], globals()["V_D"], globals()["V_A"], globals()["NA"])
     PF = NA - 1
-    NJ = 13 * NT                     # jobs per layer
+    NJ = (9 if HELP else 13) * NT    # jobs per layer
     GATE = globals()["GATE"] if NT == 1 else GATE_WIDE
     WINDOW = globals()["WINDOW"] if NT == 1 else WINDOW_WIDE
     WINDOWS = globals()["WINDOWS"] if NT == 1 else [WINDOW_WIDE] * 4
+    if HELP:
+        GATE, WINDOW, WINDOWS = GATE_HELP, WINDOW_HELP, [WINDOW_HELP] * 4
     NREAL = NJ * KW
     PP = (NREAL + R - 1) // R * R
     RB = NV - 4 * R
@@ -115,8 +124,8 @@ def gen(KW, R, NV, NSH):
     for gi in range(NT):
         jobs.append(dict(ph=1, gi=gi, ptr=3, stride=TB, aset="C", aoff=0, first=True, park=gi * SPG))
     for gi in range(NT):
-        jobs.append(dict(ph=2, gi=gi, ptr=4, stride=TB, aset="C", aoff=4 * PS, first=True, park=gi * SPG))
-        for r in range(4):
+        jobs.append(dict(ph=2, gi=gi, ptr=4, stride=TB, aset="C", aoff=0 if HELP else 4 * PS, first=True, park=gi * SPG))
+        for r in range(0 if HELP else 4):
             jobs.append(dict(ph=2, gi=gi, ptr=5 + r, stride=TB, aset="C", aoff=0, first=True, park=gi * SPG + 1 + r))
     for gi in range(NT):
         for q in range(4):
@@ -228,8 +237,10 @@ def gen(KW, R, NV, NSH):
     # the statistics barrier (att output -> ffn key/receptance; ffn value -> next layer / head).  What the ffn value
     # phase carries over is issued at the top of the next layer, after that layer's first barrier - also in the
     # first layer, which is why the prologue leaves those positions out.
-    NB = NT * KW
-    phases = [(0, 3 * NB, 2), (3 * NB, 4 * NB, 1), (4 * NB, 9 * NB, 2), (9 * NB, 13 * NB, 1)]   # start, end, barriers before
+    phases = []                                # start, end, barriers before
+    for ph in range(4):
+        idx = [i for i, jb in enumerate(jobs) if jb["ph"] == ph]
+        phases.append((idx[0] * KW, (idx[-1] + 1) * KW, 2 if ph in (0, 2) else 1))
     def deferred_of(ph):
         ps, pe, _ = phases[ph]
         d = [p for p in range(ps, pe) if not (p + R < pe and DEFER) and DEFER]
@@ -465,13 +476,14 @@ def main():
     w("// Generated by gen_decode_back.py - do not edit.  One asm statement per kernel width: the program")
     w("// of a weight-streaming wave of the single-token kernel (see the generator for the register map).")
     w("template <int KW, int FW> struct BackCfg;")
-    for KW, FW, R in CONFIGS:
+    w("template <int KW, int FW> struct BackCfgH;      // with helper workgroups: no ffn key tiles")
+    for KW, FW, R, HELP in [c + (False,) for c in CONFIGS] + [(5, 8, R_HELP, True)]:
         NV = 168 if FW == 4 else 128
         clob = ", ".join(f'"v{i}"' for i in range(V_APC, NV)) + ", " + ", ".join(f'"s{i}"' for i in range(S_CUR, 102 if KW > 8 else 100))
         tiles_per_body = R // math.gcd(R, KW)
         NSH = max(d for d in range(1, 5) if tiles_per_body % d == 0)     # head tiles per barrier round
-        lines, info = gen(KW, R, NV, NSH)
-        w(f"template <> struct BackCfg<{KW}, {FW}> {{")
+        lines, info = gen(KW, R, NV, NSH, HELP)
+        w(f"template <> struct BackCfg{'H' if HELP else ''}<{KW}, {FW}> {{")
         w(f"    static constexpr int R = {R}, RED = {info['RED']}, FLAG = {info['FLAG']}, RED_SLOTS = {info['RED_SLOTS']}, NS = {info['NS']};")
         w("    static __device__ __forceinline__ void run(const unsigned long long *jt, const uint8_t *wh, int L, int hr, int vt,")
         w("                                                int g, int wb, unsigned lds) {")

@@ -99,6 +99,7 @@ struct DSetup {
 };
 
 bool decode_supported(int64_t L, int64_t C, int64_t F, int64_t V);
+int64_t decode_helper_workgroups(int64_t C);   // workgroups that only stream the ffn key matrix (launched after the owners)
 int64_t decode_workgroups(int64_t C);          // grid of the single-token kernel (C / 16, or C / 32 where a workgroup owns two groups)
 unsigned decode_epochs_per_token(int64_t L);
 constexpr int kTraceStampsPerLayer = 24;

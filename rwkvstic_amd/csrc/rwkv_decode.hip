@@ -97,6 +97,22 @@ struct GroupShape {
     static constexpr int NT = KW > 8 ? 2 : 1, G = 32 * KW, NWG = G / NT;
 };
 
+// Helper workgroups.  At C = 2560 the grid of C / 16 = 160 owner workgroups leaves 96 compute units without
+// work; 80 more workgroups there own the ffn key matrix (31 % of a layer's bytes): helper h keeps its 8 tiles of
+// the NEXT layer in registers (fetched right after it has multiplied the current ones, a whole layer ahead of
+// their use), waits like everybody else for the input of the ffn phase, and publishes relu(k)^2 with its records.
+// The owner workgroups then stream 9 tiles per layer instead of 13 and have the ffn receptance tile only to
+// multiply in that phase.
+#ifndef RWKV_T_PACE
+#define RWKV_T_PACE 20
+#endif
+template <int KW>
+struct HelperShape {
+    static constexpr int NH = KW == 5 ? 80 : 0;                    // helper workgroups
+    static constexpr int TILES = NH ? (4 * 32 * KW) / NH : 1;      // ffn key tiles of 16 columns per helper
+    static constexpr int LDS_BLOCKS = 6;                           // weight blocks per wavefront that wait in LDS instead of registers
+};
+
 struct DArgs {
     DModel m;
     DecodeBuffers b;
@@ -535,7 +551,8 @@ __device__ __forceinline__ double ln_zp(const double *stat, const u64 *rec, int 
 template <int KW, int FW, int NM>
 __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, const float *P32, const float *Q32,
                                          const u64 *rec, int m0, unsigned epoch, signed char *dig, double *stat,
-                                         long long *tr, long long *tp) {
+                                         long long *tr, long long *tp, int xr_m0 = 0) {
+    // xr_m0: the first of the NM products among those the publisher wrote records for
     constexpr int C = 512 * KW, G = 32 * KW, FT = 64 * FW, NQ = C / 4, NQT = (NQ + FT - 1) / FT;
     constexpr int PS = C + 64;
     static_assert(FW >= 4, "one front wave per product plus wave 0");
@@ -573,7 +590,7 @@ __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, co
         const int m = fx.wave - 1;
         if (m < NM) {
             RowPoll<3, G> r;
-            r.poll(fx, a.b.XR + (size_t)(kStatRows + 3 * m) * G, epoch);
+            r.poll(fx, a.b.XR + (size_t)(kStatRows + 3 * (xr_m0 + m)) * G, epoch);
             const float mx = wave_max_dpp(r.lane_max(fx, 0));
             const double so = wave_sum_dpp(r.lane_sum(fx, 1) + r.lane_sum(fx, 2));
             if (fx.lane == 0) { stat[2 + 2 * m] = (double)mx; stat[3 + 2 * m] = so; }
@@ -618,10 +635,10 @@ __device__ __forceinline__ void ln_front(Front &fx, int &seq, const DArgs &a, co
 // Front side of a product whose input was scaled by its producers (att output, ffn value):
 // the records carry max |xs| and the shares of the zero-point sum.  Leaves the scale in stat[16],
 // the zero-point sum in stat[17].  Ends with the "digits ready" barrier.
-template <int KW, int FW, int NQT>
+template <int KW, int FW, int NQT, int G = 32 * KW>     // G: workgroups that publish a record each
 __device__ __forceinline__ void vec_front(Front &fx, int &seq, const u64 *src, const u64 *rec, int nq, unsigned epoch,
                                           signed char *dig, int plane_stride, double *stat, long long *tr, long long *tp) {
-    constexpr int G = 32 * KW, FT = 64 * FW;
+    constexpr int FT = 64 * FW;
     constexpr int CH = NQT <= 5 ? NQT : ((NQT + 1) / 2 <= 5 ? (NQT + 1) / 2 : 3), NCH = (NQT + CH - 1) / CH;
     fx.refresh();
     ++seq;
@@ -666,7 +683,9 @@ __device__ __forceinline__ void vec_front(Front &fx, int &seq, const u64 *src, c
 }
 
 // =============================================================================
-template <int KW, int FW, bool TRACE>
+template <int KW, int FW, bool HELP> using BackOf = std::conditional_t<HELP, BackCfgH<KW, FW>, BackCfg<KW, FW>>;
+
+template <int KW, int FW, bool TRACE, bool HELP>
 __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, const v4i *red, double *stat, double *rf_lds,
                                            lds_flag_t *flags, u64 *own_lds, double *st_lds, long long *trace_lds) {
     constexpr int C = 512 * KW, F = 4 * C, G = GroupShape<KW>::G, NT = GroupShape<KW>::NT, NWG = GroupShape<KW>::NWG, FT = 64 * FW;
@@ -773,14 +792,22 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
         if (tr && fx.tid == 0) tr[8] = wall_clock64();
 
         // ===================== phase 3: ffn receptance + key ===================
-        ln_front<KW, FW, 2>(fx, seq, a, P32, Q32, rec, 3, e + 2u, dig, stat, tr ? tr + 9 : nullptr, tr ? tr + 18 : nullptr);   // [0] ffn_k, [1] ffn_r
+        if constexpr (HELP)      // the ffn key tiles are the helper workgroups': the receptance alone, second of the two products published
+            ln_front<KW, FW, 1>(fx, seq, a, P32, Q32, rec, 4, e + 2u, dig, stat, tr ? tr + 9 : nullptr, tr ? tr + 18 : nullptr, 1);
+        else
+            ln_front<KW, FW, 2>(fx, seq, a, P32, Q32, rec, 3, e + 2u, dig, stat, tr ? tr + 9 : nullptr, tr ? tr + 18 : nullptr);   // [0] ffn_k, [1] ffn_r
         if (!fx.ok) break;
         RWKV_IDS();
         // the LayerNorm output of the own channel is the new ffn shift state (block.py:82,87-88)
         if (fin && row == 0) put_state(1, n, or_d(rec, OR_LN2W * 16 + n) * ((x_lds[n] - stat[0]) * stat[1]) + or_d(rec, OR_LN2B * 16 + n));
         __syncthreads();
         if (tr && fx.tid == 0) tr[11] = wall_clock64();
-        if (fin) {
+        if constexpr (HELP) {
+            if (fin && row == 0) {                         // the receptance gate of the own channels (block.py:95)
+                const double yr = finish_col(red, 0, n, stat[8], (int)or_hi(rec, OR_CSR_CSFR * 16 + n), stat[9]);
+                rf_lds[n] = (double)sigmoid_f32((float)yr);
+            }
+        } else if (fin) {
             // parked tiles: 0 = ffn_r, 1..4 = ffn_k tiles g, g+G, g+2G, g+3G
             const int f_own = 16 * (g + G * row) + n;      // column of ffn_k tile `row`
             const double y = finish_col(red, 1 + row, n, stat[8], (int)or_hi(rec, kOrRngVCs + lane), stat[9]);
@@ -800,7 +827,8 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
         if (tr && fx.tid == 0) tr[12] = wall_clock64();
 
         // ===================== phase 4: ffn value ==============================
-        vec_front<KW, FW, NQTH>(fx, seq, a.b.H, a.b.HR, NQH, e + 3u, dig, PSF, stat, tr ? tr + 13 : nullptr, tr ? tr + 19 : nullptr);
+        vec_front<KW, FW, NQTH, HELP ? HelperShape<KW>::NH : G>(fx, seq, a.b.H, a.b.HR, NQH, e + 3u, dig, PSF, stat, tr ? tr + 13 : nullptr,
+                                                                tr ? tr + 19 : nullptr);
         if (!fx.ok) break;
         __syncthreads();
         if (tr && fx.tid == 0) tr[15] = wall_clock64();
@@ -843,7 +871,7 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
     RWKV_IDS();
 #undef RWKV_IDS
     unsigned par = 0;
-    constexpr int NS = BackCfg<KW, FW>::NS;               // head tiles per barrier round
+    constexpr int NS = BackOf<KW, FW, HELP>::NS;          // head tiles per barrier round
     double Sh;
     float invSh;
     ln_scale(stat, rec_h, 0, 0, Sh, invSh);
@@ -879,29 +907,248 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
         for (int i = fx.tid; i < L * kTraceStampsPerLayer; i += FT) a.b.trace[(size_t)wg * L * kTraceStampsPerLayer + i] = trace_lds[i];
 }
 
+
+// =============================================================================
+// A helper workgroup (see HelperShape): all of its wavefronts gather and quantise the ffn phase's input, wavefront
+// w multiplies NTW neighbouring tiles over one part of the contraction (every digit fragment it reads from LDS serves
+// NTW matrix instructions: with one tile per wavefront the LDS reads of the fragments took longer than the matrix
+// cores), wavefront 0 finishes the columns.
+// Three workgroup barriers per layer, each followed by a test of the abort word, so that every wavefront leaves
+// after the same barrier.
 template <int KW, int FW>
+__device__ __forceinline__ void helper_path(const DArgs &a, signed char *dig, v4i *red, double *stat, lds_flag_t *flags,
+                                            v4i *stash) {
+    constexpr int C = 512 * KW, G = GroupShape<KW>::G, NWG = GroupShape<KW>::NWG;
+    constexpr int NH = HelperShape<KW>::NH, TPH = HelperShape<KW>::TILES, NWV = FW + kBW, FT = 64 * NWV;
+    // NTW tiles per wavefront, WPT wavefronts (parts of the contraction) per tile, KB blocks per tile, KPW blocks of
+    // the contraction per wavefront, BPW weight blocks per wavefront
+    constexpr int NTW = 2, WPT = NWV * NTW / TPH, KB = 8 * KW, KPW = KB / WPT, BPW = NTW * KPW;
+    static_assert(TPH % NTW == 0 && (TPH / NTW) * WPT == NWV && WPT * KPW == KB && TPH * 16 == 128 && NWV >= 3, "helper shape");
+    // Of a wavefront's BPW blocks the last BLDS wait in LDS (64 lanes x 16 bytes each, `stash`), the others in
+    // registers: all of them in registers would leave too few for the gather and the digits, and the compiler
+    // would park blocks in scratch memory - a reload from memory in the middle of the phase.
+    constexpr int BLDS = HelperShape<KW>::LDS_BLOCKS, BREG = BPW - BLDS, KREG = BREG / NTW;      // per tile: blocks 0 .. KREG - 1 in registers
+    static_assert(BLDS % NTW == 0, "the same blocks of every tile wait in LDS");
+    constexpr int PS = C + 64, NQ = C / 4, NQT = (NQ + FT - 1) / FT, MFK = 3;      // MFK: the ffn key product in the layer's tables
+    Front fx;
+    fx.abort_flag = a.b.abort_flag; fx.flags = flags; fx.spin_limit = a.spin_limit; fx.ok = true;
+    fx.refresh();
+    const int h = (int)blockIdx.x - NWG, L = a.m.L;
+    const int tile0 = h * TPH;
+    int seq = 0;
+    v4i W[BREG];
+    auto load_weights = [&](int l, bool paced) {
+        const int tid = opaque((int)threadIdx.x), wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+        // block b (of KPW) of tile t (of NTW) of this wavefront: tile tile0 + NTW (wv / WPT) + t, contraction block KPW (wv % WPT) + b
+        const uint8_t *base = gld(&a.m.layers[l].w[MAT_FFN_K]) + ((size_t)(tile0 + NTW * (wv / WPT)) * KB + (size_t)(wv % WPT) * KPW) * 1024 + (tid & 63) * 16;
+        auto blk = [&](int t, int b) { return (const RWKV_GLOBAL v4i *)(base + ((size_t)t * KB + b) * 1024); };
+        // The helpers' 26 MB per layer are not wanted anywhere for a whole layer: they are requested a few blocks at a
+        // time with pauses in between (about 10 us in all), so that they never stand as one burst in front of the
+        // owners' polls, gathers and weight stream.  (`paced` is off for the first layer, before anything runs.)
+        v4i T[BLDS];
+#pragma unroll
+        for (int i = 0; i < BLDS; ++i) {
+            if (paced && RWKV_T_PACE && i % 3 == 0) asm volatile("s_sleep %0" :: "n"(RWKV_T_PACE) : "memory");
+            T[i] = *blk(i / (KPW - KREG), KREG + i % (KPW - KREG));
+        }
+#pragma unroll
+        for (int i = 0; i < BREG; ++i) {
+            if (paced && RWKV_T_PACE && i % 3 == 0) asm volatile("s_sleep %0" :: "n"(RWKV_T_PACE) : "memory");
+            W[i] = *blk(i / KREG, i % KREG);
+        }
+#pragma unroll
+        for (int i = 0; i < BLDS; ++i) stash[(wv * BLDS + i) * 64 + (tid & 63)] = T[i];
+        // The blocks are needed a whole layer later; left alone, the compiler moves the loads down to their use,
+        // into the critical path of the ffn phase.  Naming the values here pins the loads (and their wait) to this
+        // point, where the helper has nothing else to do.
+#pragma unroll
+        for (int i = 0; i < BREG; ++i) asm volatile("" : "+v"(W[i]));
+    };
+    load_weights(0, false);
+    for (int l = 0; l < L; ++l) {
+        fx.refresh();
+        const unsigned e = a.epoch0 + 4u * (unsigned)l + 2u;      // the input of the ffn phase
+        // stamps of a helper: [0] records seen, [1] statistics, [2] digits, [3] tiles parked, [4] published, [5] next weights here
+        long long *tr = (a.b.trace && fx.tid == 0) ? a.b.trace + ((size_t)blockIdx.x * L + l) * kTraceStampsPerLayer : nullptr;
+        const float *P32 = a.m.P32 + ((size_t)l * kLnMats + MFK) * C, *Q32 = a.m.Q32 + ((size_t)l * kLnMats + MFK) * C;
+        // constants, requested before any waiting
+        float4 P[NQT], Q[NQT];
+#pragma unroll
+        for (int i = 0; i < NQT; ++i) {
+            const int qi = fx.tid + FT * i;
+            if (qi < NQ) { P[i] = *reinterpret_cast<const float4 *>(P32 + 4 * qi); Q[i] = *reinterpret_cast<const float4 *>(Q32 + 4 * qi); }
+        }
+        int csc[2] = {0, 0};
+        float rgv[2] = {0.f, 0.f};
+        double ofv[2] = {0.0, 0.0};
+        if (fx.wave == 0) {                                // the columns this lane finishes: lane and lane + 64 of the helper's 128
+            const DPrep &pr = a.m.prep[l];
+            const float *rv = gld(&pr.range_v);
+            const double *ov = gld(&pr.offset_v);
+            const int *csl = a.m.cs + (size_t)l * (6 * C + 4 * C) + 5 * C;
+#pragma unroll
+            for (int cc = 0; cc < 2; ++cc) {
+                const int f = 16 * tile0 + fx.lane + 64 * cc;
+                csc[cc] = gld(csl + f); rgv[cc] = gld(rv + f); ofv[cc] = gld(ov + f);
+            }
+        }
+        // (as with the weights: without these the compiler moves the loads, two of them through a pointer that is
+        // itself loaded, down into the epilogue)
+#pragma unroll
+        for (int i = 0; i < NQT; ++i) {
+            asm volatile("" : "+v"(P[i].x), "+v"(P[i].y), "+v"(P[i].z), "+v"(P[i].w));
+            asm volatile("" : "+v"(Q[i].x), "+v"(Q[i].y), "+v"(Q[i].z), "+v"(Q[i].w));
+        }
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) asm volatile("" : "+v"(csc[cc]), "+v"(rgv[cc]), "+v"(ofv[cc]));
+        if (fx.wave == 2 && fx.lane == 0) {                // the product's scalars (the per-token ones: parts in a fixed order)
+            const DScal *sc = a.m.sc + l, *sp = a.m.scp + (size_t)l * KW;
+            double sq = 0.0;
+            float mq = 0.f;
+#pragma unroll
+            for (int q = 0; q < KW; ++q) { sq += gld(&sp[q].sumQO[MFK]); mq = fmaxf(mq, gld(&sp[q].maxQ[MFK])); }
+            stat[20] = gld(&sc->sumPO[MFK]); stat[21] = sq; stat[22] = (double)gld(&sc->maxP[MFK]); stat[23] = (double)mq;
+        }
+        ++seq;
+        u64 w[NQT][4];
+        const xtab_t xt = make_xtab(a.b.X, C);
+        if (fx.wave == 0) {
+            RowPoll<kStatRows, G> r;
+            r.poll(fx, a.b.XR, e, seq, kStatRows * (G / kEarlyDiv), [&] { issue_quads<FT, NQT>(xt, fx.tid, 0, NQ, w); });
+            const double mean = wave_sum_dpp(r.lane_sum(fx, 0)) * (1.0 / (double)C);
+            const double var = wave_sum_dpp(r.lane_sum(fx, 1) + r.lane_group_dev2(fx, 0, mean)) * (1.0 / (double)C);
+            const double rsd = 1.0 / sqrt(var + 1e-5);                 // layernorm.py:15-20
+            if (fx.lane == 0) { stat[0] = mean; stat[1] = rsd; }
+            if (tr) gst(tr + 0, (long long)wall_clock64());
+        } else {
+            wait_flag(fx, FLAG_ARRIVED, seq);
+            issue_quads<FT, NQT>(xt, fx.tid, 0, NQ, w);
+            if (fx.wave == 1) {
+                RowPoll<3, G> r;
+                r.poll(fx, a.b.XR + (size_t)kStatRows * G, e);          // the records of the first product published: ffn key
+                const float mx = wave_max_dpp(r.lane_max(fx, 0));
+                const double so = wave_sum_dpp(r.lane_sum(fx, 1) + r.lane_sum(fx, 2));
+                if (fx.lane == 0) { stat[2] = (double)mx; stat[3] = so; }
+            }
+        }
+        __syncthreads();                                               // statistics
+        if (flags[FLAG_ABORT]) break;
+        if (tr) gst(tr + 1, (long long)wall_clock64());
+        const double mean = stat[0], rsd = stat[1];
+        double S;
+        float invS;
+        {
+            const double bound = rsd * (stat[2] + fabs(mean) * stat[22]) + stat[23];
+            scale_from_amax((float)(bound * 1.000001) + 1e-37f, S, invS);
+        }
+        const double zp = rsd * (stat[3] - mean * stat[20]) + stat[21];
+        settle_quads<FT, NQT>(fx, xt, 0, NQ, e, w);
+#pragma unroll
+        for (int i = 0; i < NQT; ++i) {
+            const int qi = fx.tid + FT * i;
+            if (qi < NQ) {
+                const float p[4] = {P[i].x, P[i].y, P[i].z, P[i].w}, qq[4] = {Q[i].x, Q[i].y, Q[i].z, Q[i].w};
+                int q[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const float t = (float)(((double)__uint_as_float((unsigned)w[i][k]) - mean) * rsd);
+                    q[k] = __float2int_rn(fmaf(t, p[k], qq[k]) * invS);                             // matmul.py:131
+                }
+                write_digits4(dig, PS, 4 * qi, q[0], q[1], q[2], q[3]);
+            }
+        }
+        __syncthreads();                                               // digits ready
+        if (flags[FLAG_ABORT]) break;
+        fx.refresh();
+        tr = (a.b.trace && fx.tid == 0) ? a.b.trace + ((size_t)blockIdx.x * L + l) * kTraceStampsPerLayer : nullptr;
+        if (tr) gst(tr + 2, (long long)wall_clock64());
+        {
+            // A operand: lane 16 g4 + m holds bytes 16 g4 .. 16 g4 + 15 of digit plane m & 3 of a 64-row block
+            const int part = fx.wave % WPT;
+            const signed char *ap = dig + (fx.lane & 3) * PS + 16 * (fx.lane >> 4) + 64 * (part * KPW);
+            const v4i *sp = stash + (fx.wave * BLDS) * 64 + fx.lane;
+            // LDS reads run two blocks ahead of the matrix instructions that take them
+            v4i A[3], acc[NTW], Bl[2][NTW];
+#pragma unroll
+            for (int t = 0; t < NTW; ++t) acc[t] = v4i{0, 0, 0, 0};
+            A[0] = *reinterpret_cast<const v4i *>(ap); A[1] = *reinterpret_cast<const v4i *>(ap + 64);
+#pragma unroll
+            for (int b = 0; b < KPW; ++b) {
+                if (b + 2 < KPW) A[(b + 2) % 3] = *reinterpret_cast<const v4i *>(ap + 64 * (b + 2));
+                if (b + 1 >= KREG && b + 1 < KPW) {
+#pragma unroll
+                    for (int t = 0; t < NTW; ++t) Bl[(b + 1) & 1][t] = sp[(t * (KPW - KREG) + (b + 1 - KREG)) * 64];
+                }
+#pragma unroll
+                for (int t = 0; t < NTW; ++t)
+                    acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[b % 3], b < KREG ? W[t * KREG + (b < KREG ? b : 0)] : Bl[b & 1][t], acc[t], 0, 0, 0);
+            }
+            // rows 0..3 of a result: the four digit sums of column `lane`; parked per (tile of the helper, part)
+            if (fx.lane < 16) {
+#pragma unroll
+                for (int t = 0; t < NTW; ++t) red[((NTW * (fx.wave / WPT) + t) * WPT + part) * 16 + fx.lane] = acc[t];
+            }
+        }
+        __syncthreads();                                               // partial tiles parked
+        if (tr) gst(tr + 3, (long long)wall_clock64());
+        if (fx.wave == 0) {
+            float xs2[2], mx = 0.f;
+            double so = 0.0;
+#pragma unroll
+            for (int cc = 0; cc < 2; ++cc) {
+                const int col = fx.lane + 64 * cc, tile = col >> 4, n = col & 15;
+                int d0 = 0, d1 = 0, d2 = 0, d3 = 0;
+#pragma unroll
+                for (int pt = 0; pt < WPT; ++pt) { const v4i v = red[(tile * WPT + pt) * 16 + n]; d0 += v.x; d1 += v.y; d2 += v.z; d3 += v.w; }
+                const double tot = fma(fma(fma((double)d0, 256.0, (double)d1), 256.0, (double)d2), 256.0, (double)d3);
+                const double y = fma(S, tot + (double)(0x808080LL * (long long)csc[cc]), zp);
+                const double hv = y > 0.0 ? y : 0.0;                                             // block.py:97-98
+                const double hh = hv * hv;
+                xs2[cc] = (float)(hh * (double)rgv[cc]);
+                put_word(a.b.H + 16 * tile0 + col, e + 1u, xs2[cc]);
+                mx = fmaxf(mx, fabsf(xs2[cc]));
+                so += hh * ofv[cc] + 128.0 * (double)xs2[cc];
+            }
+            mx = wave_max_dpp(mx);
+            so = wave_sum_dpp(so);
+            const float hi = (float)so, lo = (float)(so - (double)hi);
+            if (fx.lane < 3) put_word(a.b.HR + (size_t)fx.lane * NH + h, e + 1u, fx.lane == 0 ? mx : (fx.lane == 1 ? hi : lo));
+        }
+        if (tr) gst(tr + 4, (long long)wall_clock64());
+        if (l + 1 < L) load_weights(l + 1, true);           // a whole layer ahead of their use, after the results are out
+        if (tr) gst(tr + 5, (long long)wall_clock64());
+    }
+}
+
+template <int KW, int FW, bool HELP = false>
 struct DecodeLds {
+    using Back = BackOf<KW, FW, HELP>;
     static constexpr int C = 512 * KW, F = 4 * C, NT = GroupShape<KW>::NT;
     static constexpr int PS = C + 64, PSF = F + 64;
     static constexpr int DIG_BYTES = (3 * 4 * PS > 4 * PSF) ? 3 * 4 * PS : 4 * PSF;
-    static constexpr int RED_SLOTS = BackCfg<KW, FW>::RED_SLOTS;
+    static constexpr int RED_SLOTS = Back::RED_SLOTS;
     static constexpr int RED_BYTES = RED_SLOTS * kBW * 16 * 16;
     static constexpr int STAT_BYTES = 32 * 8, RF_BYTES = NT * 32 * 8, FLAG_BYTES = FLAG_COUNT * 4;   // RF: gate and residual of the own channels
     static constexpr int OWN_OFFSET = DIG_BYTES + RED_BYTES + STAT_BYTES + RF_BYTES + FLAG_BYTES;
     static constexpr int STATE_OFFSET = OWN_OFFSET + NT * 2 * kOrSlots * 8;
     static __host__ __device__ int state_bytes(int L) { return NT == 1 ? L * 5 * 16 * 8 : 0; }  // the new state rows of the own channels
+    // a helper workgroup's stash of weight blocks lies over the owner records and state rows, which it does not have
+    static constexpr int STASH_OFFSET = OWN_OFFSET;
+    static constexpr int STASH_BYTES = HELP ? (FW + kBW) * HelperShape<KW>::LDS_BLOCKS * 1024 : 0;
     static __host__ __device__ int total(int L, bool trace = false) {                           // (+ the stamps)
-        return STATE_OFFSET + state_bytes(L) + (trace ? L * kTraceStampsPerLayer * 8 : 0);
+        const int own = STATE_OFFSET + state_bytes(L);
+        return (own > STASH_OFFSET + STASH_BYTES ? own : STASH_OFFSET + STASH_BYTES) + (trace ? L * kTraceStampsPerLayer * 8 : 0);
     }
     // the generated back-wave program addresses LDS by these offsets
-    static_assert(BackCfg<KW, FW>::RED == DIG_BYTES, "parked tiles follow the digit planes");
-    static_assert(BackCfg<KW, FW>::FLAG == DIG_BYTES + RED_BYTES + STAT_BYTES + RF_BYTES + FLAG_ABORT * 4, "abort flag offset");
-    static_assert(RED_SLOTS >= kSlotsPerGroup * NT && RED_SLOTS >= 2 * BackCfg<KW, FW>::NS, "park slots");
+    static_assert(Back::RED == DIG_BYTES, "parked tiles follow the digit planes");
+    static_assert(Back::FLAG == DIG_BYTES + RED_BYTES + STAT_BYTES + RF_BYTES + FLAG_ABORT * 4, "abort flag offset");
+    static_assert(RED_SLOTS >= kSlotsPerGroup * NT && RED_SLOTS >= 2 * Back::NS, "park slots");
+    static_assert(!HELP || RED_BYTES >= (FW + kBW) * 2 * 256, "a helper's parked partial tiles: two per wavefront");
 };
 
-template <int KW, int FW, bool TRACE>
+template <int KW, int FW, bool TRACE, bool HELP>
 __global__ void __launch_bounds__((FW + kBW) * 64) decode_kernel(const DArgs a) {
-    using Lds = DecodeLds<KW, FW>;
+    using Lds = DecodeLds<KW, FW, HELP>;
     extern __shared__ __align__(16) unsigned char smem[];
     signed char *dig = reinterpret_cast<signed char *>(smem);
     v4i *red = reinterpret_cast<v4i *>(smem + Lds::DIG_BYTES);
@@ -912,15 +1159,21 @@ __global__ void __launch_bounds__((FW + kBW) * 64) decode_kernel(const DArgs a) 
     if (threadIdx.x < FLAG_COUNT) flags[threadIdx.x] = 0;
     __syncthreads();
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    if constexpr (HELP) {
+        if ((int)blockIdx.x >= GroupShape<KW>::NWG) {          // (uniform for the workgroup)
+            helper_path<KW, FW>(a, dig, red, stat, flags, reinterpret_cast<v4i *>(smem + Lds::STASH_OFFSET));
+            return;
+        }
+    }
     if (wave < FW) {
-        front_path<KW, FW, TRACE>(a, dig, red, stat, rf_lds, flags, reinterpret_cast<u64 *>(smem + Lds::OWN_OFFSET),
+        front_path<KW, FW, TRACE, HELP>(a, dig, red, stat, rf_lds, flags, reinterpret_cast<u64 *>(smem + Lds::OWN_OFFSET),
                                   reinterpret_cast<double *>(smem + Lds::STATE_OFFSET),
                                   reinterpret_cast<long long *>(smem + Lds::total(a.m.L)));       // (total without the stamps = where they start)
     } else {
         constexpr int NWG = GroupShape<KW>::NWG;
         const int v_tiles = (a.m.V + 15) / 16, head_rounds = (v_tiles + NWG - 1) / NWG;
         const unsigned lds = (unsigned)(uintptr_t)(RWKV_LDS unsigned char *)smem;
-        BackCfg<KW, FW>::run(a.m.jt + (size_t)blockIdx.x * (a.m.L + 1) * 16, a.m.w_head, a.m.L, head_rounds, v_tiles,
+        BackOf<KW, FW, HELP>::run(a.m.jt + (size_t)blockIdx.x * (a.m.L + 1) * 16, a.m.w_head, a.m.L, head_rounds, v_tiles,
                          (int)blockIdx.x, wave - FW, lds);
     }
 }
@@ -1250,6 +1503,7 @@ bool decode_supported(int64_t L, int64_t C, int64_t F, int64_t V) {
 }
 
 int64_t decode_workgroups(int64_t C) { return C > 4096 ? C / 32 : C / 16; }
+int64_t decode_helper_workgroups(int64_t C) { return C == 2560 ? HelperShape<5>::NH : 0; }
 
 unsigned decode_epochs_per_token(int64_t L) { return (unsigned)(4 * L + 1); }
 
@@ -1386,8 +1640,9 @@ constexpr int kMaxDevices = 64;
 
 template <int KW, int FW>
 static int launch_one(hipStream_t st, const DArgs &args, bool with_prep) {
+    constexpr bool HELP = HelperShape<KW>::NH > 0;
     const bool trace = args.b.trace != nullptr;
-    const int lds = DecodeLds<KW, FW>::total(args.m.L, trace);
+    const int lds = DecodeLds<KW, FW, HELP>::total(args.m.L, trace);
     if (lds > 160 * 1024) return set_error(RWKV_ERR_SIZE, "decode kernel: %d layers need %d bytes of LDS", args.m.L, lds);
     // the dynamic LDS limit is a per-device attribute of the function; it only ever grows
     static std::mutex mu;
@@ -1398,9 +1653,9 @@ static int launch_one(hipStream_t st, const DArgs &args, bool with_prep) {
     {
         std::lock_guard<std::mutex> lock(mu);
         if (configured[dev] < lds) {
-            RWKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_kernel<KW, FW, false>),
+            RWKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_kernel<KW, FW, false, HELP>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-            RWKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_kernel<KW, FW, true>),
+            RWKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_kernel<KW, FW, true, HELP>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds));
             configured[dev] = lds;
         }
@@ -1409,10 +1664,12 @@ static int launch_one(hipStream_t st, const DArgs &args, bool with_prep) {
         hipLaunchKernelGGL(prep_kernel, dim3((unsigned)(args.m.L * (args.m.C / kPrepThreads) + 1)), dim3(kPrepThreads), 0, st, args);
         RWKV_CHECK_LAUNCH("prep_kernel");
     }
+    // owner workgroups first, then the helpers: every one of them is resident at once (one per compute unit)
+    const dim3 grid((unsigned)(args.m.NWG + HelperShape<KW>::NH));
     if (trace)
-        hipLaunchKernelGGL((decode_kernel<KW, FW, true>), dim3((unsigned)args.m.NWG), dim3((FW + kBW) * 64), lds, st, args);
+        hipLaunchKernelGGL((decode_kernel<KW, FW, true, HELP>), grid, dim3((FW + kBW) * 64), lds, st, args);
     else
-        hipLaunchKernelGGL((decode_kernel<KW, FW, false>), dim3((unsigned)args.m.NWG), dim3((FW + kBW) * 64), lds, st, args);
+        hipLaunchKernelGGL((decode_kernel<KW, FW, false, HELP>), grid, dim3((FW + kBW) * 64), lds, st, args);
     RWKV_CHECK_LAUNCH("decode_kernel");
     return RWKV_OK;
 }

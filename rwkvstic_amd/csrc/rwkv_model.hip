@@ -736,6 +736,11 @@ void rwkv_model_destroy(rwkv_model *m) {
 
 int rwkv_model_has_fused_step(const rwkv_model *m) { return (m && m->fused) ? 1 : 0; }
 
+int rwkv_model_trace_workgroups(const rwkv_model *m) {
+    if (!m || !m->fused) return 0;
+    return (int)(decode_workgroups(m->dm.C) + decode_helper_workgroups(m->dm.C));
+}
+
 int rwkv_model_set_trace(rwkv_model *m, int64_t *device_buffer) {
     RWKV_CHECK_ARG(m, "rwkv_model_set_trace: null handle");
     m->db.trace = reinterpret_cast<long long *>(device_buffer);
