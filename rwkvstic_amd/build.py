@@ -33,7 +33,7 @@ def hipcc() -> str:
 
 def build(verbose: bool = True, extra_flags=(), output: str | None = None) -> str:
     """output: write the library there instead of next to this file (diagnostic builds, e.g. with
-    ``-DRWKV_DIAG_HOT_WEIGHTS``; ``bench.py --lib`` loads such a file)."""
+    ``-DRWKV_DIAG``, the library's one diagnostic switch: weights of the single-token kernel served from cache, results wrong; ``bench.py --lib`` loads such a file)."""
     srcs = [os.path.join(CSRC, s) for s in SOURCES]
     out = os.path.abspath(output) if output else LIB
     tmp = out + ".tmp"

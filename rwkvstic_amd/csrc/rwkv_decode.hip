@@ -62,10 +62,7 @@ constexpr int kRealJobs = 13;          // tile jobs per layer: k v r | o | ffn_r
 constexpr unsigned kSpinLimit = 1u << 20;        // polls before a wait gives up (DArgs::spin_limit; a self-test passes a small one)
 constexpr int kStatRows = 2;           // XR rows 0-1: sum x of a workgroup's 16 channels, and their squared deviations from the workgroup's own mean
 constexpr int kLnRows = kStatRows + 3 * 3;     // rows of the XR record table
-#ifndef RWKV_EARLY_DIV
-#define RWKV_EARLY_DIV 4
-#endif
-constexpr int kEarlyDiv = RWKV_EARLY_DIV;           // gathers start when all but G / kEarlyDiv workgroups have published (measured flat from G/20 to G)
+constexpr int kEarlyDiv = 4;           // gathers start when all but G / kEarlyDiv workgroups have published (measured flat from G/20 to G)
 constexpr int kSlotsPerGroup = 5;      // parked-tile slots a group of 16 channels needs at once (ffn receptance + 4 ffn key tiles)
 constexpr int kHeadCsPerThread = 4;    // head column sums a front thread fetches: 16 per head tile of the workgroup
 
@@ -103,14 +100,17 @@ struct GroupShape {
 // their use), waits like everybody else for the input of the ffn phase, and publishes relu(k)^2 with its records.
 // The owner workgroups then stream 9 tiles per layer instead of 13 and have the ffn receptance tile only to
 // multiply in that phase.
-#ifndef RWKV_T_PACE
-#define RWKV_T_PACE 20
-#endif
+constexpr int kHelperPace = 20;        // s_sleep units (64 cycles) between groups of three weight loads of a helper (10 and 30: within 0.5 %; 0: +2 %, 60: +3 %)
+template <int KW>
+struct DecodeLdsDigBytes {          // bytes of the digit planes at the start of LDS (three C-row sets, or one F-row set)
+    static constexpr int value = (3 * 4 * (512 * KW + 64) > 4 * (2048 * KW + 64)) ? 3 * 4 * (512 * KW + 64) : 4 * (2048 * KW + 64);
+};
+
 template <int KW>
 struct HelperShape {
     static constexpr int NH = KW == 5 ? 80 : 0;                    // helper workgroups
     static constexpr int TILES = NH ? (4 * 32 * KW) / NH : 1;      // ffn key tiles of 16 columns per helper
-    static constexpr int LDS_BLOCKS = 6;                           // weight blocks per wavefront that wait in LDS instead of registers
+    static constexpr int LDS_BLOCKS = 4;                           // weight blocks per wavefront that wait in LDS instead of registers
 };
 
 struct DArgs {
@@ -827,7 +827,7 @@ __device__ __forceinline__ void front_path(const DArgs &a, signed char *dig, con
         if (tr && fx.tid == 0) tr[12] = wall_clock64();
 
         // ===================== phase 4: ffn value ==============================
-        vec_front<KW, FW, NQTH, HELP ? HelperShape<KW>::NH : G>(fx, seq, a.b.H, a.b.HR, NQH, e + 3u, dig, PSF, stat, tr ? tr + 13 : nullptr,
+        vec_front<KW, FW, NQTH, HELP ? 2 * HelperShape<KW>::NH : G>(fx, seq, a.b.H, a.b.HR, NQH, e + 3u, dig, PSF, stat, tr ? tr + 13 : nullptr,
                                                                 tr ? tr + 19 : nullptr);
         if (!fx.ok) break;
         __syncthreads();
@@ -922,14 +922,23 @@ __device__ __forceinline__ void helper_path(const DArgs &a, signed char *dig, v4
     constexpr int NH = HelperShape<KW>::NH, TPH = HelperShape<KW>::TILES, NWV = FW + kBW, FT = 64 * NWV;
     // NTW tiles per wavefront, WPT wavefronts (parts of the contraction) per tile, KB blocks per tile, KPW blocks of
     // the contraction per wavefront, BPW weight blocks per wavefront
-    constexpr int NTW = 2, WPT = NWV * NTW / TPH, KB = 8 * KW, KPW = KB / WPT, BPW = NTW * KPW;
+    constexpr int NTW = 4, WPT = NWV * NTW / TPH, KB = 8 * KW, KPW = KB / WPT, BPW = NTW * KPW;
     static_assert(TPH % NTW == 0 && (TPH / NTW) * WPT == NWV && WPT * KPW == KB && TPH * 16 == 128 && NWV >= 3, "helper shape");
-    // Of a wavefront's BPW blocks the last BLDS wait in LDS (64 lanes x 16 bytes each, `stash`), the others in
-    // registers: all of them in registers would leave too few for the gather and the digits, and the compiler
+    // Of a wavefront's BPW blocks the last of every tile waits in LDS (64 lanes x 16 bytes each, `stash`), the others
+    // in registers: all of them in registers would leave too few for the gather and the digits, and the compiler
     // would park blocks in scratch memory - a reload from memory in the middle of the phase.
     constexpr int BLDS = HelperShape<KW>::LDS_BLOCKS, BREG = BPW - BLDS, KREG = BREG / NTW;      // per tile: blocks 0 .. KREG - 1 in registers
-    static_assert(BLDS % NTW == 0, "the same blocks of every tile wait in LDS");
+    static_assert(BLDS == NTW && KREG == KPW - 1, "one block of every tile waits in LDS");
     constexpr int PS = C + 64, NQ = C / 4, NQT = (NQ + FT - 1) / FT, MFK = 3;      // MFK: the ffn key product in the layer's tables
+    static_assert(NQT == 1, "one group of four channels per thread");
+    // LDS behind the digit planes: this layer's constants, written by the thread that reads them back (they are
+    // fetched a whole phase early, and holding them in registers through the wait would push weight blocks out)
+    float4 *cP = reinterpret_cast<float4 *>(dig + 4 * PS), *cQ = cP + NQ;
+    int *c_cs = reinterpret_cast<int *>(cQ + NQ);
+    float *c_rg = reinterpret_cast<float *>(c_cs + 128);
+    double *c_of = reinterpret_cast<double *>(c_rg + 128);
+    static_assert(4 * PS + 2 * NQ * 16 + 128 * 16 <= DecodeLdsDigBytes<KW>::value, "constants fit between the digit planes and the parked sums");
+    int *redi = reinterpret_cast<int *>(red);              // [TPH][16 columns][4 digit sums], added to by the WPT parts of a tile
     Front fx;
     fx.abort_flag = a.b.abort_flag; fx.flags = flags; fx.spin_limit = a.spin_limit; fx.ok = true;
     fx.refresh();
@@ -940,20 +949,24 @@ __device__ __forceinline__ void helper_path(const DArgs &a, signed char *dig, v4
     auto load_weights = [&](int l, bool paced) {
         const int tid = opaque((int)threadIdx.x), wv = __builtin_amdgcn_readfirstlane(tid >> 6);
         // block b (of KPW) of tile t (of NTW) of this wavefront: tile tile0 + NTW (wv / WPT) + t, contraction block KPW (wv % WPT) + b
+#ifdef RWKV_DIAG
+        const uint8_t *base = a.m.w_head + (tid & 63) * 16;       // (see build_jobtab_kernel)
+#else
         const uint8_t *base = gld(&a.m.layers[l].w[MAT_FFN_K]) + ((size_t)(tile0 + NTW * (wv / WPT)) * KB + (size_t)(wv % WPT) * KPW) * 1024 + (tid & 63) * 16;
+#endif
         auto blk = [&](int t, int b) { return (const RWKV_GLOBAL v4i *)(base + ((size_t)t * KB + b) * 1024); };
         // The helpers' 26 MB per layer are not wanted anywhere for a whole layer: they are requested a few blocks at a
-        // time with pauses in between (about 10 us in all), so that they never stand as one burst in front of the
-        // owners' polls, gathers and weight stream.  (`paced` is off for the first layer, before anything runs.)
+        // time with pauses in between, so that they never stand as one burst in front of the owners' polls, gathers
+        // and weight stream.  (`paced` is off for the first layer, before anything runs.)
         v4i T[BLDS];
 #pragma unroll
         for (int i = 0; i < BLDS; ++i) {
-            if (paced && RWKV_T_PACE && i % 3 == 0) asm volatile("s_sleep %0" :: "n"(RWKV_T_PACE) : "memory");
-            T[i] = *blk(i / (KPW - KREG), KREG + i % (KPW - KREG));
+            if (paced && i % 3 == 0) asm volatile("s_sleep %0" :: "n"(kHelperPace) : "memory");
+            T[i] = *blk(i, KREG);
         }
 #pragma unroll
         for (int i = 0; i < BREG; ++i) {
-            if (paced && RWKV_T_PACE && i % 3 == 0) asm volatile("s_sleep %0" :: "n"(RWKV_T_PACE) : "memory");
+            if (paced && i % 3 == 0) asm volatile("s_sleep %0" :: "n"(kHelperPace) : "memory");
             W[i] = *blk(i / KREG, i % KREG);
         }
 #pragma unroll
@@ -968,39 +981,22 @@ __device__ __forceinline__ void helper_path(const DArgs &a, signed char *dig, v4
     for (int l = 0; l < L; ++l) {
         fx.refresh();
         const unsigned e = a.epoch0 + 4u * (unsigned)l + 2u;      // the input of the ffn phase
-        // stamps of a helper: [0] records seen, [1] statistics, [2] digits, [3] tiles parked, [4] published, [5] next weights here
+        // stamps of a helper: [0] records seen, [1] statistics, [2] digits, [3] tiles multiplied, [4] published, [5] next weights here
         long long *tr = (a.b.trace && fx.tid == 0) ? a.b.trace + ((size_t)blockIdx.x * L + l) * kTraceStampsPerLayer : nullptr;
-        const float *P32 = a.m.P32 + ((size_t)l * kLnMats + MFK) * C, *Q32 = a.m.Q32 + ((size_t)l * kLnMats + MFK) * C;
-        // constants, requested before any waiting
-        float4 P[NQT], Q[NQT];
-#pragma unroll
-        for (int i = 0; i < NQT; ++i) {
-            const int qi = fx.tid + FT * i;
-            if (qi < NQ) { P[i] = *reinterpret_cast<const float4 *>(P32 + 4 * qi); Q[i] = *reinterpret_cast<const float4 *>(Q32 + 4 * qi); }
+        // this layer's constants -> LDS, long before they are needed
+        if (fx.tid < NQ) {
+            const float *P32 = a.m.P32 + ((size_t)l * kLnMats + MFK) * C, *Q32 = a.m.Q32 + ((size_t)l * kLnMats + MFK) * C;
+            const float4 p4 = *reinterpret_cast<const float4 *>(P32 + 4 * fx.tid), q4 = *reinterpret_cast<const float4 *>(Q32 + 4 * fx.tid);
+            cP[fx.tid] = p4; cQ[fx.tid] = q4;
         }
-        int csc[2] = {0, 0};
-        float rgv[2] = {0.f, 0.f};
-        double ofv[2] = {0.0, 0.0};
-        if (fx.wave == 0) {                                // the columns this lane finishes: lane and lane + 64 of the helper's 128
+        if (fx.wave < 2) {                                 // the columns the two finishing wavefronts own: 64 wave + lane of the helper's 128
             const DPrep &pr = a.m.prep[l];
             const float *rv = gld(&pr.range_v);
             const double *ov = gld(&pr.offset_v);
             const int *csl = a.m.cs + (size_t)l * (6 * C + 4 * C) + 5 * C;
-#pragma unroll
-            for (int cc = 0; cc < 2; ++cc) {
-                const int f = 16 * tile0 + fx.lane + 64 * cc;
-                csc[cc] = gld(csl + f); rgv[cc] = gld(rv + f); ofv[cc] = gld(ov + f);
-            }
+            const int col = 64 * fx.wave + fx.lane, f = 16 * tile0 + col;
+            c_cs[col] = gld(csl + f); c_rg[col] = gld(rv + f); c_of[col] = gld(ov + f);
         }
-        // (as with the weights: without these the compiler moves the loads, two of them through a pointer that is
-        // itself loaded, down into the epilogue)
-#pragma unroll
-        for (int i = 0; i < NQT; ++i) {
-            asm volatile("" : "+v"(P[i].x), "+v"(P[i].y), "+v"(P[i].z), "+v"(P[i].w));
-            asm volatile("" : "+v"(Q[i].x), "+v"(Q[i].y), "+v"(Q[i].z), "+v"(Q[i].w));
-        }
-#pragma unroll
-        for (int cc = 0; cc < 2; ++cc) asm volatile("" : "+v"(csc[cc]), "+v"(rgv[cc]), "+v"(ofv[cc]));
         if (fx.wave == 2 && fx.lane == 0) {                // the product's scalars (the per-token ones: parts in a fixed order)
             const DScal *sc = a.m.sc + l, *sp = a.m.scp + (size_t)l * KW;
             double sq = 0.0;
@@ -1043,20 +1039,18 @@ __device__ __forceinline__ void helper_path(const DArgs &a, signed char *dig, v4
         }
         const double zp = rsd * (stat[3] - mean * stat[20]) + stat[21];
         settle_quads<FT, NQT>(fx, xt, 0, NQ, e, w);
+        if (fx.tid < NQ) {
+            const float4 p4 = cP[fx.tid], q4 = cQ[fx.tid];
+            const float p[4] = {p4.x, p4.y, p4.z, p4.w}, qq[4] = {q4.x, q4.y, q4.z, q4.w};
+            int q[4];
 #pragma unroll
-        for (int i = 0; i < NQT; ++i) {
-            const int qi = fx.tid + FT * i;
-            if (qi < NQ) {
-                const float p[4] = {P[i].x, P[i].y, P[i].z, P[i].w}, qq[4] = {Q[i].x, Q[i].y, Q[i].z, Q[i].w};
-                int q[4];
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const float t = (float)(((double)__uint_as_float((unsigned)w[i][k]) - mean) * rsd);
-                    q[k] = __float2int_rn(fmaf(t, p[k], qq[k]) * invS);                             // matmul.py:131
-                }
-                write_digits4(dig, PS, 4 * qi, q[0], q[1], q[2], q[3]);
+            for (int k = 0; k < 4; ++k) {
+                const float t = (float)(((double)__uint_as_float((unsigned)w[0][k]) - mean) * rsd);
+                q[k] = __float2int_rn(fmaf(t, p[k], qq[k]) * invS);                             // matmul.py:131
             }
+            write_digits4(dig, PS, 4 * fx.tid, q[0], q[1], q[2], q[3]);
         }
+        if (fx.tid >= FT - 128) red[fx.tid - (FT - 128)] = v4i{0, 0, 0, 0};      // the sums the parts will add to
         __syncthreads();                                               // digits ready
         if (flags[FLAG_ABORT]) break;
         fx.refresh();
@@ -1064,55 +1058,49 @@ __device__ __forceinline__ void helper_path(const DArgs &a, signed char *dig, v4
         if (tr) gst(tr + 2, (long long)wall_clock64());
         {
             // A operand: lane 16 g4 + m holds bytes 16 g4 .. 16 g4 + 15 of digit plane m & 3 of a 64-row block
-            const int part = fx.wave % WPT;
+            const int part = fx.wave % WPT, tq = fx.wave / WPT;
             const signed char *ap = dig + (fx.lane & 3) * PS + 16 * (fx.lane >> 4) + 64 * (part * KPW);
             const v4i *sp = stash + (fx.wave * BLDS) * 64 + fx.lane;
-            // LDS reads run two blocks ahead of the matrix instructions that take them
-            v4i A[3], acc[NTW], Bl[2][NTW];
+            // every digit fragment read from LDS serves NTW matrix instructions; the reads run two blocks ahead
+            v4i A[3], acc[NTW], Bl[NTW];
 #pragma unroll
             for (int t = 0; t < NTW; ++t) acc[t] = v4i{0, 0, 0, 0};
             A[0] = *reinterpret_cast<const v4i *>(ap); A[1] = *reinterpret_cast<const v4i *>(ap + 64);
 #pragma unroll
             for (int b = 0; b < KPW; ++b) {
                 if (b + 2 < KPW) A[(b + 2) % 3] = *reinterpret_cast<const v4i *>(ap + 64 * (b + 2));
-                if (b + 1 >= KREG && b + 1 < KPW) {
+                if (b + 2 == KPW) {
 #pragma unroll
-                    for (int t = 0; t < NTW; ++t) Bl[(b + 1) & 1][t] = sp[(t * (KPW - KREG) + (b + 1 - KREG)) * 64];
+                    for (int t = 0; t < NTW; ++t) Bl[t] = sp[t * 64];
                 }
 #pragma unroll
                 for (int t = 0; t < NTW; ++t)
-                    acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[b % 3], b < KREG ? W[t * KREG + (b < KREG ? b : 0)] : Bl[b & 1][t], acc[t], 0, 0, 0);
+                    acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[b % 3], b < KREG ? W[t * KREG + (b < KREG ? b : 0)] : Bl[t], acc[t], 0, 0, 0);
             }
-            // rows 0..3 of a result: the four digit sums of column `lane`; parked per (tile of the helper, part)
+            // rows 0..3 of a result are the four digit sums of column `lane`: integers, added in any order
             if (fx.lane < 16) {
 #pragma unroll
-                for (int t = 0; t < NTW; ++t) red[((NTW * (fx.wave / WPT) + t) * WPT + part) * 16 + fx.lane] = acc[t];
+                for (int t = 0; t < NTW; ++t) {
+                    int *dst = redi + ((NTW * tq + t) * 16 + fx.lane) * 4;
+                    atomicAdd(dst + 0, acc[t].x); atomicAdd(dst + 1, acc[t].y); atomicAdd(dst + 2, acc[t].z); atomicAdd(dst + 3, acc[t].w);
+                }
             }
         }
-        __syncthreads();                                               // partial tiles parked
+        __syncthreads();                                               // tiles multiplied
         if (tr) gst(tr + 3, (long long)wall_clock64());
-        if (fx.wave == 0) {
-            float xs2[2], mx = 0.f;
-            double so = 0.0;
-#pragma unroll
-            for (int cc = 0; cc < 2; ++cc) {
-                const int col = fx.lane + 64 * cc, tile = col >> 4, n = col & 15;
-                int d0 = 0, d1 = 0, d2 = 0, d3 = 0;
-#pragma unroll
-                for (int pt = 0; pt < WPT; ++pt) { const v4i v = red[(tile * WPT + pt) * 16 + n]; d0 += v.x; d1 += v.y; d2 += v.z; d3 += v.w; }
-                const double tot = fma(fma(fma((double)d0, 256.0, (double)d1), 256.0, (double)d2), 256.0, (double)d3);
-                const double y = fma(S, tot + (double)(0x808080LL * (long long)csc[cc]), zp);
-                const double hv = y > 0.0 ? y : 0.0;                                             // block.py:97-98
-                const double hh = hv * hv;
-                xs2[cc] = (float)(hh * (double)rgv[cc]);
-                put_word(a.b.H + 16 * tile0 + col, e + 1u, xs2[cc]);
-                mx = fmaxf(mx, fabsf(xs2[cc]));
-                so += hh * ofv[cc] + 128.0 * (double)xs2[cc];
-            }
-            mx = wave_max_dpp(mx);
-            so = wave_sum_dpp(so);
+        if (fx.wave < 2) {                                 // each of the two finishing wavefronts publishes its 64 columns and a record of its own
+            const int col = 64 * fx.wave + fx.lane;
+            const v4i d = red[col];
+            const double tot = fma(fma(fma((double)d.x, 256.0, (double)d.y), 256.0, (double)d.z), 256.0, (double)d.w);
+            const double y = fma(S, tot + (double)(0x808080LL * (long long)c_cs[col]), zp);
+            const double hv = y > 0.0 ? y : 0.0;                                                 // block.py:97-98
+            const double hh = hv * hv;
+            const float xs = (float)(hh * (double)c_rg[col]);
+            put_word(a.b.H + 16 * tile0 + col, e + 1u, xs);
+            const float mx = wave_max_dpp(fabsf(xs));
+            const double so = wave_sum_dpp(hh * c_of[col] + 128.0 * (double)xs);
             const float hi = (float)so, lo = (float)(so - (double)hi);
-            if (fx.lane < 3) put_word(a.b.HR + (size_t)fx.lane * NH + h, e + 1u, fx.lane == 0 ? mx : (fx.lane == 1 ? hi : lo));
+            if (fx.lane < 3) put_word(a.b.HR + (size_t)fx.lane * (2 * NH) + 2 * h + fx.wave, e + 1u, fx.lane == 0 ? mx : (fx.lane == 1 ? hi : lo));
         }
         if (tr) gst(tr + 4, (long long)wall_clock64());
         if (l + 1 < L) load_weights(l + 1, true);           // a whole layer ahead of their use, after the results are out
@@ -1143,7 +1131,8 @@ struct DecodeLds {
     static_assert(Back::RED == DIG_BYTES, "parked tiles follow the digit planes");
     static_assert(Back::FLAG == DIG_BYTES + RED_BYTES + STAT_BYTES + RF_BYTES + FLAG_ABORT * 4, "abort flag offset");
     static_assert(RED_SLOTS >= kSlotsPerGroup * NT && RED_SLOTS >= 2 * Back::NS, "park slots");
-    static_assert(!HELP || RED_BYTES >= (FW + kBW) * 2 * 256, "a helper's parked partial tiles: two per wavefront");
+    static_assert(DIG_BYTES == DecodeLdsDigBytes<KW>::value, "digit planes");
+    static_assert(!HELP || RED_BYTES >= HelperShape<KW>::TILES * 256, "a helper's tile sums");
 };
 
 template <int KW, int FW, bool TRACE, bool HELP>
@@ -1423,9 +1412,10 @@ __global__ void build_jobtab_kernel(const DLayer *__restrict__ layers, const uin
             const int tile = wg + NWG * j;
             p = w_head + (size_t)(tile < v_tiles ? tile : 0) * TB;
         }
-#ifdef RWKV_DIAG_HOT_WEIGHTS
-        // Diagnostic build only (results are wrong): every job streams the same cache-resident tile, which
-        // takes HBM out of the picture and leaves the time of the dependency chain between the workgroups.
+#ifdef RWKV_DIAG
+        // Diagnostic build only (-DRWKV_DIAG, the one such switch of the library; results are wrong): every job
+        // streams the same cache-resident tile, which takes HBM out of the picture and leaves the time of the
+        // dependency chain between the workgroups.
         p = w_head;
 #endif
         jt[(size_t)wg * (L + 1) * 16 + i] = (u64) reinterpret_cast<uintptr_t>(p);

@@ -586,9 +586,7 @@ struct GemmArgs {
 };
 
 constexpr int kGemmNT = 8, kGemmWideNT = 10;     // N-tiles per workgroup (two wavefronts side by side)
-#ifndef RWKV_WIDE_RING
-#define RWKV_WIDE_RING 4
-#endif
+constexpr int kWideRing = 4;                     // LDS buffers of the 64 x 160 variant
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global load
 // the wavefront has in flight, which would drain the prefetched contraction blocks at every step.
@@ -759,7 +757,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
     gemm8_body<4, 4, 3>(a);
 }
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) gemm8_wide_kernel(const GemmArgs a) {
-    gemm8_body<5, 4, RWKV_WIDE_RING>(a);
+    gemm8_body<5, 4, kWideRing>(a);
 }
 
 // ---------------------------------------------------------------------------
@@ -1311,14 +1309,8 @@ size_t rows_dig_bytes(int64_t R, int64_t K) { return (size_t)(ceil_div(R, 4) * (
 size_t rows_wkv_scratch_bytes(int64_t R, int64_t C) { return (size_t)(ceil_div(R, kWkvChunk) * 3 * C * 8); }
 constexpr int kVecFillWgs = 256;        // products of at most 8 rows: the contraction is split until there are this many workgroups
 constexpr int kMaxSplit = 8;
-#ifndef RWKV_GEMM_WIDE_NUM
-#define RWKV_GEMM_WIDE_NUM 10
-#define RWKV_GEMM_WIDE_DEN 9
-#endif
-#ifndef RWKV_GEMM_FILL
-#define RWKV_GEMM_FILL 256
-#endif
-constexpr int kGemmFillWgs = RWKV_GEMM_FILL;   // the contraction is split until the grid has this many workgroups
+constexpr int kGemmWideNum = 10, kGemmWideDen = 9;     // the 64 x 160 variant is taken when its cost is below 9/10 of the 64 x 128 variant's
+constexpr int kGemmFillWgs = 256;       // the contraction is split until the grid has this many workgroups
 
 // Which kernel serves n products of MT row tiles x NT column tiles over KB contraction blocks, its grid and
 // the number of contraction splits.  The ONE place these are decided: the launches and the sizing of the
@@ -1343,7 +1335,7 @@ static ProductPlan plan_products(int64_t MT, int64_t NT, int64_t KB, int n) {
         const int64_t w4 = ceil_div(NT, kGemmNT) * p.gy * n, w5 = ceil_div(NT, kGemmWideNT) * p.gy * n;
         const int64_t rem = w4 % 512;
         const int64_t cost4 = (w4 / 512) * 64 + (rem == 0 ? 0 : rem <= 256 ? 32 : 64), cost5 = ceil_div(w5, 256) * 40;
-        if (w4 >= 256 && RWKV_GEMM_WIDE_NUM * cost5 < RWKV_GEMM_WIDE_DEN * cost4) p.kind = PLAN_WIDE;
+        if (w4 >= 256 && kGemmWideNum * cost5 < kGemmWideDen * cost4) p.kind = PLAN_WIDE;
     }
     p.gx = (int)ceil_div(NT, p.kind == PLAN_SKINNY ? kSkinnyNT : p.kind == PLAN_WIDE ? kGemmWideNT : kGemmNT);
     // Split the contraction until the grid has a few workgroups per compute unit.
