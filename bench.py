@@ -26,7 +26,7 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E vendor peak
 # both scaled by a 1 GiB device copy in the same run; profiles/decode_kernel_3B_b1_hbm_traffic.md): a measured
 # constant per shape, not something this script can read live.  It is tied to the kernel sources it was measured on
 # by their digest (csrc_digest() below): with any other sources the bench reports null instead of a stale figure.
-PMC_TRAFFIC = {"3B": {"bytes": 2_965_300_000, "csrc_digest": "0dc82f02332f326f"}}
+PMC_TRAFFIC = {"3B": {"bytes": 2_974_128_334, "csrc_digest": "1d0f2145494a3c09"}}
 
 
 DECODE_SOURCES = ("gen_decode_back.py", "rwkv_common.h", "rwkv_decode.h", "rwkv_decode.hip", "rwkv_decode_back.inc")
