@@ -386,6 +386,21 @@ def main() -> int:
     torch.cuda.synchronize()
     prefill_ms = e0.elapsed_time(e1)
     tok = int(logits.argmax())
+    # the same prompt in 256-token chunks (the chunk size the 14B configuration prescribes): its own key of the line
+    chunked_tok_s = None
+    if chunk > 256 and args.prefill >= 512:
+        st256 = model.emptyState.clone()
+        model.forward(prompt[:256], st256.clone())
+        f0, f1 = ev(), ev()
+        torch.cuda.synchronize()
+        f0.record(stream)
+        for c0 in range(0, args.prefill, 256):
+            lg256, st256 = model.forward(prompt[c0:c0 + 256], st256)
+        f1.record(stream)
+        torch.cuda.synchronize()
+        chunked_tok_s = round(args.prefill / (f0.elapsed_time(f1) / 1e3), 1)
+        # (chunking changes the order of float operations only in the WKV scan: same token, close logits)
+        assert int(lg256.argmax()) == tok and float((lg256 - logits).abs().max()) < 1e-4, "256-token chunks disagree with the whole prompt"
 
     # ---- decode --------------------------------------------------------------
     if args.warmup > 0:
@@ -438,6 +453,7 @@ def main() -> int:
                    "weight_bytes_per_token": wbytes, "load_seconds": round(load_s, 2)},
         "prefill_tokens_per_s": round(args.prefill / (prefill_ms / 1e3), 1),
         "prefill_chunk": chunk,
+        "prefill_tokens_per_s_chunk256": chunked_tok_s,
         "roofline": {"bound": "hbm",
                      "kernel": "rwkv::decode_kernel (persistent, one launch per token; kernel_us = its own duration, launch_us = one "
                                "single-token forward call = prep_kernel + decode_kernel)"

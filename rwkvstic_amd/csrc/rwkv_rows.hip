@@ -187,7 +187,7 @@ __device__ __forceinline__ void lsum(double (&v)[N], double *red /*[N*kLW]*/) {
 }
 
 template <int NM, int NSEG, int kLT>
-__global__ void __launch_bounds__(kLT) rows_ln_mix_quant_kernel(const LnQuantArgs a) {
+__device__ __forceinline__ void ln_mix_quant_body(const LnQuantArgs &a) {
     constexpr int NO = NM > 0 ? NM : 1, kLW = kLT / 64;
     __shared__ double red[3 * kLW];
     __shared__ float redf[NO * kLW];
@@ -318,6 +318,15 @@ __global__ void __launch_bounds__(kLT) rows_ln_mix_quant_kernel(const LnQuantArg
 #pragma unroll
         for (int m = 0; m < NO; ++m) { a.S[m][t] = S[m]; a.qs[m][t] = qsum[m]; a.zp[m][t] = z[m]; }
     }
+}
+
+template <int NM, int NSEG, int kLT>
+__global__ void __launch_bounds__(kLT) rows_ln_mix_quant_kernel(const LnQuantArgs a) { ln_mix_quant_body<NM, NSEG, kLT>(a); }
+// The same for so few rows that at most two workgroups share a compute unit: twice the registers, so that the
+// parameter vectors of all of a thread's channels can be on their way at once instead of one group after the other.
+template <int NM, int NSEG, int kLT>
+__global__ void __launch_bounds__(kLT) __attribute__((amdgpu_waves_per_eu(1, 2))) rows_ln_mix_quant_few_kernel(const LnQuantArgs a) {
+    ln_mix_quant_body<NM, NSEG, kLT>(a);
 }
 
 // ---------------------------------------------------------------------------
@@ -1399,7 +1408,8 @@ int rows_ln_mix_quant(hipStream_t st, int n_mix, int64_t R, int C, bool sequence
     const bool small = many ? C <= 3 * 4 * 256 : C <= 2 * 4 * 512;
 #define RWKV_LNQ(NM)                                                                                  \
     do {                                                                                              \
-        if (many && small) hipLaunchKernelGGL((rows_ln_mix_quant_kernel<NM, 3, 256>), grid, block, 0, st, a);   \
+        if (many && small && R <= 512) hipLaunchKernelGGL((rows_ln_mix_quant_few_kernel<NM, 3, 256>), grid, block, 0, st, a);   \
+        else if (many && small) hipLaunchKernelGGL((rows_ln_mix_quant_kernel<NM, 3, 256>), grid, block, 0, st, a);   \
         else if (many) hipLaunchKernelGGL((rows_ln_mix_quant_kernel<NM, 6, 256>), grid, block, 0, st, a);       \
         else if (small) hipLaunchKernelGGL((rows_ln_mix_quant_kernel<NM, 2, 512>), grid, block, 0, st, a);      \
         else hipLaunchKernelGGL((rows_ln_mix_quant_kernel<NM, 3, 512>), grid, block, 0, st, a);                 \
