@@ -95,6 +95,24 @@ int rwkv_mm8_three(rwkv_stream_t stream, int64_t n_in, int64_t n_out,
                    const float *r0, const float *r1, const float *r2,
                    void *workspace, size_t workspace_bytes);
 
+/* The float64 instances of the two operators (the `double` branch of
+ * wrapper.cpp:60-77,95-127; kernels operators.cu:58-80,84-118): x, r, y and
+ * the sums are float64, everything else as above.  FASTQUANT itself only ever
+ * calls the float32 instances (matmul.py:58,72-74). */
+size_t rwkv_mm8_f64_workspace_bytes(int64_t n_in, int64_t n_out, int n_mat);
+int rwkv_mm8_one_f64(rwkv_stream_t stream, int64_t n_in, int64_t n_out,
+                     const double *x, const uint8_t *w, int64_t w_stride,
+                     double *y, const double *r,
+                     void *workspace, size_t workspace_bytes);
+int rwkv_mm8_three_f64(rwkv_stream_t stream, int64_t n_in, int64_t n_out,
+                       const double *x0, const double *x1, const double *x2,
+                       const uint8_t *w0, int64_t w0_stride,
+                       const uint8_t *w1, int64_t w1_stride,
+                       const uint8_t *w2, int64_t w2_stride,
+                       double *y0, double *y1, double *y2,
+                       const double *r0, const double *r1, const double *r2,
+                       void *workspace, size_t workspace_bytes);
+
 /* wkv_forward (wrapper.cpp:45-50, operators.cu:6-44), float64, reference
  * state convention: k, v, y are [B, T, C]; w (= -exp(time_decay)), u are [C];
  * aa, bb, pp are [B, C] and are updated in place; on return aa, bb hold the

@@ -16,6 +16,7 @@ EXPORTS = (
     "rwkv_version", "rwkv_last_error",
     "rwkv_mm8_workspace_bytes", "rwkv_mm8_one", "rwkv_mm8_three", "rwkv_wkv_forward_f64",
     "rwkv_mm8_one_static", "rwkv_mm8_one_static_max_bytes",
+    "rwkv_mm8_f64_workspace_bytes", "rwkv_mm8_one_f64", "rwkv_mm8_three_f64",
     "rwkv_quantize_u8", "rwkv_packed_bytes", "rwkv_pack_u8", "rwkv_unpack_u8", "rwkv_dequant_packed",
     "rwkv_packed_m16_bytes", "rwkv_pack_m16", "rwkv_unpack_m16",
     "rwkv_mm8_packed", "rwkv_mm8_m16_workspace_bytes", "rwkv_mm8_m16", "rwkv_wkv_f32",
@@ -78,6 +79,11 @@ def lib() -> C.CDLL:
     L.rwkv_mm8_one_static_max_bytes.argtypes = []
     L.rwkv_mm8_three.argtypes = [vp, i64, i64, vp, vp, vp, vp, i64, vp, i64, vp, i64,
                                  vp, vp, vp, vp, vp, vp, vp, sz]
+    L.rwkv_mm8_f64_workspace_bytes.restype = sz
+    L.rwkv_mm8_f64_workspace_bytes.argtypes = [i64, i64, ci]
+    L.rwkv_mm8_one_f64.argtypes = [vp, i64, i64, vp, vp, i64, vp, vp, vp, sz]
+    L.rwkv_mm8_three_f64.argtypes = [vp, i64, i64, vp, vp, vp, vp, i64, vp, i64, vp, i64,
+                                     vp, vp, vp, vp, vp, vp, vp, sz]
     L.rwkv_wkv_forward_f64.argtypes = [vp, i64, i64, i64] + [vp] * 8
     L.rwkv_quantize_u8.argtypes = [vp, vp, i64, i64, vp, vp, vp]
     L.rwkv_packed_bytes.restype = sz

@@ -616,18 +616,20 @@ argmax_f64_kernel(const double *__restrict__ logits, int V, int64_t *__restrict_
 // ---------------------------------------------------------------------------
 constexpr int kRefSplitRows = 128;
 
-template <int NM, int VEC>
+// T: float (operators32.cu) or double (operators.cu:58-80, the dispatch of wrapper.cpp:60-77): the type of x, r, y and
+// of the sums.
+template <typename T, int NM, int VEC>
 __global__ void __launch_bounds__(kThreads)
 mm8_ref_partial_kernel(int n_in, int n_out,
-                       const float *x0, const float *x1, const float *x2,
+                       const T *x0, const T *x1, const T *x2,
                        const uint8_t *w0, const uint8_t *w1, const uint8_t *w2,
                        int64_t s0, int64_t s1, int64_t s2,
-                       const float *r0, const float *r1, const float *r2,
-                       float *__restrict__ scratch) {
-    __shared__ float xs[NM][kRefSplitRows];
-    __shared__ float red[kWaves][NM][64 * VEC];
-    const float *xp[3] = {x0, x1, x2};
-    const float *rp[3] = {r0, r1, r2};
+                       const T *r0, const T *r1, const T *r2,
+                       T *__restrict__ scratch) {
+    __shared__ T xs[NM][kRefSplitRows];
+    __shared__ T red[kWaves][NM][64 * VEC];
+    const T *xp[3] = {x0, x1, x2};
+    const T *rp[3] = {r0, r1, r2};
     const uint8_t *wp[3] = {w0, w1, w2};
     const int64_t sp_[3] = {s0, s1, s2};
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -638,21 +640,21 @@ mm8_ref_partial_kernel(int n_in, int n_out,
         // operators32.cu:33-36 multiplies x[j] * (w * r[j]); here x[j]*r[j] is
         // formed once per row (same rounding as the reference CPU path,
         // matmul.py:131).
-        xs[m][jj] = jj < rows ? xp[m][j0 + jj] * rp[m][j0 + jj] : 0.f;
+        xs[m][jj] = jj < rows ? xp[m][j0 + jj] * rp[m][j0 + jj] : (T)0;
     }
     __syncthreads();
     const int k0 = (blockIdx.x * 64 + lane) * VEC;
-    float acc[NM][VEC];
+    T acc[NM][VEC];
 #pragma unroll
     for (int m = 0; m < NM; ++m)
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) acc[m][e] = 0.f;
+        for (int e = 0; e < VEC; ++e) acc[m][e] = (T)0;
     if (k0 < n_out) {
         for (int jj = wave; jj < rows; jj += kWaves) {
 #pragma unroll
             for (int m = 0; m < NM; ++m) {
                 const uint8_t *row = wp[m] + (size_t)(j0 + jj) * sp_[m] + k0;
-                const float xv = xs[m][jj];
+                const T xv = xs[m][jj];
                 if (VEC == 4) {
                     uint32_t d;
                     if (k0 + 4 <= n_out) {
@@ -661,12 +663,12 @@ mm8_ref_partial_kernel(int n_in, int n_out,
                         d = 0;
                         for (int e = 0; k0 + e < n_out; ++e) d |= (uint32_t)row[e] << (8 * e);
                     }
-                    acc[m][0] = fmaf(ubyte0(d), xv, acc[m][0]);
-                    acc[m][1] = fmaf(ubyte1(d), xv, acc[m][1]);
-                    acc[m][2] = fmaf(ubyte2(d), xv, acc[m][2]);
-                    acc[m][3] = fmaf(ubyte3(d), xv, acc[m][3]);
+                    acc[m][0] = fma((T)ubyte0(d), xv, acc[m][0]);
+                    acc[m][1] = fma((T)ubyte1(d), xv, acc[m][1]);
+                    acc[m][2] = fma((T)ubyte2(d), xv, acc[m][2]);
+                    acc[m][3] = fma((T)ubyte3(d), xv, acc[m][3]);
                 } else {
-                    acc[m][0] = fmaf((float)row[0], xv, acc[m][0]);
+                    acc[m][0] = fma((T)row[0], xv, acc[m][0]);
                 }
             }
         }
@@ -685,42 +687,43 @@ mm8_ref_partial_kernel(int n_in, int n_out,
     }
 }
 
-template <int NM>
+template <typename T, int NM>
 __global__ void __launch_bounds__(256)
-mm8_ref_reduce_kernel(int n_out, int n_split, const float *__restrict__ scratch,
-                      float *y0, float *y1, float *y2) {
-    float *yp[3] = {y0, y1, y2};
+mm8_ref_reduce_kernel(int n_out, int n_split, const T *__restrict__ scratch,
+                      T *y0, T *y1, T *y2) {
+    T *yp[3] = {y0, y1, y2};
     const int k = blockIdx.x * blockDim.x + threadIdx.x;
     if (k >= n_out) return;
 #pragma unroll
     for (int m = 0; m < NM; ++m) {
-        float s = 0.f;
+        T s = (T)0;
         for (int sp = 0; sp < n_split; ++sp) s += scratch[((size_t)sp * NM + m) * n_out + k];
         yp[m][k] += s;   // the reference accumulates into y (operators32.cu:38)
     }
 }
 
+template <typename T>
 static int mm8_ref_launch(hipStream_t st, int nm, int64_t n_in, int64_t n_out,
-                          const float *const x[3], const uint8_t *const w[3], const int64_t stride[3],
-                          float *const y[3], const float *const r[3], void *ws, size_t ws_bytes) {
+                          const T *const x[3], const uint8_t *const w[3], const int64_t stride[3],
+                          T *const y[3], const T *const r[3], void *ws, size_t ws_bytes) {
     RWKV_CHECK_ARG(n_in > 0 && n_out > 0 && n_in < (1 << 30) && n_out < (1 << 30), "mm8: bad sizes");
     bool vec4 = true;
     for (int m = 0; m < nm; ++m) {
         RWKV_CHECK_ARG(x[m] && w[m] && y[m] && r[m], "mm8: null pointer");
         RWKV_CHECK_ARG(stride[m] >= n_out, "mm8: w_stride < n_out");
-        RWKV_CHECK_ALIGN(x[m], 4); RWKV_CHECK_ALIGN(y[m], 4); RWKV_CHECK_ALIGN(r[m], 4);
+        RWKV_CHECK_ALIGN(x[m], sizeof(T)); RWKV_CHECK_ALIGN(y[m], sizeof(T)); RWKV_CHECK_ALIGN(r[m], sizeof(T));
         if (reinterpret_cast<uintptr_t>(w[m]) % 4 || stride[m] % 4) vec4 = false;
     }
-    const size_t need = rwkv_mm8_workspace_bytes(n_in, n_out, nm);
+    const size_t need = (size_t)(ceil_div(n_in, kRefSplitRows) * nm * n_out) * sizeof(T);
     if (!ws || ws_bytes < need)
         return set_error(RWKV_ERR_WORKSPACE, "mm8: workspace of %zu bytes needed, %zu given", need, ws_bytes);
-    RWKV_CHECK_ALIGN(ws, 4);
+    RWKV_CHECK_ALIGN(ws, sizeof(T));
     const int n_split = (int)ceil_div(n_in, kRefSplitRows);
-    float *scratch = static_cast<float *>(ws);
+    T *scratch = static_cast<T *>(ws);
     const int vec = vec4 ? 4 : 1;
     dim3 grid((unsigned)ceil_div(n_out, 64 * vec), (unsigned)n_split);
 #define LAUNCH_P(NM, VEC) \
-    hipLaunchKernelGGL((mm8_ref_partial_kernel<NM, VEC>), grid, dim3(kThreads), 0, st, (int)n_in, (int)n_out, \
+    hipLaunchKernelGGL((mm8_ref_partial_kernel<T, NM, VEC>), grid, dim3(kThreads), 0, st, (int)n_in, (int)n_out, \
                        x[0], x[1], x[2], w[0], w[1], w[2], stride[0], stride[1], stride[2], r[0], r[1], r[2], scratch)
     if (nm == 1) { if (vec4) LAUNCH_P(1, 4); else LAUNCH_P(1, 1); }
     else         { if (vec4) LAUNCH_P(3, 4); else LAUNCH_P(3, 1); }
@@ -728,9 +731,9 @@ static int mm8_ref_launch(hipStream_t st, int nm, int64_t n_in, int64_t n_out,
     RWKV_CHECK_LAUNCH("mm8_ref_partial_kernel");
     dim3 rgrid((unsigned)ceil_div(n_out, 256));
     if (nm == 1)
-        hipLaunchKernelGGL(mm8_ref_reduce_kernel<1>, rgrid, dim3(256), 0, st, (int)n_out, n_split, scratch, y[0], y[1], y[2]);
+        hipLaunchKernelGGL((mm8_ref_reduce_kernel<T, 1>), rgrid, dim3(256), 0, st, (int)n_out, n_split, scratch, y[0], y[1], y[2]);
     else
-        hipLaunchKernelGGL(mm8_ref_reduce_kernel<3>, rgrid, dim3(256), 0, st, (int)n_out, n_split, scratch, y[0], y[1], y[2]);
+        hipLaunchKernelGGL((mm8_ref_reduce_kernel<T, 3>), rgrid, dim3(256), 0, st, (int)n_out, n_split, scratch, y[0], y[1], y[2]);
     RWKV_CHECK_LAUNCH("mm8_ref_reduce_kernel");
     return RWKV_OK;
 }
@@ -781,7 +784,7 @@ int rwkv_mm8_one(rwkv_stream_t stream, int64_t n_in, int64_t n_out, const float 
     const int64_t st[3] = {w_stride, w_stride, w_stride};
     float *ys[3] = {y, y, y};
     const float *rs[3] = {r, r, r};
-    return mm8_ref_launch((hipStream_t)stream, 1, n_in, n_out, xs, ws_, st, ys, rs, workspace, workspace_bytes);
+    return mm8_ref_launch<float>((hipStream_t)stream, 1, n_in, n_out, xs, ws_, st, ys, rs, workspace, workspace_bytes);
 }
 
 size_t rwkv_mm8_one_static_max_bytes(void) {
@@ -820,7 +823,36 @@ int rwkv_mm8_three(rwkv_stream_t stream, int64_t n_in, int64_t n_out,
     const int64_t st[3] = {w0_stride, w1_stride, w2_stride};
     float *ys[3] = {y0, y1, y2};
     const float *rs[3] = {r0, r1, r2};
-    return mm8_ref_launch((hipStream_t)stream, 3, n_in, n_out, xs, ws_, st, ys, rs, workspace, workspace_bytes);
+    return mm8_ref_launch<float>((hipStream_t)stream, 3, n_in, n_out, xs, ws_, st, ys, rs, workspace, workspace_bytes);
+}
+
+size_t rwkv_mm8_f64_workspace_bytes(int64_t n_in, int64_t n_out, int n_mat) {
+    if (n_in <= 0 || n_out <= 0 || n_mat <= 0) return 0;
+    return (size_t)(ceil_div(n_in, kRefSplitRows) * n_mat * n_out) * sizeof(double);
+}
+
+int rwkv_mm8_one_f64(rwkv_stream_t stream, int64_t n_in, int64_t n_out, const double *x, const uint8_t *w,
+                     int64_t w_stride, double *y, const double *r, void *workspace, size_t workspace_bytes) {
+    const double *xs[3] = {x, x, x};
+    const uint8_t *ws_[3] = {w, w, w};
+    const int64_t st[3] = {w_stride, w_stride, w_stride};
+    double *ys[3] = {y, y, y};
+    const double *rs[3] = {r, r, r};
+    return mm8_ref_launch<double>((hipStream_t)stream, 1, n_in, n_out, xs, ws_, st, ys, rs, workspace, workspace_bytes);
+}
+
+int rwkv_mm8_three_f64(rwkv_stream_t stream, int64_t n_in, int64_t n_out,
+                       const double *x0, const double *x1, const double *x2,
+                       const uint8_t *w0, int64_t w0_stride, const uint8_t *w1, int64_t w1_stride,
+                       const uint8_t *w2, int64_t w2_stride, double *y0, double *y1, double *y2,
+                       const double *r0, const double *r1, const double *r2,
+                       void *workspace, size_t workspace_bytes) {
+    const double *xs[3] = {x0, x1, x2};
+    const uint8_t *ws_[3] = {w0, w1, w2};
+    const int64_t st[3] = {w0_stride, w1_stride, w2_stride};
+    double *ys[3] = {y0, y1, y2};
+    const double *rs[3] = {r0, r1, r2};
+    return mm8_ref_launch<double>((hipStream_t)stream, 3, n_in, n_out, xs, ws_, st, ys, rs, workspace, workspace_bytes);
 }
 
 int rwkv_wkv_forward_f64(rwkv_stream_t stream, int64_t B, int64_t T, int64_t C,

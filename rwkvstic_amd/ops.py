@@ -47,23 +47,34 @@ def _workspace(nbytes: int, device) -> torch.Tensor:
 
 
 # ---------------------------------------------------------------- reference operators
+def _mm8_dtype(x: torch.Tensor, others, what: str) -> torch.dtype:
+    """float32 or float64, shared by x, y and r (the dispatch of wrapper.cpp:58-60)."""
+    if x.dtype not in (torch.float32, torch.float64):
+        raise TypeError(f"{what}: x, y, r must be float32 or float64, got {x.dtype}")
+    for t in others:
+        _req(t, x.dtype, "x/y/r")
+    return x.dtype
+
+
 def mm8_one(N_in: int, M_out: int, x: torch.Tensor, w: torch.Tensor, y: torch.Tensor, r: torch.Tensor) -> None:
-    """``y[k] += sum_j x[j]*(w[j,k]*r[j])``; argument meaning of wrapper.cpp:52-54 (N=in, M=out)."""
-    _req(x, torch.float32, "x"); _req(y, torch.float32, "y"); _req(r, torch.float32, "r"); _req(w, torch.uint8, "w")
+    """``y[k] += sum_j x[j]*(w[j,k]*r[j])``; argument meaning of wrapper.cpp:52-54 (N=in, M=out); x, y, r all
+    float32 or all float64 (wrapper.cpp:60-77)."""
+    dt = _mm8_dtype(x, (x, y, r), "mm8_one"); _req(w, torch.uint8, "w")
     if x.dim() != 1 or x.stride(0) != 1 or y.stride(0) != 1 or w.dim() != 2 or w.stride(1) != 1:
         raise ValueError("mm8_one: x, y need unit stride and w.stride(1) == 1 (wrapper.cpp:55-57)")
     if x.numel() < N_in or r.numel() < N_in or y.numel() < M_out or w.shape[0] < N_in or w.shape[1] < M_out:
         raise ValueError("mm8_one: tensor smaller than (N, M)")
     L = N.lib()
-    ws = _workspace(L.rwkv_mm8_workspace_bytes(N_in, M_out, 1), x.device)
-    N.check(L.rwkv_mm8_one(_stream(), N_in, M_out, x.data_ptr(), w.data_ptr(), w.stride(0),
-                           y.data_ptr(), r.data_ptr(), ws.data_ptr(), ws.numel()))
+    f64 = dt == torch.float64
+    ws = _workspace((L.rwkv_mm8_f64_workspace_bytes if f64 else L.rwkv_mm8_workspace_bytes)(N_in, M_out, 1), x.device)
+    N.check((L.rwkv_mm8_one_f64 if f64 else L.rwkv_mm8_one)(_stream(), N_in, M_out, x.data_ptr(), w.data_ptr(), w.stride(0),
+                                                            y.data_ptr(), r.data_ptr(), ws.data_ptr(), ws.numel()))
 
 
 def mm8_three(N_in: int, M_out: int, x0, x1, x2, w0, w1, w2, y0, y1, y2, r0, r1, r2) -> None:
-    """Three ``mm8_one`` problems in one call (wrapper.cpp:82-86)."""
+    """Three ``mm8_one`` problems in one call (wrapper.cpp:82-86); float32 or float64 like ``mm8_one``."""
+    dt = _mm8_dtype(x0, (x0, x1, x2, y0, y1, y2, r0, r1, r2), "mm8_three")
     for t in (x0, x1, x2, y0, y1, y2, r0, r1, r2):
-        _req(t, torch.float32, "x/y/r")
         if t.stride(0) != 1:
             raise ValueError("mm8_three: x, y, r need unit stride")
     for t in (w0, w1, w2):
@@ -71,11 +82,13 @@ def mm8_three(N_in: int, M_out: int, x0, x1, x2, w0, w1, w2, y0, y1, y2, r0, r1,
         if t.dim() != 2 or t.stride(1) != 1 or t.shape[0] < N_in or t.shape[1] < M_out:
             raise ValueError("mm8_three: w must be [>=N, >=M] with unit inner stride")
     L = N.lib()
-    ws = _workspace(L.rwkv_mm8_workspace_bytes(N_in, M_out, 3), x0.device)
-    N.check(L.rwkv_mm8_three(_stream(), N_in, M_out, x0.data_ptr(), x1.data_ptr(), x2.data_ptr(),
-                             w0.data_ptr(), w0.stride(0), w1.data_ptr(), w1.stride(0), w2.data_ptr(), w2.stride(0),
-                             y0.data_ptr(), y1.data_ptr(), y2.data_ptr(),
-                             r0.data_ptr(), r1.data_ptr(), r2.data_ptr(), ws.data_ptr(), ws.numel()))
+    f64 = dt == torch.float64
+    ws = _workspace((L.rwkv_mm8_f64_workspace_bytes if f64 else L.rwkv_mm8_workspace_bytes)(N_in, M_out, 3), x0.device)
+    N.check((L.rwkv_mm8_three_f64 if f64 else L.rwkv_mm8_three)(
+        _stream(), N_in, M_out, x0.data_ptr(), x1.data_ptr(), x2.data_ptr(),
+        w0.data_ptr(), w0.stride(0), w1.data_ptr(), w1.stride(0), w2.data_ptr(), w2.stride(0),
+        y0.data_ptr(), y1.data_ptr(), y2.data_ptr(),
+        r0.data_ptr(), r1.data_ptr(), r2.data_ptr(), ws.data_ptr(), ws.numel()))
 
 
 def wkv_forward(B: int, T: int, C: int, w, u, k, v, y, aa, bb, pp) -> None:

@@ -193,6 +193,38 @@ def test_mm8_three_matches_three_mm8_one(ops):
         assert torch.equal(y3[i], y1[i])       # same kernel arithmetic, deterministic
 
 
+@pytest.mark.parametrize("n_in,n_out", [(768, 768), (130, 77), (2560, 2560), (1000, 50277)])
+def test_mm8_one_and_three_float64_instances(ops, n_in, n_out):
+    """The `double` branch of the reference's operators (wrapper.cpp:60-77, operators.cu:58-118): x, r, y and the sums
+    float64.  Against the float64 dense product at float64 rounding, accumulating into y; three problems in one call
+    equal three single calls bit for bit; the float32 instance is left as it was (dtype picks the instance)."""
+    _say(f"mm8_one/three f64 in={n_in} out={n_out}")
+    g = torch.Generator().manual_seed(n_in * 7 + n_out)
+    ws = [torch.randint(0, 256, (n_in, n_out), generator=g, dtype=torch.uint8) for _ in range(3)]
+    rs = [torch.rand(n_in, generator=g, dtype=torch.float64) * 1e-3 for _ in range(3)]
+    xs = [torch.randn(n_in, generator=g, dtype=torch.float64) for _ in range(3)]
+    y0 = [torch.randn(n_out, generator=g, dtype=torch.float64) for _ in range(3)]
+    y1 = [t.clone().cuda() for t in y0]
+    y3 = [t.clone().cuda() for t in y0]
+    dws = [w.cuda() for w in ws]
+    for i in range(3):
+        ops.mm8_one(n_in, n_out, xs[i].cuda(), dws[i], y1[i], rs[i].cuda())
+        want = y0[i] + (xs[i] * rs[i]) @ ws[i].double()
+        scale = ((xs[i].abs() * rs[i]) @ ws[i].double()).max()
+        assert (y1[i].cpu() - want).abs().max() <= 2.0 ** -52 * 64 * scale + 1e-15 * y0[i].abs().max()
+    ops.mm8_three(n_in, n_out, *[x.cuda() for x in xs], *dws, *y3, *[r.cuda() for r in rs])
+    for i in range(3):
+        assert torch.equal(y3[i], y1[i])
+    with pytest.raises(TypeError):
+        ops.mm8_one(n_in, n_out, xs[0].cuda(), dws[0], y1[0].float(), rs[0].cuda())      # mixed types, as wrapper.cpp:58 asserts
+    # through the registered operator, as scripted reference code reaches it
+    ops.register_torch_ops()
+    y = torch.zeros(n_out, dtype=torch.float64, device="cuda")
+    torch.ops.rwkv.mm8_one(n_in, n_out, xs[0].cuda(), dws[0], y, rs[0].cuda())
+    want = (xs[0] * rs[0]) @ ws[0].double()
+    assert (y.cpu() - want).abs().max() <= 2.0 ** -52 * 64 * ((xs[0].abs() * rs[0]) @ ws[0].double()).max()
+
+
 def test_mm8_one_strided_rows(ops):
     big = torch.randint(0, 256, (64, 1003), dtype=torch.uint8, device="cuda")   # odd stride: byte path
     w = big[:, :1000]
