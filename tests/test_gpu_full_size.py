@@ -6,7 +6,10 @@ random-init, fp32i8), checked through properties that do not need the CPU oracle
   integer sums on every path, so the agreement is far below the 1e-3 / 1e-4 parity bounds);
 * the persistent kernel and the per-phase kernels agree on a decoded token;
 * the device-side greedy loop equals forward() + host argmax bit for bit, and is deterministic;
-* the top of the stack: 2 of the 32 layers + head against the CPU oracle at full width.
+* the top of the stack: 2 of the 32 layers + head against the CPU oracle at full width;
+* the full depth against the CPU oracle on a model whose matrices are given directly as codes (the oracle's
+  `OracleModel.synthetic`, built in a second; quantising 3 GB of weights on the CPU would take minutes): all 32
+  (14B shape: 40) layers, a prompt through the many-row path and single tokens through the persistent kernel.
 """
 import pytest
 import torch
@@ -290,3 +293,93 @@ def test_14b_full_depth_prompt_and_single_token_kernel_agree():
     m.check()
     assert got1.tolist()[-6:] == want and got2.tolist() == got1.tolist()
     assert torch.equal(sb, sc) and torch.equal(sb, sa)
+
+
+def _state_err_against_reference_state(s_hip, s_ref):
+    """(largest shift-row difference, largest relative difference of the WKV sums) between a state of this backend,
+    converted to the reference's convention, and an oracle state."""
+    from rwkvstic_amd.model import wkv_state_to_reference
+    ra = wkv_state_to_reference(s_hip)
+    shift = float((ra[:, :2] - s_ref[:, :2]).abs().max())
+    den = torch.maximum(s_ref[:, 2].abs(), s_ref[:, 3].abs()) + 1e-300
+    wkv = float(torch.maximum((ra[:, 2] - s_ref[:, 2]).abs() / den, (ra[:, 3] - s_ref[:, 3]).abs() / den).max())
+    return shift, wkv
+
+
+def _quantized_tree(m):
+    """The oracle model's tensors under the attribute names of the reference's quantised export
+    (opt.py:31-48, block.py:13-47, matmul.py:12,67-68): what ``HipRWKV.from_quantized`` takes."""
+    t = {"emb.w": m.emb, "ln_in.weight": m.ln_in[0], "ln_in.bias": m.ln_in[1],
+         "ln_out.weight": m.ln_out[0], "ln_out.bias": m.ln_out[1]}
+
+    def put(prefix, suffix, q):
+        t[f"{prefix}weight{suffix}"] = q.codes
+        t[f"{prefix}range{suffix}"] = q.range
+        t[f"{prefix}offset{suffix}"] = q.offset
+
+    put("head.weights.0.", "", m.head)
+    for i, b in enumerate(m.blocks):
+        p = f"blocks.{i}."
+        t[p + "ln1.weight"], t[p + "ln1.bias"] = b["ln1"]
+        t[p + "ln2.weight"], t[p + "ln2.bias"] = b["ln2"]
+        put(p + "att.weights.0.", "", b["att_k"]); put(p + "att.weights.0.", "1", b["att_v"]); put(p + "att.weights.0.", "2", b["att_r"])
+        put(p + "attout.weights.0.", "", b["att_o"]); put(p + "ffnkey.weights.0.", "", b["ffn_k"])
+        put(p + "ffnreceptance.weights.0.", "", b["ffn_r"]); put(p + "ffnvalue.weights.0.", "", b["ffn_v"])
+        t[p + "attmix"], t[p + "ffnmix"] = b["attmix"], b["ffnmix"]
+        t[p + "time_first"], t[p + "time_decay"] = b["time_first"], b["time_decay"]
+    return t
+
+
+def _full_depth_oracles(shape, seed):
+    """(float32-accumulating oracle, the same model with exact accumulation), LayerNorm weights and biases random."""
+    import copy
+    L, C, F, V = shape
+    m = O.OracleModel.synthetic(L, C, F, V, seed=seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    rnd = lambda: (1.0 + 0.2 * (torch.rand(C, generator=g, dtype=torch.float64) - 0.5),          # noqa: E731
+                   0.1 * (torch.rand(C, generator=g, dtype=torch.float64) - 0.5))
+    m.ln_in, m.ln_out = rnd(), rnd()
+    for b in m.blocks:
+        b["ln1"], b["ln2"] = rnd(), rnd()
+    ex = copy.copy(m)
+    ex.matmul_dtype = torch.float64
+    as64 = lambda q: (lambda c: (setattr(c, "dtype", torch.float64), c)[1])(copy.copy(q))           # noqa: E731
+    ex.head = as64(m.head)
+    ex.blocks = [{k: (as64(v) if isinstance(v, O.QMat) else v) for k, v in b.items()} for b in m.blocks]
+    return m, ex
+
+
+@pytest.mark.parametrize("name,n_prompt,n_steps", [("3B", 24, 3), ("14B", 5, 1)])
+def test_full_depth_against_the_oracle(name, n_prompt, n_steps):
+    """Every layer of the shape, full width and vocabulary: the prompt through the many-row path, then single tokens
+    through the persistent kernel (at the 3B width with its helper workgroups), against the CPU oracle with exact
+    accumulation (logits 1e-4, shift rows 5e-5, WKV sums 1e-4 relative) and with the reference's float32
+    accumulation (1e-3, or that oracle's own distance from the exact one + 5e-4 where that is larger)."""
+    from rwkvstic_amd.model import HipRWKV
+    shape = synth.SHAPES[name]
+    V = shape[3]
+    torch.set_num_threads(16)
+    _say(f"building the {name} oracle pair and the HIP model from the same codes")
+    ref, exact = _full_depth_oracles(shape, seed=5)
+    hip = HipRWKV.from_quantized(_quantized_tree(ref))
+    assert hip.fused_step and hip.layers == shape[0]
+    prompt = synth.random_tokens(n_prompt, V=V, seed=14).tolist()
+    lr, sr = ref.forward(prompt, ref.emptyState.clone())
+    le, se = exact.forward(prompt, exact.emptyState.clone())
+    lg, sg = hip.forward(prompt, hip.emptyState.clone())
+    for i in range(n_steps + 1):
+        e32, e64 = float((lg.cpu() - lr).abs().max()), float((lg.cpu() - le).abs().max())
+        noise = float((lr - le).abs().max())
+        shift, wkv = _state_err_against_reference_state(sg.cpu(), se)
+        _say(f"  {'prompt' if i == 0 else f'token {i}'}: |gpu - fp64 oracle| {e64:.2e}  |gpu - fp32 oracle| {e32:.2e}  "
+             f"(fp32 oracle - fp64 oracle {noise:.2e})  shift {shift:.2e}  wkv {wkv:.2e}")
+        assert e64 < 1e-4 and e32 < max(1e-3, noise + 5e-4)
+        assert int(lg.argmax()) == int(le.argmax())
+        assert shift < 5e-5 and wkv < 1e-4
+        if i == n_steps:
+            break
+        t = int(le.argmax())
+        lr, sr = ref.forward([t], sr)
+        le, se = exact.forward([t], se)
+        lg, sg = hip.forward([t], sg)
+    hip.check()
