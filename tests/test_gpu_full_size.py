@@ -349,9 +349,10 @@ def _full_depth_oracles(shape, seed):
     return m, ex
 
 
-@pytest.mark.parametrize("name,n_prompt,n_steps", [("3B", 24, 3), ("14B", 5, 1)])
+@pytest.mark.parametrize("name,n_prompt,n_steps", [("3B", 24, 3), ("3B", 1024, 1), ("14B", 5, 1)])
 def test_full_depth_against_the_oracle(name, n_prompt, n_steps):
-    """Every layer of the shape, full width and vocabulary: the prompt through the many-row path, then single tokens
+    """Every layer of the shape, full width and vocabulary: the prompt through the many-row path (once at the
+    benchmark's own length of 1024 tokens: the large product kernels and the chunked WKV scan), then single tokens
     through the persistent kernel (at the 3B width with its helper workgroups), against the CPU oracle with exact
     accumulation (logits 1e-4, shift rows 5e-5, WKV sums 1e-4 relative) and with the reference's float32
     accumulation (1e-3, or that oracle's own distance from the exact one + 5e-4 where that is larger)."""
