@@ -383,4 +383,17 @@ def test_full_depth_against_the_oracle(name, n_prompt, n_steps):
         lr, sr = ref.forward([t], sr)
         le, se = exact.forward([t], se)
         lg, sg = hip.forward([t], sg)
+    if name == "14B":
+        # the configuration's batch-32 decode at the full depth: 32 sequences continue from this state with a token of
+        # their own each; the first and the last are set against the oracle
+        B = 32
+        toks = synth.random_tokens(B, V=V, seed=21)
+        sb = sg.unsqueeze(0).repeat(B, 1, 1, 1).contiguous()
+        lb, sb = hip.forward_batch(toks.cuda(), sb)
+        for b in (0, B - 1):
+            lo, so = exact.forward([int(toks[b])], se.clone())
+            e64 = float((lb[b].cpu() - lo).abs().max())
+            shift, wkv = _state_err_against_reference_state(sb[b].cpu(), so)
+            _say(f"  batch step, sequence {b}: |gpu - fp64 oracle| {e64:.2e}  shift {shift:.2e}  wkv {wkv:.2e}")
+            assert e64 < 1e-4 and int(lb[b].argmax()) == int(lo.argmax()) and shift < 5e-5 and wkv < 1e-4
     hip.check()
