@@ -187,146 +187,14 @@ __device__ __forceinline__ void lsum(double (&v)[N], double *red /*[N*kLW]*/) {
 }
 
 template <int NM, int NSEG, int kLT>
-__device__ __forceinline__ void ln_mix_quant_body(const LnQuantArgs &a) {
-    constexpr int NO = NM > 0 ? NM : 1, kLW = kLT / 64;
-    __shared__ double red[3 * kLW];
-    __shared__ float redf[NO * kLW];
-    const int t = blockIdx.x, C = a.C, tid = threadIdx.x;
-    const bool need_prev = NM > 0 && a.sequence && t > 0;
-    const double *xr = a.x + (size_t)t * C;
-    const double *pr = NM == 0 ? xr : need_prev ? xr - C : a.sequence ? a.prev0 : a.prev0 + (size_t)t * a.prev_stride;
-    double xv[NSEG][4], pv[NSEG][4], lw[NSEG][4], lb[NSEG][4];
-    double s[2] = {0.0, 0.0};
-#pragma unroll
-    for (int g = 0; g < NSEG; ++g) {
-        const int c0 = 4 * (tid + g * kLT);
-        if (c0 < C) {
-            const double2 x0 = *reinterpret_cast<const double2 *>(xr + c0), x1 = *reinterpret_cast<const double2 *>(xr + c0 + 2);
-            xv[g][0] = x0.x; xv[g][1] = x0.y; xv[g][2] = x1.x; xv[g][3] = x1.y;
-            if (NM > 0) {
-                const double2 p0 = *reinterpret_cast<const double2 *>(pr + c0), p1 = *reinterpret_cast<const double2 *>(pr + c0 + 2);
-                pv[g][0] = p0.x; pv[g][1] = p0.y; pv[g][2] = p1.x; pv[g][3] = p1.y;
-            }
-            // few rows: the LayerNorm weights travel with the row, nothing is left to fetch between the
-            // reductions; many rows: fetched where they are used, for fewer registers and more rows in flight
-#pragma unroll
-            for (int i = 0; i < 4; ++i) { s[0] += xv[g][i]; if (NM > 0) s[1] += pv[g][i]; }
-            if (kLT < 512) continue;
-            const double2 w0 = *reinterpret_cast<const double2 *>(a.ln_w + c0), w1 = *reinterpret_cast<const double2 *>(a.ln_w + c0 + 2);
-            const double2 b0 = *reinterpret_cast<const double2 *>(a.ln_b + c0), b1 = *reinterpret_cast<const double2 *>(a.ln_b + c0 + 2);
-            lw[g][0] = w0.x; lw[g][1] = w0.y; lw[g][2] = w1.x; lw[g][3] = w1.y;
-            lb[g][0] = b0.x; lb[g][1] = b0.y; lb[g][2] = b1.x; lb[g][3] = b1.y;
-        }
-    }
-    lsum<2, kLW>(s, red);
-    const double mean = s[0] / (double)C, meanp = s[1] / (double)C;
-    double q[2] = {0.0, 0.0};
-#pragma unroll
-    for (int g = 0; g < NSEG; ++g) {
-        if (4 * (tid + g * kLT) < C) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const double d = xv[g][i] - mean;
-                q[0] += d * d;
-                if (NM > 0) { const double dp = pv[g][i] - meanp; q[1] += dp * dp; }
-            }
-        }
-    }
-    lsum<2, kLW>(q, red);
-    // (one reciprocal per row instead of a float64 division per channel: the last bit of a float64 is far below
-    // anything the float32 quantiser input can see)
-    const double rsd = 1.0 / sqrt(q[0] / (double)C + 1e-5), rsdp = 1.0 / sqrt(q[1] / (double)C + 1e-5);
-    float xs[NO][NSEG][4];
-    float amax[NO];
-    double z[NO];
-#pragma unroll
-    for (int m = 0; m < NO; ++m) { amax[m] = 0.f; z[m] = 0.0; }
-#pragma unroll
-    for (int g = 0; g < NSEG; ++g) {
-        const int c0 = 4 * (tid + g * kLT);
-        if (c0 < C) {
-            double xy[4], prev[4];
-            if (kLT < 512 && NM > 0) {
-                // many rows: the previous row's values are read again here (a cache hit) instead of staying in
-                // registers through the two reductions above: 48 registers less, one more row per compute unit
-                const double2 p0 = *reinterpret_cast<const double2 *>(pr + c0), p1 = *reinterpret_cast<const double2 *>(pr + c0 + 2);
-                pv[g][0] = p0.x; pv[g][1] = p0.y; pv[g][2] = p1.x; pv[g][3] = p1.y;
-            }
-            if (kLT < 512) {
-                const double2 w0 = *reinterpret_cast<const double2 *>(a.ln_w + c0), w1 = *reinterpret_cast<const double2 *>(a.ln_w + c0 + 2);
-                const double2 b0 = *reinterpret_cast<const double2 *>(a.ln_b + c0), b1 = *reinterpret_cast<const double2 *>(a.ln_b + c0 + 2);
-                lw[g][0] = w0.x; lw[g][1] = w0.y; lw[g][2] = w1.x; lw[g][3] = w1.y;
-                lb[g][0] = b0.x; lb[g][1] = b0.y; lb[g][2] = b1.x; lb[g][3] = b1.y;
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                xy[i] = lw[g][i] * ((xv[g][i] - mean) * rsd) + lb[g][i];
-                if (NM > 0) prev[i] = need_prev ? lw[g][i] * ((pv[g][i] - meanp) * rsdp) + lb[g][i] : pv[g][i];
-            }
-#pragma unroll
-            for (int m = 0; m < NO; ++m) {
-                const float4 r = *reinterpret_cast<const float4 *>(a.range[m] + c0);
-                const float rr[4] = {r.x, r.y, r.z, r.w};
-#pragma unroll
-                for (int i = 0; i < 4; i += 2) {
-                    const double2 o = *reinterpret_cast<const double2 *>(a.offset[m] + c0 + i);
-                    double v0 = xy[i], v1 = xy[i + 1];
-                    if (NM > 0) {
-                        const double2 mu = *reinterpret_cast<const double2 *>(a.mu + (size_t)m * C + c0 + i);
-                        v0 = xy[i] * mu.x + prev[i] * (1.0 - mu.x);
-                        v1 = xy[i + 1] * mu.y + prev[i + 1] * (1.0 - mu.y);
-                    }
-                    xs[m][g][i] = (float)(v0 * (double)rr[i]);
-                    xs[m][g][i + 1] = (float)(v1 * (double)rr[i + 1]);
-                    amax[m] = fmaxf(amax[m], fmaxf(fabsf(xs[m][g][i]), fabsf(xs[m][g][i + 1])));
-                    z[m] += v0 * o.x;
-                    z[m] += v1 * o.y;
-                }
-            }
-            if (NM > 0) {
-                double *sh = !a.sequence ? a.shift_dst + (size_t)t * a.prev_stride : t == a.R - 1 ? a.shift_dst : nullptr;
-                if (sh) {
-                    *reinterpret_cast<double2 *>(sh + c0) = make_double2(xy[0], xy[1]);
-                    *reinterpret_cast<double2 *>(sh + c0 + 2) = make_double2(xy[2], xy[3]);
-                }
-            }
-        }
-    }
-#pragma unroll
-    for (int m = 0; m < NO; ++m) {
-        amax[m] = wmaxf(amax[m]);
-        if ((tid & 63) == 0) redf[m * kLW + (tid >> 6)] = amax[m];
-    }
-    lsum<NO, kLW>(z, red);                      // (its barriers also publish redf)
-    double S[NO], invS[NO], qsum[NO];
-    const int KB = C >> 6;
-#pragma unroll
-    for (int m = 0; m < NO; ++m) {
-        float am = redf[m * kLW];
-#pragma unroll
-        for (int w = 1; w < kLW; ++w) am = fmaxf(am, redf[m * kLW + w]);
-        row_scale(am, S[m], invS[m]);
-        qsum[m] = 0.0;
-#pragma unroll
-        for (int g = 0; g < NSEG; ++g) {
-            const int c0 = 4 * (tid + g * kLT);
-            if (c0 < C) qsum[m] += emit_quad(xs[m][g], invS[m], c0, t, KB, a.dig[m]);
-        }
-    }
-    lsum<NO, kLW>(qsum, red);
-    if (tid == 0) {
-#pragma unroll
-        for (int m = 0; m < NO; ++m) { a.S[m][t] = S[m]; a.qs[m][t] = qsum[m]; a.zp[m][t] = z[m]; }
-    }
+__global__ void __launch_bounds__(kLT) rows_ln_mix_quant_kernel(const LnQuantArgs a) {
+#include "rwkv_rows_ln_body.inc"
 }
-
-template <int NM, int NSEG, int kLT>
-__global__ void __launch_bounds__(kLT) rows_ln_mix_quant_kernel(const LnQuantArgs a) { ln_mix_quant_body<NM, NSEG, kLT>(a); }
 // The same for so few rows that at most two workgroups share a compute unit: twice the registers, so that the
 // parameter vectors of all of a thread's channels can be on their way at once instead of one group after the other.
 template <int NM, int NSEG, int kLT>
 __global__ void __launch_bounds__(kLT) __attribute__((amdgpu_waves_per_eu(1, 2))) rows_ln_mix_quant_few_kernel(const LnQuantArgs a) {
-    ln_mix_quant_body<NM, NSEG, kLT>(a);
+#include "rwkv_rows_ln_body.inc"
 }
 
 // ---------------------------------------------------------------------------
