@@ -1187,7 +1187,11 @@ size_t rows_wkv_scratch_bytes(int64_t R, int64_t C) { return (size_t)(ceil_div(R
 constexpr int kVecFillWgs = 256;        // products of at most 8 rows: the contraction is split until there are this many workgroups
 constexpr int kMaxSplit = 8;
 constexpr int kGemmWideNum = 10, kGemmWideDen = 9;     // the 64 x 160 variant is taken when its cost is below 9/10 of the 64 x 128 variant's
-constexpr int kGemmFillWgs = 256;       // the contraction is split until the grid has this many workgroups
+// ... except a contraction of 200 blocks and more, which splits in two while the grid is below the device (14B shape,
+// 256-token chunks: the [256 x 20480] x [20480 x 5120] product; 14,080 against 13,190 tokens/s)
+constexpr int kGemmLongFillWgs = 256, kGemmLongBlocks = 200;
+constexpr int kSkinnyFillWgs = 256;     // 9..32 rows (weight streaming): the contraction is split until the grid has this many workgroups
+constexpr int kGemmFillWgs = 96;         // larger products: split until the grid has this many workgroups.  A split costs a second launch and a round trip of the integer totals through memory, so it only pays for grids far below the device (3B shape, tokens/s in chunks of 64 / 128 / 256 / 512 tokens: 13,180 / 23,640 / 37,610 / 52,070 at 96; 12,480 / 21,280 / 34,650 / 49,380 at 256; 12,540 / 21,470 / 31,520 / 51,160 at 64)
 
 // Which kernel serves n products of MT row tiles x NT column tiles over KB contraction blocks, its grid and
 // the number of contraction splits.  The ONE place these are decided: the launches and the sizing of the
@@ -1216,7 +1220,10 @@ static ProductPlan plan_products(int64_t MT, int64_t NT, int64_t KB, int n) {
     }
     p.gx = (int)ceil_div(NT, p.kind == PLAN_SKINNY ? kSkinnyNT : p.kind == PLAN_WIDE ? kGemmWideNT : kGemmNT);
     // Split the contraction until the grid has a few workgroups per compute unit.
-    while ((int64_t)p.gx * p.gy * n * p.split < kGemmFillWgs && KB / (p.split * 2) >= 8 && p.split < kMaxSplit) p.split *= 2;
+    const int fill = p.kind == PLAN_SKINNY ? kSkinnyFillWgs : kGemmFillWgs;
+    while ((int64_t)p.gx * p.gy * n * p.split < fill && KB / (p.split * 2) >= 8 && p.split < kMaxSplit) p.split *= 2;
+    // a long contraction on a grid still below the device: one split more (two slices at most)
+    if (p.kind != PLAN_SKINNY && p.split == 1 && (int64_t)p.gx * p.gy * n < kGemmLongFillWgs && KB >= kGemmLongBlocks) p.split = 2;
     return p;
 }
 // Upper bound of the splits plan_products chooses for R rows and N columns, whatever the contraction length and

@@ -402,9 +402,11 @@ def test_pack_m16_round_trip(ops):
                                    (4, 8320, 48),       # the same with parts that have to be rounded up to whole groups of 16 values
                                    (9, 20544, 32),      # rows too long for the register-resident quantiser
                                    (20, 2560, 2560), (32, 640, 5000),    # 9..32 rows: the few-row variant with LDS staging
-                                   # 769..960 rows on a long contraction: the 160-column workgroups with the
-                                   # contraction split in two (integer slices added by the tail kernel)
-                                   (800, 2560, 2560), (900, 2560, 5120)])
+                                   # 769..960 rows on a long contraction: the 160-column workgroups (208 of them)
+                                   (800, 2560, 2560), (900, 2560, 5120),
+                                   # the 128-column workgroups with the contraction split (80 workgroups x 2,
+                                   # 20 x 4: integer slices added by the tail kernel), ragged rows
+                                   (250, 2560, 2560), (60, 10240, 2560)])
 def test_gemm8_matches_fp64_dense(ops, T, K, N):
     """Prompt GEMM (matmul.py:56-57 without its bfloat16 rounding) against the float64 dense product."""
     g = torch.Generator().manual_seed(T * 7 + K + N)

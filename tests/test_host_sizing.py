@@ -46,12 +46,23 @@ def test_totals_buffer_holds_every_slice(lib):
     assert worst > 1          # the sweep does reach split contractions
 
 
-def test_wide_variant_with_split_contraction_is_covered(lib):
-    """The 64 x 160 variant has fewer workgroups than the 64 x 128 one for the same product, so it can split the
-    contraction where the other would not: [800 x 2560] x [2560 x 2560] is such a case."""
+def test_split_contractions_are_where_the_grid_is_small(lib):
+    """A split contraction costs a second launch, so only grids far below the device split: [800 x 2560] x
+    [2560 x 2560] takes the 64 x 160 variant (208 workgroups) unsplit with the tail in its epilogue, the same
+    product for 250 rows (80 workgroups of 64 x 128) splits in two, for 60 rows (20 workgroups) in four (parts of
+    at least 8 contraction blocks)."""
     (kind, gx, gy, split), tot = _plan(lib, 800, 2560, 2560, 1)
-    assert kind == 3 and split == 2
-    assert split * 800 * 2560 * 8 <= tot
+    assert kind == 3 and split == 1 and gx * gy == 208
+    (kind, gx, gy, split), tot = _plan(lib, 250, 2560, 2560, 1)
+    assert kind == 2 and split == 2 and gx * gy == 80
+    assert split * 252 * 2560 * 8 <= tot
+    (kind, gx, gy, split), tot = _plan(lib, 60, 2560, 2560, 1)
+    assert kind == 2 and split == 4 and split * 60 * 2560 * 8 <= tot
+    # a contraction of 200 blocks and more splits once while the grid is below the device: the ffn value product of
+    # the 14B shape on a 256-token chunk (160 workgroups), not the same width's [5120 x 5120] products
+    (kind, gx, gy, split), tot = _plan(lib, 256, 20480, 5120, 1)
+    assert kind == 2 and gx * gy == 160 and split == 2 and split * 256 * 5120 * 8 <= tot
+    assert _plan(lib, 256, 5120, 5120, 1)[0][3] == 1
 
 
 def test_gemm8_workspace_covers_quantiser_scratch(lib):
