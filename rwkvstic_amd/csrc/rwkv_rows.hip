@@ -1184,13 +1184,13 @@ __global__ void __launch_bounds__(1024) mv16_kernel(const Mv16Args a) {
 // ---------------------------------------------------------------------------
 size_t rows_dig_bytes(int64_t R, int64_t K) { return (size_t)(ceil_div(R, 4) * (K / 64) * 1024); }
 size_t rows_wkv_scratch_bytes(int64_t R, int64_t C) { return (size_t)(ceil_div(R, kWkvChunk) * 3 * C * 8); }
-constexpr int kVecFillWgs = 256;        // products of at most 8 rows: the contraction is split until there are this many workgroups
+constexpr int kVecFillWgs = 128;        // products of at most 8 rows: the contraction is split until there are this many workgroups (batch step of 8 / 4 sequences, 3B shape: 3.06 / 2.64 ms at 128, 3.19 / 2.81 at 256, 3.30 / 2.94 at 512)
 constexpr int kMaxSplit = 8;
 constexpr int kGemmWideNum = 10, kGemmWideDen = 9;     // the 64 x 160 variant is taken when its cost is below 9/10 of the 64 x 128 variant's
 // ... except a contraction of 200 blocks and more, which splits in two while the grid is below the device (14B shape,
 // 256-token chunks: the [256 x 20480] x [20480 x 5120] product; 14,080 against 13,190 tokens/s)
 constexpr int kGemmLongFillWgs = 256, kGemmLongBlocks = 200;
-constexpr int kSkinnyFillWgs = 256;     // 9..32 rows (weight streaming): the contraction is split until the grid has this many workgroups
+constexpr int kSkinnyFillWgs = 128;     // 9..32 rows (weight streaming): the contraction is split until the grid has this many workgroups (batch-32 step: 8.07 ms at 128, 8.73 at 256, 9.17 at 64 for the 14B shape; 4.06 / 4.13 / 4.11 ms for the 3B shape)
 constexpr int kGemmFillWgs = 96;         // larger products: split until the grid has this many workgroups.  A split costs a second launch and a round trip of the integer totals through memory, so it only pays for grids far below the device (3B shape, tokens/s in chunks of 64 / 128 / 256 / 512 tokens: 13,180 / 23,640 / 37,610 / 52,070 at 96; 12,480 / 21,280 / 34,650 / 49,380 at 256; 12,540 / 21,470 / 31,520 / 51,160 at 64)
 
 // Which kernel serves n products of MT row tiles x NT column tiles over KB contraction blocks, its grid and
@@ -1206,6 +1206,8 @@ static ProductPlan plan_products(int64_t MT, int64_t NT, int64_t KB, int n) {
         // units split the contraction (their integer slices are added by the tail kernel)
         p.kind = PLAN_VEC; p.gx = (int)NT; p.gy = 1;
         while (NT * n * p.split < kVecFillWgs && KB / (p.split * 2) >= 8 && p.split < kMaxSplit) p.split *= 2;
+        // a very long contraction: one split (the 14B shape's ffn value product, 8 sequences: 6.97 against 7.26 ms per step)
+        if (p.split == 1 && NT * n < 512 && KB >= kGemmLongBlocks) p.split = 2;
         return p;
     }
     p.gy = (int)ceil_div(MT, 16);
