@@ -290,9 +290,18 @@ class HipRWKV:
             raise ValueError(f"state must be a contiguous CUDA float64 tensor of shape "
                              f"({self.layers}, 5, {self.dims})")
 
+    def _tokens(self, tokens) -> torch.Tensor:
+        """Token ids as an int64 vector on the device.  Ids that arrive on the host are range-checked there, as the
+        reference's host-side table lookup does (emb.py:9 raises IndexError); ids already on the device are not read
+        back: the kernels clamp them to the table."""
+        tok = torch.as_tensor(tokens, dtype=torch.int64).reshape(-1)
+        if tok.device.type == "cpu" and tok.numel() and (int(tok.min()) < 0 or int(tok.max()) >= self.vocab):
+            raise IndexError(f"token id out of range for a vocabulary of {self.vocab}")
+        return tok.to(self.device)
+
     def forward(self, tokens, state: torch.Tensor):
         """``(logits[V] float64, state)``; ``state`` is updated in place and returned (opt.py:61-76)."""
-        tok = torch.as_tensor(tokens, dtype=torch.int64).reshape(-1).to(self.device)
+        tok = self._tokens(tokens)
         if tok.numel() == 0:
             raise ValueError("forward needs at least one token")
         self._check_state(state)
@@ -310,7 +319,7 @@ class HipRWKV:
     def forward_batch(self, tokens, states: torch.Tensor):
         """One token for each of B independent sequences: ``tokens[B]``, ``states[B, L, 5, C]`` float64
         (updated in place) -> ``(logits[B, V] float64, states)``."""
-        tok = torch.as_tensor(tokens, dtype=torch.int64).reshape(-1).to(self.device)
+        tok = self._tokens(tokens)
         B = tok.numel()
         if (not isinstance(states, torch.Tensor) or states.device.type != "cuda" or states.dtype != torch.float64
                 or tuple(states.shape) != (B, self.layers, 5, self.dims) or not states.is_contiguous()):
@@ -333,6 +342,8 @@ class HipRWKV:
         """Feed ``token`` then greedily generate: returns ``(tokens[n] int64 on device, last logits, state)``
         where ``tokens[i] = argmax(forward(previous token))``.  No host round trip per token."""
         self._check_state(state)
+        if not 0 <= int(token) < self.vocab:
+            raise IndexError(f"token id out of range for a vocabulary of {self.vocab}")
         toks = torch.empty(n + 1, dtype=torch.int64, device=self.device)
         toks[0] = int(token)
         ws = self._workspace(1)
@@ -355,6 +366,8 @@ class HipRWKV:
         self._check_state(state)
         if not self.fused_step:
             raise RuntimeError("decode_sample needs the persistent single-token kernel (fused_step)")
+        if not 0 <= int(token) < self.vocab:
+            raise IndexError(f"token id out of range for a vocabulary of {self.vocab}")
         toks = torch.empty(n + 1, dtype=torch.int64, device=self.device)
         toks[0] = int(token)
         stops = torch.as_tensor(list(stop_tokens), dtype=torch.int64, device=self.device)

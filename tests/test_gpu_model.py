@@ -104,6 +104,18 @@ def test_forward_rejects_bad_state(tiny):
         hip.forward([1], hip.emptyState.clone()[:2])
     with pytest.raises(ValueError):
         hip.forward([], hip.emptyState.clone())
+    # ids given on the host are checked there, as the reference's host-side table lookup is (emb.py:9)
+    for bad in ([512], [3, -1], torch.tensor([0, 600])):
+        with pytest.raises(IndexError):
+            hip.forward(bad, hip.emptyState.clone())
+    with pytest.raises(IndexError):
+        hip.decode_greedy(512, 2, hip.emptyState.clone())
+    with pytest.raises(IndexError):
+        hip.forward_batch([1, 999], torch.stack([hip.emptyState.clone()] * 2))
+    # ids already on the device are not read back; the kernels clamp them to the table
+    lg, _ = hip.forward(torch.tensor([600], device="cuda"), hip.emptyState.clone())
+    lc, _ = hip.forward([511], hip.emptyState.clone())
+    assert torch.equal(lg, lc)
 
 
 def test_169m_shape_greedy_128_tokens():
