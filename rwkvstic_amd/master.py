@@ -194,17 +194,54 @@ class RWKVMaster:
         self.lastToken = [187]
 
 
+def _loader_options(device: str, kwargs: Dict) -> Dict:
+    """The options ``OptRWKV`` reads (opt.py:15-19, matmul.py:177-199) turned into this backend's: ``jit`` means
+    nothing here (there is no script compiler in the path); ``config["devices"]`` must name one GPU holding uint8
+    weights - the reference's split over several devices, its CPU / MPS fallbacks and its unquantised dtypes are not
+    part of this backend - and its ``stream`` entry keeps the codes in pinned host memory (matmul.py:21,186);
+    ``config["custom"]`` (which WKV operator, wkv.py:56-60) has one answer here.  ``export`` is returned for the
+    caller to act on.  Anything else raises: ``strategy`` would select another loader in the reference (load.py:48)."""
+    opts = dict(kwargs)
+    opts.pop("jit", None)
+    out = {"device": device, "stream": False, "export": opts.pop("export", False)}
+    config = opts.pop("config", None)
+    if opts:
+        raise TypeError(f"unsupported options for mode {MODE!r}: {sorted(opts)}")
+    if config is not None:
+        devices = config.get("devices") if isinstance(config, dict) else None
+        if not isinstance(devices, (list, tuple)) or len(devices) != 1 or not isinstance(devices[0], dict):
+            raise ValueError("config['devices'] must hold exactly one device entry: this backend runs on one GPU")
+        entry = devices[0]
+        name = str(entry.get("device", "cuda"))
+        if not name.startswith("cuda"):
+            raise ValueError(f"device {name!r}: this backend has no CPU / MPS path")
+        if entry.get("dtype", torch.uint8) != torch.uint8 or entry.get("naive", False):
+            raise ValueError("this backend holds uint8 (fp32i8) weights and runs its own kernels only")
+        if device in ("cuda", name):
+            out["device"] = name
+        else:
+            raise ValueError(f"device={device!r} and config['devices'][0]['device']={name!r} disagree")
+        out["stream"] = bool(entry.get("stream", False))
+    if out["export"] is not False and not isinstance(out["export"], str):
+        raise TypeError("export must be a file name stem (opt.py:112-113)")
+    return out
+
+
 def RWKV(path: Union[str, Dict[str, torch.Tensor]], mode: str = MODE, *, tokenizer=None, device: str = "cuda",
          sampler: Optional[Callable] = typical, **kwargs) -> RWKVMaster:
     """``path``: a BlinkDL ``.pth`` checkpoint, a file written by ``HipRWKV.save_quantized`` (the quantised
     attribute tree of the reference's .rwkv export as plain tensors; by convention ``.rwkvq``), both loaded with
     ``weights_only=True``; a TorchScript ``.rwkv`` archive (opt.py:89-92), of which only the tensors are read, by
     attribute path, without compiling or running the code stored in it (``rwkvstic_amd.archive``); or an already
-    loaded dict of either kind.  Only the FASTQUANT mode exists in this backend (load.py:42-47); other modes raise."""
+    loaded dict of either kind.  Only the FASTQUANT mode exists in this backend (load.py:42-47); other modes raise.
+    Of ``OptRWKV``'s options (opt.py:15-19) ``jit`` is accepted and means nothing, ``config`` may name the one GPU and
+    ask for host-resident weights (``{"devices": [{"device": "cuda:0", "dtype": torch.uint8, "stream": True}]}``),
+    and ``export="stem"`` writes the quantised model to ``stem.rwkvq`` and then ends the program, as the reference
+    does after writing ``stem.rwkv`` (opt.py:112-116)."""
     if mode != MODE:
         raise ValueError(f"mode {mode!r} is not provided by this backend (only {MODE!r})")
-    if kwargs:
-        raise TypeError(f"unsupported options for mode {MODE!r}: {sorted(kwargs)}")
+    opts = _loader_options(device, kwargs)
+    device = opts["device"]
     from .model import HipRWKV
     if isinstance(path, str):
         if path.endswith(".rwkv"):
@@ -218,5 +255,11 @@ def RWKV(path: Union[str, Dict[str, torch.Tensor]], mode: str = MODE, *, tokeniz
             raise ValueError("only .pth checkpoints, .rwkvq quantised trees and .rwkv archives are supported")
     else:
         weights = path
-    model = HipRWKV.from_quantized(weights, device=device) if "emb.w" in weights else HipRWKV(weights, device=device)
+    if "emb.w" in weights:
+        model = HipRWKV.from_quantized(weights, device=device, stream=opts["stream"])
+    else:
+        model = HipRWKV(weights, device=device, stream=opts["stream"])
+    if opts["export"] is not False:
+        model.save_quantized(opts["export"] + ".rwkvq")
+        raise SystemExit(0)                      # opt.py:115
     return RWKVMaster(model, model.emptyState.clone(), sampler, tokenizer)

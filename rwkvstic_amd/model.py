@@ -170,9 +170,10 @@ class HipRWKV:
         return out
 
     @classmethod
-    def from_quantized(cls, tree: Dict[str, torch.Tensor], device: str = "cuda") -> "HipRWKV":
+    def from_quantized(cls, tree: Dict[str, torch.Tensor], device: str = "cuda", stream: bool = False) -> "HipRWKV":
         """From ``quantized_tree()`` (or the same attributes taken from a reference model): nothing is
-        quantised again, the codes are only repacked into the streaming layouts."""
+        quantised again, the codes are only repacked into the streaming layouts (``stream``: kept in pinned host
+        memory, as in the constructor)."""
         if not torch.cuda.is_available():
             raise RuntimeError("HipRWKV needs a ROCm GPU (gfx950); there is no CPU path in this backend")
         N.lib()
@@ -188,7 +189,7 @@ class HipRWKV:
             if codes.dtype != torch.uint8 or codes.dim() != 2:
                 raise ValueError(f"{prefix}weight{suffix}: expected uint8 codes [in, out]")
             return QuantMatrix.from_codes(codes.contiguous(), tree[f"{prefix}range{suffix}"].reshape(-1),
-                                          tree[f"{prefix}offset{suffix}"].reshape(-1), self.device)
+                                          tree[f"{prefix}offset{suffix}"].reshape(-1), self.device, stream=stream)
 
         self.emb = tree["emb.w"].to(device=self.device, dtype=torch.float32).contiguous()
         layers = len([k for k in tree if k.startswith("blocks.") and k.endswith(".ln1.bias")])

@@ -486,6 +486,28 @@ def test_rwkv_shell_loads_checkpoint_file_and_generates(tmp_path, tiny):
     assert torch.equal(out["state"], s2)
 
 
+def test_rwkv_shell_takes_the_reference_loader_options(tmp_path, tiny):
+    """opt.py:15-19,112-116: ``export`` writes the quantised model and ends the program; ``config`` names the GPU and
+    may ask for host-resident codes; what is loaded back from the export gives the same logits bit for bit."""
+    import os
+    from rwkvstic_amd.master import RWKV, greedy
+    _, hip = tiny
+    sd = synth.make_state_dict(layers=3, C=64, V=512, seed=5, ln="random")
+    path, stem = str(tmp_path / "tiny.pth"), str(tmp_path / "exported")
+    torch.save(sd, path)
+    with pytest.raises(SystemExit):
+        RWKV(path, jit=False, export=stem)
+    assert os.path.exists(stem + ".rwkvq")
+    toks = synth.random_tokens(7, V=512, seed=2).tolist()
+    want, _ = hip.forward(toks, hip.emptyState.clone())
+    cfg = {"devices": [{"device": "cuda:0", "dtype": torch.uint8, "stream": True}]}
+    for r in (RWKV(stem + ".rwkvq", sampler=greedy), RWKV(stem + ".rwkvq", sampler=greedy, config=cfg),
+              RWKV(path, sampler=greedy, config=cfg)):
+        got, _ = r.model.forward(toks, r.emptyState.clone())
+        assert torch.equal(got, want)
+    assert not RWKV(path, config=cfg).model.blocks[0]["att_k"].packed.is_cuda        # the codes stayed on the host
+
+
 def test_quantized_tree_round_trip_and_oracle_layout(tmp_path, tiny):
     """The quantised model under the reference's attribute names (what its .rwkv export holds, opt.py:89-92;
     names from matmul.py:12,67-68, block.py:13-47, opt.py:31-48): the codes and ranges equal the CPU oracle's

@@ -145,6 +145,32 @@ def test_rwkv_rejects_unknown_modes_and_files():
         RWKV({}, strategy="cuda fp16")
 
 
+def test_rwkv_reads_the_reference_loader_options():
+    """opt.py:15-19, matmul.py:177-199: ``jit`` means nothing here, ``config`` may name the one GPU and ask for
+    host-resident codes, everything this backend does not provide is refused before any weight is touched."""
+    from rwkvstic_amd.master import _loader_options
+    assert _loader_options("cuda", {}) == {"device": "cuda", "stream": False, "export": False}
+    assert _loader_options("cuda", {"jit": False, "export": "out"})["export"] == "out"
+    one = {"devices": [{"device": "cuda:0", "dtype": torch.uint8, "stream": True}], "custom": True}
+    assert _loader_options("cuda", {"config": one}) == {"device": "cuda:0", "stream": True, "export": False}
+    assert _loader_options("cuda:0", {"config": one})["device"] == "cuda:0"
+    for bad in ({"devices": []},
+                {"devices": [{"device": "cuda:0"}, {"device": "cuda:1"}]},          # the reference's split over devices
+                {"devices": [{"device": "cpu", "dtype": torch.uint8}]},
+                {"devices": [{"device": "cuda", "dtype": torch.float16}]},
+                {"devices": [{"device": "cuda", "naive": True}]}):
+        with pytest.raises(ValueError):
+            _loader_options("cuda", {"config": bad})
+    with pytest.raises(ValueError):
+        _loader_options("cuda:1", {"config": one})
+    with pytest.raises(TypeError):
+        _loader_options("cuda", {"export": True})
+    with pytest.raises(TypeError):
+        _loader_options("cuda", {"strategy": "cuda fp16"})
+    with pytest.raises(ValueError):                     # refused before the (missing) file is opened
+        RWKV("no_such_model.pth", config={"devices": [{"device": "cpu"}]})
+
+
 def test_post_contract_and_state_json_round_trip():
     """server.py:56-86: state in and out as nested float lists, "input" loaded as context, the rest passed to forward."""
     import json
