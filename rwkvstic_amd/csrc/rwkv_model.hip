@@ -583,12 +583,20 @@ bool rows_supported(const rwkv_model *m) {
 
 // R rows through every layer.  sequence: rows are consecutive tokens of one sequence whose state is
 // `state` [L,5,C]; otherwise row b is one token of sequence b with state at state + b * state_stride.
+// pending (batch rows only, or null): the last layer's ffn value product may come back unfinished, for the
+// LayerNorm kernel in front of the head to finish.
 int rows_layers(rwkv_model *m, hipStream_t st, const int64_t *tokens, int64_t R, bool sequence, double *state,
-                int64_t state_stride, const RowsWs &w) {
+                int64_t state_stride, const RowsWs &w, RowsDeferred *pending = nullptr) {
     const rwkv_model_desc &d = m->d;
     const int C = (int)d.n_embd, F = (int)d.n_ffn, V = (int)d.n_vocab;
     const size_t RC = (size_t)R * C;
     RWKV_TRY(rows_embed(st, tokens, R, V, C, d.emb, d.ln0_w, d.ln0_b, w.x));
+    // Few batch rows: the products split their contraction, and the three whose result goes straight into one
+    // row-wise kernel (k, v, r -> WKV; the two residual updates -> the next LayerNorm) leave the sum of their slices
+    // to that kernel instead of a launch of their own.
+    const bool defer = !sequence && R < kRowsDeferMax;
+    RowsDeferred dk[3], dx;
+    dx.tot = nullptr;
     for (int64_t l = 0; l < d.n_layer; ++l) {
         const rwkv_layer_desc &L = m->layers[l];
         double *sl = state + (size_t)l * 5 * C;
@@ -600,30 +608,34 @@ int rows_layers(rwkv_model *m, hipStream_t st, const int64_t *tokens, int64_t R,
         const float *rg[3] = {kvr[0]->range, kvr[1]->range, kvr[2]->range};
         const double *of[3] = {kvr[0]->offset, kvr[1]->offset, kvr[2]->offset};
         RWKV_TRY(rows_ln_mix_quant(st, 3, R, C, sequence, w.x, L.ln1_w, L.ln1_b, L.att_mix, copy_prev ? w.prev0 : sl, sl,
-                                   state_stride, rg, of, w.q));
+                                   state_stride, rg, of, w.q, &dx));
         // k, v, r (and the ffn receptance below) are kept as float32 arrays in the kvr slab
         float *kvr32 = reinterpret_cast<float *>(w.kvr);
         RowsProduct pk[3];
         for (int i = 0; i < 3; ++i) { pk[i].a = w.q[i]; pk[i].w16 = kvr[i]->packed16; pk[i].out = reinterpret_cast<double *>(kvr32 + i * RC); }
-        RWKV_TRY(rows_products(st, 3, pk, w.tot, R, C, C, ROW_STORE_F32, nullptr));
+        RWKV_TRY(rows_products(st, 3, pk, w.tot, R, C, C, ROW_STORE_F32, nullptr, defer ? dk : nullptr));
         RWKV_TRY(rows_wkv(st, R, C, sequence, kvr32, kvr32 + RC, kvr32 + 2 * RC, L.time_decay, L.time_first,
-                          sl + 2 * (size_t)C, state_stride, reinterpret_cast<float *>(w.att), w.wkv_scr));
+                          sl + 2 * (size_t)C, state_stride, reinterpret_cast<float *>(w.att), w.wkv_scr, defer ? dk : nullptr));
         RWKV_TRY(rows_quant(st, R, C, w.att, true, L.att_o.range, L.att_o.offset, w.q[0], (double *)w.tot));    // att and h: float32 arrays
         const RowsProduct po = {w.q[0], L.att_o.packed16, w.x};
-        RWKV_TRY(rows_products(st, 1, &po, w.tot, R, C, C, ROW_ADD, nullptr));
+        RWKV_TRY(rows_products(st, 1, &po, w.tot, R, C, C, ROW_ADD, nullptr, defer ? &dx : nullptr));
         // ChannelMix (block.py:82-100)
         if (copy_prev) RWKV_CHECK_HIP(hipMemcpyAsync(w.prev0, sl + C, (size_t)C * 8, hipMemcpyDeviceToDevice, st));
         const float *rg2[2] = {L.ffn_k.range, L.ffn_r.range};
         const double *of2[2] = {L.ffn_k.offset, L.ffn_r.offset};
         RWKV_TRY(rows_ln_mix_quant(st, 2, R, C, sequence, w.x, L.ln2_w, L.ln2_b, L.ffn_mix, copy_prev ? w.prev0 : sl + C,
-                                   sl + C, state_stride, rg2, of2, w.q + 1));
+                                   sl + C, state_stride, rg2, of2, w.q + 1, &dx));
+        dx.tot = nullptr;
         const RowsProduct pfk = {w.q[1], L.ffn_k.packed16, w.h}, pfr = {w.q[2], L.ffn_r.packed16, w.kvr};
         RWKV_TRY(rows_products(st, 1, &pfk, w.tot, R, C, F, ROW_RELU2, nullptr));
         RWKV_TRY(rows_products(st, 1, &pfr, w.tot, R, C, C, ROW_STORE_F32, nullptr));
         RWKV_TRY(rows_quant(st, R, F, w.h, true, L.ffn_v.range, L.ffn_v.offset, w.q[0], (double *)w.tot));
         const RowsProduct pfv = {w.q[0], L.ffn_v.packed16, w.x};
-        RWKV_TRY(rows_products(st, 1, &pfv, w.tot, R, F, C, ROW_GATE_ADD, kvr32));
+        // (the ffn receptance stays in the kvr slab and the totals untouched until the next LayerNorm kernel has run)
+        const bool hand_on = defer && (l + 1 < d.n_layer || pending);
+        RWKV_TRY(rows_products(st, 1, &pfv, w.tot, R, F, C, ROW_GATE_ADD, kvr32, hand_on ? &dx : nullptr));
     }
+    if (pending) *pending = dx;
     return RWKV_OK;
 }
 
@@ -854,12 +866,13 @@ int rwkv_model_forward_batch(rwkv_model *m, rwkv_stream_t stream, const int64_t 
     const rwkv_model_desc &d = m->d;
     const int64_t C = d.n_embd, F = d.n_ffn, V = d.n_vocab;
     const RowsWs rw = rows_carve(workspace, batch, C, F, F > V ? F : V, 0);
-    int rc = rows_layers(m, st, tokens, batch, false, states, d.n_layer * 5 * C, rw);
+    RowsDeferred pending;
+    int rc = rows_layers(m, st, tokens, batch, false, states, d.n_layer * 5 * C, rw, &pending);
     if (rc) return rc;
     const float *rg[1] = {d.head.range};
     const double *of[1] = {d.head.offset};
     rc = rows_ln_mix_quant(st, 0, batch, (int)C, false, rw.x, d.ln_out_w, d.ln_out_b, nullptr, nullptr, nullptr, 0, rg, of,
-                           rw.q);
+                           rw.q, &pending);
     if (rc) return rc;
     const RowsProduct ph = {rw.q[0], d.head.packed16, logits};
     return rows_products(st, 1, &ph, rw.tot, batch, C, V, ROW_STORE, nullptr);

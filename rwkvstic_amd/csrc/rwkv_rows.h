@@ -22,6 +22,19 @@ struct RowsProduct {        // out[R, N] (tail op) a x quantised matrix in M16 b
     double *out;
 };
 constexpr int kRowsMaxProducts = 3;     // products of equal shape and tail that share one launch
+// A product whose contraction was split, handed on unfinished: its consumer (the LayerNorm kernel for the two
+// residual updates, the WKV kernel for k, v, r) adds the slices of integer totals up itself and applies the tail,
+// which saves the launch that would otherwise do only that.  tot == nullptr: nothing is pending (the product was not
+// split and its epilogue applied the tail).  Only for batches of fewer than kRowsDeferMax independent rows.
+struct RowsDeferred {
+    const long long *tot;   // [slices][slice] totals of this product; element (t, j) at t * ldd + j
+    size_t slice;
+    int slices, ldd, op;    // op: the RowTail still to be applied
+    const double *S, *qs, *zp;
+    const float *gate;      // ROW_GATE_ADD
+};
+constexpr int64_t kRowsDeferMax = 128;
+constexpr int kRowsDeferSlices = 4;     // a contraction split further than this is finished by a launch of its own
 size_t rows_dig_bytes(int64_t R, int64_t K);
 size_t rows_tot_bytes(int64_t R, int64_t N);        // integer totals of ONE product (times the products in a launch)
 size_t rows_wkv_scratch_bytes(int64_t R, int64_t C);
@@ -38,18 +51,24 @@ int rows_embed(hipStream_t st, const int64_t *tokens, int64_t R, int V, int C, c
 int rows_ln_mix_quant(hipStream_t st, int n_mix, int64_t R, int C, bool sequence, const double *x, const double *ln_w,
                       const double *ln_b, const double *mu, const double *prev0, double *shift_dst,
                       int64_t prev_stride, const float *const *range, const double *const *offset,
-                      const RowsOperand *out);
+                      const RowsOperand *out, const RowsDeferred *add = nullptr /* pending residual update of x: applied
+                      and stored first (x is then written too); batch rows only */);
 // Rows of float64 values quantised for a matrix with the given per-input-channel range / offset.
 // scratch: rows_quant_scratch_bytes(R, K) bytes (any buffer free until the product starts, e.g. its totals), or null.
 int rows_quant(hipStream_t st, int64_t R, int64_t K, const void *in, bool in_f32, const float *range, const double *offset,
                const RowsOperand &out, double *scratch);
 // n (<= kRowsMaxProducts) products of the same shape [R, K] x [K, N] and tail in one launch;
 // tot: n * rows_tot_bytes(R, N) bytes of scratch.
+// defer (null, or n entries): where the contraction is split (in at most kRowsDeferSlices) and R < kRowsDeferMax the tail is left to the consumer
+// and described here (tot and the operand's row constants must stay untouched until that kernel has run); entries of
+// products that were finished here get tot = nullptr.
 int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, int64_t R, int64_t K, int64_t N, int op,
-                  const float *gate);
+                  const float *gate, RowsDeferred *defer = nullptr);
+// kvr (null, or 3 entries, batch rows only): k, v, r still pending as split products (ROW_STORE_F32) where tot is set.
 int rows_wkv(hipStream_t st, int64_t R, int C, bool sequence, const float *k, const float *v, const float *r,
              const double *w, const double *u, double *state, int64_t state_stride, float *out,
-             double *scratch /* rows_wkv_scratch_bytes(R, C), or null: serial over the rows */);
+             double *scratch /* rows_wkv_scratch_bytes(R, C), or null: serial over the rows */,
+             const RowsDeferred *kvr = nullptr);
 
 // Stand-alone product of 1..8 float32 vectors with one matrix in M16 blocks, four-vector dequantisation (row and
 // column ranges / offsets; r_col, m_col may be null); ws: rows_mv16_workspace_bytes(B, n_in) bytes, 256-byte aligned.

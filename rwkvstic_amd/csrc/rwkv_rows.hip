@@ -150,9 +150,45 @@ __device__ __forceinline__ void row_scale(float amax, double &S, double &invS) {
 // One workgroup per row; a thread keeps its NSEG groups of four channels in registers from the one
 // read of x to the digits, so the mixed rows never travel through memory.
 // ---------------------------------------------------------------------------
+// Element (t, j) of a product handed on unfinished: the slices added up (integers: exact in any order), then
+// y = S_t * tot + 128 * S_t * sum q_t + zp_t as in rows_finish_kernel.
+__device__ __forceinline__ double deferred_y(const RowsDeferred &d, int t, long long tot) {
+    const double S = d.S[t];
+    return S * (double)tot + 128.0 * (S * d.qs[t]) + d.zp[t];
+}
+// The slices are requested together, without a branch (always kRowsDeferSlices of them: one past the last reads
+// slice 0 again and is not counted): a loop over a run-time count would wait for every slice before asking for the
+// next, and a branch would keep the loads of a thread's channel groups apart.
+__device__ __forceinline__ long long slices_sum1(const long long *tp, size_t slice, int slices) {
+    long long u[kRowsDeferSlices], tot = 0;
+#pragma unroll
+    for (int z = 0; z < kRowsDeferSlices; ++z) u[z] = tp[(size_t)(z < slices ? z : 0) * slice];
+#pragma unroll
+    for (int z = 0; z < kRowsDeferSlices; ++z) tot += z < slices ? u[z] : 0;
+    return tot;
+}
+__device__ __forceinline__ void slices_sum4(const long long *tp, size_t slice, int slices, long long (&tot)[4]) {
+    longlong2 u[kRowsDeferSlices][2];
+#pragma unroll
+    for (int z = 0; z < kRowsDeferSlices; ++z) {
+        const long long *q = tp + (size_t)(z < slices ? z : 0) * slice;
+        u[z][0] = *reinterpret_cast<const longlong2 *>(q); u[z][1] = *reinterpret_cast<const longlong2 *>(q + 2);
+    }
+#pragma unroll
+    for (int z = 0; z < kRowsDeferSlices; ++z) {
+        const bool on = z < slices;
+        tot[0] += on ? u[z][0].x : 0; tot[1] += on ? u[z][0].y : 0; tot[2] += on ? u[z][1].x : 0; tot[3] += on ? u[z][1].y : 0;
+    }
+}
+__device__ __forceinline__ double deferred_value(const RowsDeferred &d, int t, int j) {
+    return deferred_y(d, t, slices_sum1(d.tot + (size_t)t * d.ldd + j, d.slice, d.slices));
+}
+
 struct LnQuantArgs {
     int C, R, sequence;
     const double *x;            // [R, C]
+    RowsDeferred add;           // batch rows, 512 threads per row: x += this product first, stored to x_rw (tot null: none)
+    double *x_rw;
     const double *ln_w, *ln_b;  // [C]
     const double *mu;           // [NM, C]
     const double *prev0;        // sequence: [C]; batch: row t at prev0 + t * prev_stride
@@ -864,6 +900,7 @@ struct WkvRowsArgs {
     double *state;              // rows aa, bb, pp of the layer: state + 2C; batch: + row * state_stride
     int64_t state_stride;
     float *out;                 // [R, C]  wkv * sigmoid(r): a float32 product
+    RowsDeferred pend[3];       // batch rows: k, v, r still in slices (tot null: read from the arrays above)
 };
 
 __global__ void __launch_bounds__(64) wkv_rows_kernel(const WkvRowsArgs a) {
@@ -877,8 +914,12 @@ __global__ void __launch_bounds__(64) wkv_rows_kernel(const WkvRowsArgs a) {
     double pp = st[2 * C + c];
     for (int t = t0; t < t1; ++t) {
         const size_t i = (size_t)t * C + c;
-        const float y = wkv_step_f32(w, u, a.k[i], a.v[i], aa, bb, pp);
-        a.out[i] = y * sigmoid_f32(a.r[i]);
+        // (uniform branches; a pending product is rounded to float32 exactly as ROW_STORE_F32 would have stored it)
+        const float kk = a.pend[0].tot ? (float)deferred_value(a.pend[0], t, c) : a.k[i];
+        const float vv = a.pend[1].tot ? (float)deferred_value(a.pend[1], t, c) : a.v[i];
+        const float rr = a.pend[2].tot ? (float)deferred_value(a.pend[2], t, c) : a.r[i];
+        const float y = wkv_step_f32(w, u, kk, vv, aa, bb, pp);
+        a.out[i] = y * sigmoid_f32(rr);
     }
     st[c] = (double)aa; st[C + c] = (double)bb; st[2 * C + c] = pp;
 }
@@ -1268,11 +1309,19 @@ bool rows_ln_width_supported(int64_t C) { return C % 4 == 0 && C <= 3 * 4 * kLnM
 int rows_ln_mix_quant(hipStream_t st, int n_mix, int64_t R, int C, bool sequence, const double *x, const double *ln_w,
                       const double *ln_b, const double *mu, const double *prev0, double *shift_dst,
                       int64_t prev_stride, const float *const *range, const double *const *offset,
-                      const RowsOperand *out) {
+                      const RowsOperand *out, const RowsDeferred *add) {
     if (C % 64 != 0 || !rows_ln_width_supported(C))
         return set_error(RWKV_ERR_SIZE, "rows_ln_mix_quant: width %d is not a multiple of 64 up to %d", C, 3 * 4 * kLnMaxThreads);
     LnQuantArgs a;
     a.C = C; a.R = (int)R; a.sequence = sequence ? 1 : 0; a.x = x; a.ln_w = ln_w; a.ln_b = ln_b; a.mu = mu;
+    a.add.tot = nullptr; a.x_rw = nullptr;
+    if (add && add->tot) {
+        // every row is read and rewritten by its own workgroup only: rows of a sequence read their neighbour's x too
+        if (sequence || R >= kRowsDeferMax || (add->op != ROW_ADD && add->op != ROW_GATE_ADD))
+            return set_error(RWKV_ERR_ARG, "rows_ln_mix_quant: a pending product needs fewer than %d batch rows and a residual tail",
+                             (int)kRowsDeferMax);
+        a.add = *add; a.x_rw = const_cast<double *>(x);
+    }
     a.prev0 = prev0; a.shift_dst = shift_dst; a.prev_stride = prev_stride;
     const int n_out = n_mix > 0 ? n_mix : 1;
     for (int m = 0; m < 3; ++m) {
@@ -1282,7 +1331,7 @@ int rows_ln_mix_quant(hipStream_t st, int n_mix, int64_t R, int C, bool sequence
     }
     // few rows: 512 threads per row shorten the chain of dependent steps; many rows: 256 threads with twice
     // the channels each keep more rows resident per compute unit
-    const bool many = R >= 128;
+    const bool many = R >= kRowsDeferMax;           // (a pending product is only ever handed to the 512-thread form)
     const dim3 grid((unsigned)R), block(many ? 256 : 512);
     const bool small = many ? C <= 3 * 4 * 256 : C <= 2 * 4 * 512;
 #define RWKV_LNQ(NM)                                                                                  \
@@ -1342,7 +1391,7 @@ int rows_quant(hipStream_t st, int64_t R, int64_t K, const void *in, bool in_f32
 }
 
 int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, int64_t R, int64_t K, int64_t N, int op,
-                  const float *gate) {
+                  const float *gate, RowsDeferred *defer) {
     if (K % 64 != 0) return set_error(RWKV_ERR_SIZE, "rows_products: contraction length %lld is not a multiple of 64",
                                       (long long)K);
     if (n < 1 || n > kRowsMaxProducts) return set_error(RWKV_ERR_ARG, "rows_products: %d products in one launch", n);
@@ -1380,7 +1429,13 @@ int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, i
         else hipLaunchKernelGGL(gemm8_kernel, grid, dim3(512), 0, st, g);
         RWKV_CHECK_LAUNCH("gemm8_kernel");
     }
+    for (int m = 0; defer && m < n; ++m) defer[m].tot = nullptr;
     if (split == 1) return RWKV_OK;     // the tail was applied in the product's epilogue
+    if (defer && R < kRowsDeferMax && split <= kRowsDeferSlices) {   // the consumer adds the slices up
+        for (int m = 0; m < n; ++m)
+            defer[m] = RowsDeferred{tot + (size_t)m * split * g.slice, g.slice, split, g.ldd, op, p[m].a.S, p[m].a.qs, p[m].a.zp, gate};
+        return RWKV_OK;
+    }
 
     f.R = (int)R; f.N = (int)N; f.ldd = g.ldd; f.slices = split; f.slice = g.slice; f.tot = tot; f.gate = gate;
     const dim3 fg((unsigned)ceil_div(N, 256), (unsigned)R, (unsigned)n), fb(256);
@@ -1396,10 +1451,17 @@ int rows_products(hipStream_t st, int n, const RowsProduct *p, long long *tot, i
 }
 
 int rows_wkv(hipStream_t st, int64_t R, int C, bool sequence, const float *k, const float *v, const float *r,
-             const double *w, const double *u, double *state, int64_t state_stride, float *out, double *scratch) {
+             const double *w, const double *u, double *state, int64_t state_stride, float *out, double *scratch,
+             const RowsDeferred *kvr) {
     WkvRowsArgs a;
     a.C = C; a.R = (int)R; a.sequence = sequence ? 1 : 0; a.k = k; a.v = v; a.r = r; a.w = w; a.u = u;
     a.state = state; a.state_stride = state_stride; a.out = out;
+    for (int i = 0; i < 3; ++i) {
+        if (kvr) a.pend[i] = kvr[i];
+        else a.pend[i].tot = nullptr;
+        if (a.pend[i].tot && (sequence || a.pend[i].op != ROW_STORE_F32))
+            return set_error(RWKV_ERR_ARG, "rows_wkv: a pending product needs batch rows and the float32 store tail");
+    }
     if (sequence && scratch && R >= 2 * kWkvChunk) {
         const int n_chunks = (int)ceil_div(R, kWkvChunk);
         const dim3 grid((unsigned)ceil_div(C, 64), (unsigned)n_chunks);
