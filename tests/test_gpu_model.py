@@ -403,7 +403,7 @@ def test_forward_batch_matches_per_sequence_steps(tiny, B):
 
 SWEEP = [  # layers, C, F, V, prompt length, chunking, batch sizes (None: widths the batch path does not take)
     (2, 72, 200, 301, 63, (31, 1, 31), None),
-    (3, 128, 512, 1000, 130, (3, 31, 1, 95), (1, 2, 40)),
+    (3, 128, 512, 1000, 130, (3, 31, 1, 95), (1, 2, 40, 127, 128, 131)),     # 128: where the batch path changes its row kernels
     (2, 192, 768, 777, 64, (64,), (3, 33)),
     (2, 448, 1000, 333, 130, (3, 7, 7, 64, 49), None),
     (2, 512, 2048, 50277, 257, (31, 31, 2, 16, 100, 16, 1, 60), (17,)),
